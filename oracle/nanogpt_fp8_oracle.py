@@ -1,0 +1,386 @@
+"""CPU oracle for the FP8 contraction path -- TEST INFRASTRUCTURE ONLY.
+
+Plain PyTorch-eager restatement of the reference's arithmetic for `nanogpt::mm`
+(+ backward, + the transposed-weight `_t` pair), the FP8 MLP forward/backward
+and the fused softcapped cross-entropy.  Only tests, the smoke check and the
+benchmark's cpu_baseline leg may import this module, and only as the checker;
+the shipped package never does.
+
+Normative semantics are PyTorch *eager* on CPU: a bf16 tensor divided by a
+Python float is `bf16_rne(fp32(x) / fp32(s))`, fp8 casts round to nearest even
+and do not saturate, GEMMs are exact products of the decoded fp8 operands
+summed in fp32 (here: fp32/fp64 matmul of the dequantised operands), results
+are scaled by the fp32 product of the two per-tensor scales and rounded once
+to the output dtype.
+
+Every function cites the reference lines it follows (paths relative to the
+reference checkout).  What pins each function without running the reference:
+
+  quant_e4m3 / quant_e5m2      exhaustive 65536-entry tables + oracle/fp8_codec.c
+                               (closed-form encode/decode)            -> pinned
+  mm_* / mm_t_*                brute-force triple loop on fp8 codes in double
+                               (fp8_codec.c), linearity, transposition identities -> pinned
+  fc_relu2_* / mlp_*           invariants (post >= 0, post == 0 <=> pre <= 0),
+                               autograd of relu(x W1^T)^2 W2 in fp32   -> pinned
+  ce_fwd_bwd                   closed form F.cross_entropy of the softcapped logits
+                               (reference train_gpt.py:1689-1692), the unfold/MTP
+                               form (train_gpt_medium.py:1206-1215), autograd and
+                               fp64 finite differences, sum_j p_ij = 1 -> pinned
+  parity unpinned (cannot be pinned without the reference's GPU stack):
+      cuBLASLt `use_fast_accum=True` accumulation order, the CUDA fast-math
+      intrinsics (tanh.approx, __expf, __logf) of the CE kernel, inductor's
+      single-rounding fused quantise.  All are below the stated tolerances.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor
+
+E4M3 = torch.float8_e4m3fn
+E5M2 = torch.float8_e5m2
+E4M3_MAX = 448.0
+E5M2_MAX = 57344.0
+
+
+# ----------------------------------------------------------------------------
+# a1: quantisers
+
+def quant_e4m3(x: Tensor, s: float) -> Tensor:
+    """`x.div(x_s).to(torch.float8_e4m3fn)` -- train_gpt_medium.py:45-46,
+    train_gpt.py:78-79, triton_kernels.py:1212-1213."""
+    return x.div(s).to(E4M3)
+
+
+def quant_e5m2(g: Tensor, s: float) -> Tensor:
+    """`grad.div(grad_s).to(torch.float8_e5m2)` -- train_gpt_medium.py:75, train_gpt.py:114."""
+    return g.div(s).to(E5M2)
+
+
+def e5m2_satfinite(v: Tensor) -> Tensor:
+    """fp32 -> e5m2, round-to-nearest-even, finite values clamp to +-57344
+    (`cvt.rn.satfinite.e5m2x2.f32`, triton_kernels.py:923-933)."""
+    return v.float().clamp(-E5M2_MAX, E5M2_MAX).to(E5M2)
+
+
+def _scale(a: float, b: float) -> Tensor:
+    """fp32 product of two per-tensor scales, as `_scaled_mm` forms alpha."""
+    return torch.tensor(a, dtype=torch.float32) * torch.tensor(b, dtype=torch.float32)
+
+
+def _mm_f8(a_f8: Tensor, b_f8: Tensor) -> Tensor:
+    """Exact-ish product of decoded fp8 operands: `a @ b` with fp32 inputs.
+    Products of two fp8 values are exact in fp32; only the summation rounds."""
+    return a_f8.float() @ b_f8.float()
+
+
+# ----------------------------------------------------------------------------
+# a2-a4: nanogpt::mm, weight stored (out, in)
+
+def mm_fwd(x: Tensor, w: Tensor, x_s: float, w_s: float):
+    """train_gpt_medium.py:40-57.  x [M,K] bf16, w [N,K] bf16 ->
+    (out [M,N] bf16, x_f8 [M,K], w_f8 [N,K])."""
+    assert x.is_contiguous() and w.is_contiguous()
+    x_f8 = quant_e4m3(x, x_s)
+    w_f8 = quant_e4m3(w, w_s)
+    out = (_mm_f8(x_f8, w_f8.T) * _scale(x_s, w_s)).to(torch.bfloat16)
+    return out, x_f8, w_f8
+
+
+def mm_bwd(g: Tensor, x_f8: Tensor, w_f8: Tensor, x_s: float, w_s: float, grad_s: float):
+    """train_gpt_medium.py:67-95.  g [M,N] bf16 -> (dx [M,K] bf16, dW [N,K] fp32 as a
+    transposed view of a contiguous [K,N] buffer, strides (1, N))."""
+    assert g.is_contiguous()
+    g_f8 = quant_e5m2(g, grad_s)
+    dx = (_mm_f8(g_f8, w_f8) * _scale(grad_s, w_s)).to(torch.bfloat16)
+    dw_kn = (_mm_f8(x_f8.T, g_f8) * _scale(x_s, grad_s)).contiguous()      # [K, N]
+    return dx, dw_kn.T
+
+
+# a5: nanogpt::mm_t, weight stored (in, out)
+
+def mm_t_fwd(x: Tensor, w: Tensor, x_s: float, w_s: float):
+    """train_gpt.py:70-95.  x [M,K], w [K,N] -> (out [M,N] bf16, x_f8, w_f8 [K,N])."""
+    assert x.is_contiguous() and w.is_contiguous()
+    assert x.shape[1] == w.shape[0]
+    x_f8 = quant_e4m3(x, x_s)
+    w_f8 = quant_e4m3(w, w_s)
+    out = (_mm_f8(x_f8, w_f8) * _scale(x_s, w_s)).to(torch.bfloat16)
+    return out, x_f8, w_f8
+
+
+def mm_t_bwd(g: Tensor, x_f8: Tensor, w_f8: Tensor, x_s: float, w_s: float, grad_s: float):
+    """train_gpt.py:105-141.  -> (dx [M,K] bf16, dW [K,N] fp32 contiguous)."""
+    assert g.is_contiguous()
+    g_f8 = quant_e5m2(g, grad_s)
+    dx = (_mm_f8(g_f8, w_f8.T) * _scale(grad_s, w_s)).to(torch.bfloat16)
+    dw = (_mm_f8(x_f8.T, g_f8) * _scale(x_s, grad_s)).contiguous()
+    return dx, dw
+
+
+# ----------------------------------------------------------------------------
+# a6, a13: MLP quantisation glue
+
+def rms_norm(x: Tensor) -> Tensor:
+    """`F.rms_norm(x, (x.size(-1),))` -- train_gpt.py:952-953."""
+    return F.rms_norm(x, (x.size(-1),))
+
+
+def mlp_input_quant(normed: Tensor, up_scale: Tensor):
+    """train_gpt.py:1645-1647.  Dynamic per-tensor e4m3 quantisation of the normed
+    activations.  Returns (x_f8, dequant) with dequant a 1-element fp32 tensor
+    `up_scale * amax / 448` computed with the reference's in-place fp32 op order."""
+    amax = normed.detach().abs().max().clamp(min=1e-12)
+    x_f8 = (normed.detach() * (448.0 / amax)).to(E4M3)
+    dequant = torch.ones(1, dtype=torch.float32)
+    dequant.copy_(up_scale.reshape(1)).mul_(amax).div_(448.0)
+    return x_f8, dequant
+
+
+def quantize_up_weights(w_fc: Tensor):
+    """Per-layer amax scale + e4m3 copy of c_fc -- train_gpt.py:1419-1422.
+    w_fc [L,H,D] -> (w_f8 [L,H,D] e4m3, scales [L] fp32)."""
+    L = w_fc.shape[0]
+    scales = w_fc.reshape(L, -1).abs().amax(dim=1).clamp(min=1e-12) / E4M3_MAX
+    w_f8 = (w_fc / scales.view(L, 1, 1)).to(E4M3)
+    return w_f8, scales.float()
+
+
+# ----------------------------------------------------------------------------
+# a7, a8: fused linear + ReLU^2 and the MLP autograd function
+
+def fc_relu2_fwd(x_f8: Tensor, w_f8: Tensor, dequant: Tensor,
+                 activation_scale: Tensor | None = None):
+    """linear_relu_square_kernel, FORWARD + USE_FP8 (+ EMIT_FP8) -- triton_kernels.py:435-471.
+    acc fp32 -> * dequant -> bf16 -> max(.,0) -> square in bf16.
+    With `activation_scale`: also `post_f8 = e4m3(min(post * (1/act_scale), 448))`
+    (the product is a bf16 * fp32 -> fp32 expression in the kernel) and amax(post)."""
+    acc = _mm_f8(x_f8, w_f8.T) * dequant.float().reshape(())
+    c = acc.to(torch.bfloat16)
+    r = torch.clamp_min(c, 0)
+    post = r * r
+    if activation_scale is None:
+        return post
+    inv = 1.0 / activation_scale.float().reshape(())
+    post_f8 = torch.minimum(post.float() * inv, torch.tensor(E4M3_MAX)).to(E4M3)
+    return post, post_f8, post.float().max()
+
+
+def fc_relu2_bwd_dpre(dy: Tensor, w2: Tensor, post: Tensor) -> Tensor:
+    """linear_relu_square_kernel, FORWARD=False -- triton_kernels.py:472-476, 493-496, 726.
+    dy [M,D] bf16, w2 [H,D] bf16, post [M,H] bf16 -> dpre = bf16(2 * bf16(dy @ w2^T) * sqrt(post))."""
+    c = (dy.float() @ w2.float().T).to(torch.bfloat16)
+    return (2 * c.float() * torch.sqrt(post.float())).to(torch.bfloat16)
+
+
+def mlp_fwd(x: Tensor, w1: Tensor, w2: Tensor, w1_f8=None, dequant=None, x_f8=None,
+            w2_f8=None, w2_scale=None, activation_scale=None):
+    """FusedLinearReLUSquareFunction.forward -- triton_kernels.py:669-718.
+    w1 [H,D], w2 [H,D] (so `post @ w2` is the down projection).
+    Returns (out, post[, amax_post])."""
+    xf = x.reshape(-1, x.shape[-1])
+    if w1_f8 is not None:
+        xq = x_f8.reshape(-1, x_f8.shape[-1])
+        if w2_f8 is not None:
+            post, post_f8, amax = fc_relu2_fwd(xq, w1_f8, dequant, activation_scale)
+            x3 = (_mm_f8(post_f8, w2_f8) * (activation_scale.float().reshape(()) *
+                                            w2_scale.float().reshape(()))).to(torch.bfloat16)
+            return x3.view(x.shape), post, amax
+        post = fc_relu2_fwd(xq, w1_f8, dequant)
+    else:
+        c = (xf.float() @ w1.float().T).to(torch.bfloat16)
+        r = torch.clamp_min(c, 0)
+        post = r * r
+    x3 = (post.float() @ w2.float()).to(torch.bfloat16)
+    return x3.view(x.shape), post
+
+
+def mlp_bwd(dy: Tensor, x: Tensor, w1: Tensor, w2: Tensor, post: Tensor):
+    """FusedLinearReLUSquareFunction.backward -- triton_kernels.py:720-729 (all bf16 GEMMs,
+    fp32 accumulate).  Returns (dx, dW1 [H,D], dW2 [H,D])."""
+    xf = x.reshape(-1, x.shape[-1])
+    dyf = dy.reshape(-1, dy.shape[-1])
+    dw2 = (post.float().T @ dyf.float()).to(torch.bfloat16)
+    dpre = fc_relu2_bwd_dpre(dyf, w2, post)
+    dw1 = (dpre.float().T @ xf.float()).to(torch.bfloat16)
+    dx = (dpre.float() @ w1.float()).to(torch.bfloat16)
+    return dx.view(x.shape), dw1, dw2
+
+
+# ----------------------------------------------------------------------------
+# a10: cross-entropy forward+backward on materialised logits
+
+def softcap_sigma(logits: Tensor, B: float, C: float) -> Tensor:
+    """bf16(sigmoid(l/C + B/C)) as fp32 values -- triton_kernels.py:991-1005.
+    The kernel evaluates `l * inv_C + B_div_C` in fp32 with inv_C = 1/C rounded to fp32."""
+    inv_c = torch.tensor(1.0, dtype=torch.float32) / torch.tensor(C, dtype=torch.float32)
+    b_div_c = torch.tensor(B, dtype=torch.float32) * inv_c
+    u = logits.float() * inv_c + b_div_c
+    return torch.sigmoid(u).to(torch.bfloat16).float()
+
+
+def ce_fwd_bwd(logits: Tensor, targets: Tensor, mtp_weights: Tensor, prefix_targets: Tensor,
+               prefix_weight: Tensor, n_rows: int, n_predict: int,
+               A: float, B: float, C: float, grad_s: float, grad_scale: float):
+    """ce_fwd_bwd_kernel -- triton_kernels.py:956-1170.  logits [M,V] bf16.
+    Returns (losses [M] fp32, grad_input [M,V] e5m2, lse [M] fp32).
+
+    Follows the kernel's quirk that the normaliser weight S_w sums all n_predict
+    weights even on tail rows whose shifted target falls past the end
+    (triton_kernels.py:1094-1098)."""
+    M, V = logits.shape
+    assert M == n_rows
+    A32 = torch.tensor(A, dtype=torch.float32)
+    sig = softcap_sigma(logits, B, C)
+    z = A32 * sig
+    mx = z.max(dim=1, keepdim=True).values
+    lse = (mx + torch.log(torch.exp(z - mx).sum(dim=1, keepdim=True))).squeeze(1)
+
+    w = mtp_weights.float()
+    pw = prefix_weight.float().reshape(())
+    rows = torch.arange(M)
+    losses = torch.zeros(M, dtype=torch.float32)
+    term2 = torch.zeros(M, V, dtype=torch.float32)
+    for k in range(n_predict):
+        idx = rows + k
+        inb = idx < M
+        t = torch.where(inb, targets[idx.clamp(max=M - 1)], torch.full_like(targets, -1))
+        valid = inb & (t >= 0) & (t < V)
+        tc = t.clamp(0, V - 1)
+        zt = z[rows, tc]
+        losses += torch.where(valid, w[k] * (lse - zt), torch.zeros(()))
+        term2[rows[valid], tc[valid]] += w[k]
+    pvalid = (prefix_targets >= 0) & (prefix_targets < V)
+    ptc = prefix_targets.clamp(0, V - 1)
+    losses += torch.where(pvalid, pw * (lse - z[rows, ptc]), torch.zeros(()))
+    term2[rows[pvalid], ptc[pvalid]] += pw
+
+    s_w = w[:n_predict].sum() + torch.where(pvalid, pw, torch.zeros(()))       # [M]
+    p = torch.exp(z - lse.unsqueeze(1))
+    grad_z = s_w.unsqueeze(1) * p - term2
+    c32 = torch.tensor(C, dtype=torch.float32)
+    coef = (torch.tensor(grad_scale, dtype=torch.float32) * (1.0 / c32 * A32)
+            * (1.0 / torch.tensor(grad_s, dtype=torch.float32)))
+    g = coef * grad_z * sig * (1.0 - sig)
+    return losses, e5m2_satfinite(g), lse
+
+
+# a12: closed form on un-rounded sigma, the pin for ce_fwd_bwd
+
+def _upcast(t: Tensor) -> Tensor:
+    """`.float()` as the reference writes it; an fp64 input (finite-difference checks) is kept."""
+    return t if t.dtype == torch.float64 else t.float()
+
+
+def softcap_ce_closed_form(logits: Tensor, targets: Tensor, A=23.0, B=5.0, C=7.5) -> Tensor:
+    """`F.cross_entropy((23*sigmoid((l+5)/7.5)).float(), targets, reduction="none")`
+    -- train_gpt.py:1689-1692."""
+    z = A * torch.sigmoid((_upcast(logits) + B) / C)
+    return F.cross_entropy(z, targets, reduction="none")
+
+
+def softcap_ce_mtp_closed_form(logits: Tensor, targets: Tensor, mtp_weights: Tensor,
+                               A=23.0, B=5.0, C=7.5) -> Tensor:
+    """logsumexp - gather over shifted targets, tail zeroed -- train_gpt_medium.py:1206-1215.
+    Returns the per-row weighted loss [M] (the reference then sums it)."""
+    z = A * torch.sigmoid((_upcast(logits) + B) / C)
+    n_predict = mtp_weights.shape[0]
+    idx = F.pad(targets, (0, n_predict - 1)).unfold(0, n_predict, 1)
+    ce = torch.logsumexp(z, dim=-1).unsqueeze(1) - z.gather(1, idx)
+    for k in range(1, n_predict):
+        ce[-k:, k] = 0
+    return (ce * mtp_weights.float()).sum(dim=1)
+
+
+# ----------------------------------------------------------------------------
+# a9, a11: FusedSoftcappedCrossEntropy (lm_head GEMM + CE), weight stored (in,out) or (out,in)
+
+def lm_head_ce_fwd(x: Tensor, targets: Tensor, mtp_weights, prefix_targets, prefix_weight,
+                   w: Tensor, x_s: float, w_s: float, grad_s: float, grad_scale: float,
+                   A=23.0, B=5.0, C=7.5, w_layout: str = "in_out"):
+    """FusedSoftcappedCrossEntropy.forward -- triton_kernels.py:1210-1253.
+    Returns (losses [M], ctx) with ctx holding what backward needs."""
+    x_f8 = quant_e4m3(x, x_s)
+    w_f8 = quant_e4m3(w, w_s)
+    w_kn = w_f8 if w_layout == "in_out" else w_f8.T
+    logits = (_mm_f8(x_f8, w_kn) * _scale(x_s, w_s)).to(torch.bfloat16)
+    M, V = logits.shape
+    if mtp_weights is None:
+        mtp_weights = torch.tensor([1.0], dtype=torch.float32)
+    if prefix_targets is None:
+        prefix_targets = torch.full((M,), -1, dtype=torch.int64)
+    if prefix_weight is None:
+        prefix_weight = torch.zeros(1, dtype=torch.float32)
+    prefix_weight = prefix_weight.reshape(1).float()
+    n_predict = mtp_weights.shape[0]
+    losses, dl_f8, lse = ce_fwd_bwd(logits, targets, mtp_weights, prefix_targets, prefix_weight,
+                                    M, n_predict, A, B, C, grad_s, grad_scale)
+    return losses, dict(x_f8=x_f8, w_f8=w_f8, dl_f8=dl_f8, lse=lse, logits=logits,
+                        scales=(x_s, w_s, grad_s), w_layout=w_layout)
+
+
+def lm_head_ce_bwd(ctx):
+    """FusedSoftcappedCrossEntropy.backward -- triton_kernels.py:1255-1292.  The incoming
+    grad_output is ignored (grad_scale was folded in by the kernel, :1117, :1262).
+    Returns (dx [M,K] bf16, dW fp32 in the weight's own layout)."""
+    x_s, w_s, grad_s = ctx["scales"]
+    x_f8, w_f8, dl = ctx["x_f8"], ctx["w_f8"], ctx["dl_f8"]
+    w_vk = w_f8.T if ctx["w_layout"] == "in_out" else w_f8                  # [V, K]
+    dx = (_mm_f8(dl, w_vk) * _scale(grad_s, w_s)).to(torch.bfloat16)
+    dw_kv = _mm_f8(x_f8.T, dl) * _scale(x_s, grad_s)                        # [K, V]
+    dw = dw_kv.contiguous() if ctx["w_layout"] == "in_out" else dw_kv.T.contiguous()
+    return dx, dw
+
+
+def lm_head_ce_chunked(x: Tensor, targets: Tensor, w: Tensor, x_s: float, w_s: float,
+                       grad_s: float, grad_scale: float, A=23.0, B=5.0, C=7.5,
+                       w_layout: str = "out_in", rows_per_chunk: int = 2048,
+                       max_rows: int | None = None):
+    """lm_head_ce_fwd + lm_head_ce_bwd with n_predict = 1 and no prefix targets, processed
+    in row chunks so the [rows, V] intermediates stay bounded; dW accumulated in fp32.
+    `max_rows` stops after that many rows (the benchmark's bounded CPU sample).
+    Returns (losses, dx, dW, rows_done)."""
+    M = x.shape[0] if max_rows is None else min(x.shape[0], max_rows)
+    one = torch.tensor([1.0], dtype=torch.float32)
+    losses, dxs, dw = [], [], None
+    for r0 in range(0, M, rows_per_chunk):
+        r1 = min(M, r0 + rows_per_chunk)
+        l, ctx = lm_head_ce_fwd(x[r0:r1], targets[r0:r1], one, None, None, w, x_s, w_s,
+                                grad_s, grad_scale, A, B, C, w_layout)
+        dx_c, dw_c = lm_head_ce_bwd(ctx)
+        losses.append(l)
+        dxs.append(dx_c)
+        dw = dw_c if dw is None else dw + dw_c
+    return torch.cat(losses), torch.cat(dxs), dw, M
+
+
+# ----------------------------------------------------------------------------
+# Seeded inputs shared by tests, smoke and bench (CPU generator, fp32 draws then cast).
+
+def make_cfg1(seed: int = 0, M: int = 1024, N: int = 3072, K: int = 768):
+    """x ~ N(0,1) bf16 [M,K]; W ~ N(0,1/K) bf16 [N,K]; x_s = 1, w_s = 1/32."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    return x, w, 1.0, 1.0 / 32
+
+
+def make_cfg2(seed: int = 0, M: int = 49152, D: int = 768, H: int = 3072):
+    """RMS-normed x, W_fc ~ N(0,1/D) with per-tensor e4m3 scale, W_proj^T stored [H,D]."""
+    g = torch.Generator().manual_seed(seed)
+    x = rms_norm(torch.randn(M, D, generator=g).bfloat16())
+    w_fc = (torch.randn(H, D, generator=g) / math.sqrt(D)).bfloat16()
+    w_proj = (torch.randn(D, H, generator=g) / math.sqrt(H)).bfloat16()
+    return x, w_fc, w_proj.T.contiguous()
+
+
+def make_cfg3(seed: int = 0, M: int = 49152, K: int = 768, V: int = 50304, n_tok: int = 50257):
+    """x ~ N(0,1), W ~ N(0,1/K) (out,in), reference lm_head scales, uniform targets."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(V, K, generator=g) / math.sqrt(K)).bfloat16()
+    t = torch.randint(0, n_tok, (M,), generator=g, dtype=torch.int64)
+    return x, w, t, dict(x_s=100 / 448, w_s=1.6 / 448, grad_s=0.75 / 448, grad_scale=1.0,
+                         A=23.0, B=5.0, C=7.5)
