@@ -1,0 +1,155 @@
+/*
+ * libngpt_fp8 -- C ABI of the MI355X (gfx950) FP8 contraction path of modded-nanogpt.
+ *
+ * Every entry point
+ *   - takes raw DEVICE pointers, sizes, float scales and a HIP stream (`void* stream` is a
+ *     hipStream_t; NULL is the default stream); no torch types cross this boundary;
+ *   - only enqueues work on `stream` and returns: no host synchronisation, no allocation, no
+ *     pointer is kept after the call.  Scratch memory is passed in by the caller
+ *     (`workspace`, sized by the matching *_workspace_bytes function);
+ *   - returns 0 on success, a negative NGPT_E* code for an argument error (nothing was
+ *     enqueued), or a positive hipError_t if a launch failed.  ngpt_last_error() returns a
+ *     thread-local message for the most recent failure.
+ *
+ * fp8 formats are the OCP ones PyTorch calls float8_e4m3fn (fmt 0) and float8_e5m2 (fmt 1).
+ * Scales follow the reference's divide convention: q = x / s, dequantised value = q * s.
+ * Weight layout: NGPT_W_OUT_IN = weight stored [N, K] (`nanogpt::mm`),
+ *                NGPT_W_IN_OUT = weight stored [K, N] (`nanogpt::mm_t`).
+ *
+ * File:line citations are relative to the reference checkout (KellerJordan/modded-nanogpt).
+ */
+#ifndef NGPT_FP8_H
+#define NGPT_FP8_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NGPT_OK            0
+#define NGPT_EINVAL       -1   /* null pointer / non-positive size */
+#define NGPT_EALIGN       -2   /* a dimension violates the stated divisibility rule */
+#define NGPT_EWORKSPACE   -3   /* workspace too small */
+#define NGPT_ERANGE       -4   /* value outside the supported range (e.g. n_predict, vocab) */
+
+#define NGPT_FMT_E4M3      0
+#define NGPT_FMT_E5M2      1
+
+#define NGPT_W_OUT_IN      0
+#define NGPT_W_IN_OUT      1
+
+#define NGPT_MAX_PREDICT   4   /* n_predict (multi-token prediction depth) supported by the CE kernels */
+
+int ngpt_abi_version(void);
+const char* ngpt_last_error(void);
+
+/* Number of compute units the persistent kernels size their grids to (0 if no device). */
+int ngpt_num_cus(void);
+
+/* ---- quantisers ---------------------------------------------------------------------------
+ * out[i] = fp8(bf16_rne(fp32(in[i]) / scale)), round-to-nearest-even, NOT saturating
+ * (e4m3fn overflow -> NaN code, e5m2 overflow -> +-inf): PyTorch-eager `x.div(s).to(fp8)`.
+ * Replaces the inductor-generated quantise kernels behind train_gpt_medium.py:45-46,75 and
+ * train_gpt.py:78-79,114, triton_kernels.py:1212-1213.  n % 8 == 0. */
+int ngpt_quant_fp8(const void* in_bf16, void* out_f8, int64_t n, float scale, int fmt, void* stream);
+
+/* Same quantiser on a [rows, cols] matrix, writing the row-major copy (out_f8, nullable) and/or
+ * the transposed copy out_f8_t [cols, rows] (nullable) in one pass over the input.  Fuses the
+ * `.T.contiguous()` copies of train_gpt_medium.py:86-87 / train_gpt.py:129-130 into the
+ * quantiser.  rows % 16 == 0, cols % 16 == 0. */
+int ngpt_quant_fp8_2d(const void* in_bf16, int rows, int cols, float scale, int fmt,
+                      void* out_f8, void* out_f8_t, void* stream);
+
+/* out[c, r] = in[r, c] for 1-byte elements: `transpose_copy` (triton_kernels.py:788-841) for
+ * the fp8 operands.  rows % 16 == 0, cols % 16 == 0. */
+int ngpt_transpose_u8(const void* in, int rows, int cols, void* out, void* stream);
+
+/* ---- the GEMM building block --------------------------------------------------------------
+ * C[r, c] = scale * sum_k A[r, k] * B[c, k]; A [R, K] and B [C, K] are fp8 with the contraction
+ * index contiguous (row strides lda / ldb bytes).  What `torch._scaled_mm` does for the
+ * reference (call sites train_gpt_medium.py:47,76,85; train_gpt.py:85,117,128;
+ * triton_kernels.py:1217,1268,1283).  out_kind: 0 = bf16, 1 = fp32, 2 = fp32 accumulate
+ * (C += ...).  ldc in elements.  K % 128 == 0, lda % 16 == 0, ldb % 16 == 0. */
+int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const void* B, int fmt_b, int64_t ldb,
+                     int R, int C, int K, float scale, void* out, int64_t ldc, int out_kind,
+                     void* stream);
+
+/* ---- nanogpt::mm / nanogpt::mm_t forward --------------------------------------------------
+ * train_gpt_medium.py:40-57 (w_layout OUT_IN, w [N,K]) and train_gpt.py:70-95 (IN_OUT, w [K,N]).
+ * x [M,K] bf16.  Writes out [M,N] bf16 = bf16((x_f8 . w_f8^T) * x_s * w_s), x_f8 [M,K] e4m3 and
+ * w_f8 (e4m3, same layout as w).  K % 128 == 0, M % 16 == 0, N % 16 == 0. */
+int64_t ngpt_mm_fwd_workspace_bytes(int M, int N, int K, int w_layout);
+int ngpt_mm_fwd(const void* x_bf16, const void* w_bf16, int M, int N, int K, float x_s, float w_s,
+                void* out_bf16, void* x_f8, void* w_f8, int w_layout,
+                void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- nanogpt::mm_backward / nanogpt::mm_t_backward ----------------------------------------
+ * train_gpt_medium.py:67-95 and train_gpt.py:105-141.  g [M,N] bf16 is quantised to e5m2 with
+ * grad_s; dx [M,K] bf16 = (g_f8 . w_f8) * grad_s * w_s; dw_kn [K,N] fp32 contiguous =
+ * (x_f8^T . g_f8) * x_s * grad_s.  For OUT_IN the caller exposes dw_kn as its transposed view
+ * ([N,K], strides (1,N)), exactly the reference's `.T`.  M % 128 == 0, N % 128 == 0, K % 16 == 0. */
+int64_t ngpt_mm_bwd_workspace_bytes(int M, int N, int K, int w_layout);
+int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f8, int M, int N, int K,
+                float x_s, float w_s, float grad_s, void* dx_bf16, void* dw_kn_f32, int w_layout,
+                void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- FP8 MLP up-projection with fused ReLU^2 ----------------------------------------------
+ * linear_relu_square_kernel FORWARD+USE_FP8(+EMIT_FP8) and its launcher, triton_kernels.py:402-499,
+ * 576-665.  x_f8 [M,K] e4m3, w_f8 [N,K] e4m3, dequant: 1-element fp32 DEVICE tensor.
+ * post [M,N] bf16 = bf16(max(bf16(acc * *dequant), 0)^2).  If post_f8 != NULL also writes
+ * post_f8 [M,N] = e4m3(min(post / *act_scale, 448)) and partial_amax[i] (n_partials fp32 entries;
+ * entry i = running max of `post` seen by persistent workgroup i, 0 for unused entries).
+ * K % 128 == 0, N % 16 == 0. */
+int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, int M, int N, int K,
+                      void* post_bf16, void* post_f8, const float* act_scale,
+                      float* partial_amax, int n_partials, void* stream);
+
+/* ---- nanogpt::ce_fwd_bwd on materialised logits -------------------------------------------
+ * ce_fwd_bwd_kernel, triton_kernels.py:956-1170, 1182-1206.  logits [n_rows, n_cols] bf16,
+ * targets/prefix_targets int64 [n_rows], mtp_weights fp32 [n_predict], prefix_weight fp32 [1].
+ * prefix_targets / prefix_weight may be NULL (no prefix term).
+ * Writes losses fp32 [n_rows] and grad e5m2 [n_rows, n_cols] (saturating store).
+ * n_cols % 8 == 0, 1 <= n_predict <= NGPT_MAX_PREDICT.  The workspace holds two lookup
+ * tables over the bf16 logit values. */
+int64_t ngpt_ce_fwd_bwd_workspace_bytes(void);
+int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, const float* mtp_weights,
+                    const int64_t* prefix_targets, const float* prefix_weight,
+                    float* losses, void* grad_e5m2, int n_rows, int n_cols, int n_predict,
+                    float A, float B, float C, float grad_s, float grad_scale,
+                    void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- fused lm_head + softcapped cross-entropy ---------------------------------------------
+ * FusedSoftcappedCrossEntropy.forward/backward, triton_kernels.py:1208-1292, without the
+ * [M, V] logits (or their gradient) ever being stored: the forward keeps per-row softmax
+ * statistics from vocabulary tiles, the backward recomputes the logits tile by tile.
+ *
+ * Forward: x [M,K] bf16, w bf16 in `w_layout` ([V,K] or [K,V]).  Writes losses [M] fp32 and,
+ * saved for backward: lse [M] fp32 (log-sum-exp of the softcapped logits), saved_sigma
+ * [(NGPT_MAX_PREDICT + 1) * M] fp32 (the bf16-rounded sigmoid at every candidate target column;
+ * entries of invalid targets are left untouched), x_f8 [M,K] and w_f8_vk [V,K] (e4m3, always
+ * vocabulary-major).  K % 128 == 0, M % 16 == 0, V % 16 == 0. */
+int64_t ngpt_lmhead_ce_fwd_workspace_bytes(int M, int K, int V, int w_layout);
+int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const int64_t* targets,
+                       const float* mtp_weights, int n_predict,
+                       const int64_t* prefix_targets, const float* prefix_weight,
+                       int M, int K, int V, float x_s, float w_s, float A, float B, float C,
+                       float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
+                       int w_layout, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Backward: gradients of sum(losses) * grad_scale (the incoming autograd gradient is ignored,
+ * as in triton_kernels.py:1117,1262).  dx [M,K] bf16; dw fp32 in the weight's own layout
+ * ([V,K] for OUT_IN, [K,V] for IN_OUT).  M % 128 == 0, V % 128 == 0, K % 128 == 0. */
+int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout);
+int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const int64_t* targets,
+                       const float* mtp_weights, int n_predict,
+                       const int64_t* prefix_targets, const float* prefix_weight,
+                       const float* lse, const float* saved_sigma, int M, int K, int V,
+                       float x_s, float w_s, float grad_s, float grad_scale,
+                       float A, float B, float C, void* dx_bf16, void* dw_f32, int w_layout,
+                       void* workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NGPT_FP8_H */

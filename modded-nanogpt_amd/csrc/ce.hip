@@ -1,0 +1,631 @@
+// Softcapped cross-entropy: the standalone op on materialised logits and the lm_head-fused
+// forward/backward that never stores the [M, V] logits.
+//
+// Reference semantics (ce_fwd_bwd_kernel): a logit l is a bf16 number; sigma = bf16(sigmoid(l/C + B/C));
+// z = A*sigma; loss = sum_k w_k (lse - z[target_k]); dlogit = coef * (S_w * p - term2) * sigma * (1 - sigma),
+// p = exp(z - lse), coef = grad_scale * (A/C) / grad_s, stored as saturating e5m2.
+//
+// Because l is a bf16 number, everything that depends only on l is a function of 16 bits.  Two
+// tables indexed by the logit's bit pattern replace all transcendental work in the hot loops:
+//   tabE[i] = exp(z - A)                     (forward: sum of exponentials, shifted by the cap A)
+//   tabD[i] = exp(z - A) * sigma * (1-sigma) (backward: dlogit = rowf[m] * tabD[i])
+// with rowf[m] = coef * S_w[m] * exp(A - lse[m]).  The tables cover |l| in [2^-16, 2^8) exactly
+// (128 mantissa steps per binade, both signs); smaller magnitudes share the entry of l = 0 and
+// larger ones the last entry, where sigma has saturated in bf16.
+#include "epilogues.h"
+#include "host_util.h"
+#include "launch.h"
+
+namespace ngpt {
+
+constexpr int TAB_LO = 0x3780;            // bf16 bits of 2^-16
+constexpr int TAB_N = 0x4380 - 0x3780;    // 3072 entries per sign, up to 2^8
+constexpr int TAB_ENTRIES = 2 * TAB_N;
+constexpr int TAB_BYTES = TAB_ENTRIES * 4;
+constexpr int MAX_CAND = NGPT_MAX_PREDICT + 1;   // shifted targets + the prefix target
+
+struct Softcap {
+    float A, inv_C, B_div_C;
+};
+
+__device__ __forceinline__ int tab_index(uint32_t bf16_bits) {
+    int t = (int)(bf16_bits & 0x7fffu) - TAB_LO;
+    t = max(0, min(t, TAB_N - 1));
+    return t + (int)(bf16_bits >> 15) * TAB_N;
+}
+
+// bf16(sigmoid(l * inv_C + B_div_C)) as an fp32 value; mul and add rounded separately.
+__device__ __forceinline__ float softcap_sigma(float l, const Softcap& sc) {
+    float u = __fadd_rn(__fmul_rn(l, sc.inv_C), sc.B_div_C);
+    float s = __fdiv_rn(1.0f, 1.0f + expf(-u));
+    return round_to_bf16(s);
+}
+__device__ __forceinline__ float softcap_E(float sigma, const Softcap& sc) { return expf(sc.A * sigma - sc.A); }
+
+__global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= TAB_ENTRIES) return;
+    int t = i % TAB_N, neg = i / TAB_N;
+    uint32_t bits = t == 0 ? 0u : (uint32_t)(TAB_LO + t);
+    float l = bf16_bits_to_f32(bits | (neg ? 0x8000u : 0u));
+    float s = softcap_sigma(l, sc);
+    float e = softcap_E(s, sc);
+    tabE[i] = e;
+    tabD[i] = e * s * (1.0f - s);
+}
+
+__global__ void fill_f32_kernel(float* p, int64_t n, float v) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+__device__ __forceinline__ void load_table(float* lds_tab, const float* gtab) {
+    for (int i = threadIdx.x; i < TAB_ENTRIES; i += blockDim.x) lds_tab[i] = gtab[i];
+}
+
+struct CandArgs {
+    const int64_t* targets;          // [M]
+    const int64_t* prefix_targets;   // [M], nullable
+    const float* mtp_weights;        // [n_predict]
+    const float* prefix_weight;      // [1], nullable
+    int n_predict;
+    int M, V;
+};
+
+// Candidate c of row m: c < n_predict -> targets[m + c] (if m + c < M), c == n_predict -> prefix target.
+__device__ __forceinline__ int64_t cand_target(const CandArgs& ca, int m, int c) {
+    if (c < ca.n_predict) return (m + c < ca.M) ? ca.targets[m + c] : -1;
+    return ca.prefix_targets ? ca.prefix_targets[m] : -1;
+}
+__device__ __forceinline__ float cand_weight(const CandArgs& ca, int c) {
+    if (c < ca.n_predict) return ca.mtp_weights[c];
+    return ca.prefix_weight ? ca.prefix_weight[0] : 0.0f;
+}
+// Normaliser weight of a row: all n_predict weights (no bounds check on the shifted index, as in the
+// reference) plus the prefix weight when the prefix target is valid.
+__device__ __forceinline__ float row_weight_sum(const CandArgs& ca, int m) {
+    float s = 0.0f;
+    for (int k = 0; k < ca.n_predict; ++k) s += ca.mtp_weights[k];
+    int64_t pt = ca.prefix_targets ? ca.prefix_targets[m] : -1;
+    if (pt >= 0 && pt < ca.V) s += cand_weight(ca, ca.n_predict);
+    return s;
+}
+
+// =====================================================================================================
+// Standalone op on materialised logits: one workgroup walks rows; two sweeps over a row (the second
+// one re-reads it from L2) instead of caching 100 KB per row in LDS.
+constexpr int ROW_THREADS = 512;
+
+__device__ __forceinline__ float block_sum(float v, float* red /* >= 16 floats */) {
+    v = wave_sum(v);
+    int wave = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float t = 0.0f;
+    for (int w = 0; w < (int)(blockDim.x >> 6); ++w) t += red[w];
+    return t;
+}
+
+__global__ __launch_bounds__(ROW_THREADS) void ce_rows_kernel(
+    const uint16_t* __restrict__ logits, CandArgs ca, float* __restrict__ losses, uint8_t* __restrict__ grad,
+    const float* __restrict__ gtabE, const float* __restrict__ gtabD, Softcap sc, float coef) {
+    __shared__ float tabE[TAB_ENTRIES];
+    __shared__ float tabD[TAB_ENTRIES];
+    __shared__ float red[16];
+    load_table(tabE, gtabE);
+    load_table(tabD, gtabD);
+    __syncthreads();
+    const int V = ca.V, n8 = V / 8;
+    for (int row = blockIdx.x; row < ca.M; row += gridDim.x) {
+        const uint16_t* lrow = logits + (int64_t)row * V;
+        float sum = 0.0f;
+        for (int i = threadIdx.x; i < n8; i += ROW_THREADS) {
+            v4i w = *(const v4i*)(lrow + i * 8);
+            uint32_t u[4] = {(uint32_t)w.x, (uint32_t)w.y, (uint32_t)w.z, (uint32_t)w.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sum += tabE[tab_index(u[j] & 0xffffu)] + tabE[tab_index(u[j] >> 16)];
+        }
+        float S = block_sum(sum, red);
+        float lse = sc.A + logf(S);
+        float s_w = row_weight_sum(ca, row);
+        float p_scale = expf(sc.A - lse);
+        float rowf = coef * (s_w * p_scale);
+        if (threadIdx.x == 0) {
+            float total = 0.0f;
+            for (int c = 0; c <= ca.n_predict; ++c) {
+                int64_t t = cand_target(ca, row, c);
+                if (t >= 0 && t < V) {
+                    float sg = softcap_sigma(bf16_bits_to_f32(lrow[t]), sc);
+                    total += cand_weight(ca, c) * (lse - sc.A * sg);
+                }
+            }
+            losses[row] = total;
+        }
+        uint8_t* grow = grad + (int64_t)row * V;
+        for (int i = threadIdx.x; i < n8; i += ROW_THREADS) {
+            v4i w = *(const v4i*)(lrow + i * 8);
+            uint32_t u[4] = {(uint32_t)w.x, (uint32_t)w.y, (uint32_t)w.z, (uint32_t)w.w};
+            float g[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                g[2 * j] = rowf * tabD[tab_index(u[j] & 0xffffu)];
+                g[2 * j + 1] = rowf * tabD[tab_index(u[j] >> 16)];
+            }
+            v2i o;
+            o.x = (int)f32x4_to_e5m2_sat(g[0], g[1], g[2], g[3]);
+            o.y = (int)f32x4_to_e5m2_sat(g[4], g[5], g[6], g[7]);
+            *(v2i*)(grow + i * 8) = o;
+        }
+        __syncthreads();   // dense stores of this row are complete before the target columns are rewritten
+        if ((int)threadIdx.x <= ca.n_predict) {
+            int c = threadIdx.x;
+            int64_t t = cand_target(ca, row, c);
+            if (t >= 0 && t < V) {
+                float sg = softcap_sigma(bf16_bits_to_f32(lrow[t]), sc);
+                float p = softcap_E(sg, sc) * p_scale;
+                float term2 = 0.0f;
+                for (int k = 0; k <= ca.n_predict; ++k) {
+                    int64_t tk = cand_target(ca, row, k);
+                    if (tk == t) term2 += cand_weight(ca, k);     // every prediction that lands on this column
+                }
+                float gz = s_w * p - term2;
+                float gx = coef * gz * sg * (1.0f - sg);
+                grow[t] = (uint8_t)(f32x2_to_e5m2_sat(gx, gx) & 0xffu);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// =====================================================================================================
+// Fused forward.  GEMM orientation: rows = vocabulary (A = w_f8 [V, K]), columns = tokens
+// (B = x_f8 [M, K]), so one lane owns one token per MFMA tile column and sums exponentials in
+// registers.  A job = (token tile, vocabulary split); XCD x (workgroups with bid % 8 == x) only
+// handles split x, so each XCD streams one eighth of the weight matrix and keeps it in its L2.
+constexpr int CE_SPLITS = 8;
+
+struct CEJobIter {
+    int tiles_v, tiles_m, slot, nslots, split, it, tr_, tr_end;
+    __device__ CEJobIter(const GemmOperands& g, int BM, int BN, int bid, int G) {
+        tiles_v = (g.R + BM - 1) / BM;
+        tiles_m = (g.C + BN - 1) / BN;
+        split = bid % CE_SPLITS;
+        slot = bid / CE_SPLITS;
+        nslots = G / CE_SPLITS;
+        it = 0;
+        tr_ = tiles_v * split / CE_SPLITS;
+        tr_end = tiles_v * (split + 1) / CE_SPLITS;
+        if (tr_ >= tr_end) it = tiles_m;     // empty vocabulary range: nothing to do
+    }
+    __device__ bool valid() const { return slot + it * nslots < tiles_m; }
+    __device__ int tr() const { return tr_; }
+    __device__ int tc() const { return slot + it * nslots; }
+    __device__ bool job_end() const { return tr_ + 1 == tr_end; }
+    __device__ int job_id() const { return split; }
+    __device__ void advance() {
+        if (++tr_ == tr_end) {
+            tr_ = tiles_v * split / CE_SPLITS;
+            ++it;
+        }
+    }
+};
+
+struct EpiCEFwd {
+    static constexpr int EXTRA_LDS = TAB_BYTES;
+    const float* gtabE;
+    float* part;          // [CE_SPLITS][M] partial sums of exp(z - A)
+    float* saved_sigma;   // [MAX_CAND][M] bf16-rounded sigma at each candidate target column
+    CandArgs ca;
+    Softcap sc;
+    float scale;
+    float* tab;
+    float sum[8];
+
+    __device__ void begin(int, int, uint8_t* extra) {
+        tab = (float*)extra;
+        load_table(tab, gtabE);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum[i] = 0.0f;
+    }
+    __device__ void end(uint8_t*, int, int) {}
+
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0 /* vocab */, int c0 /* token */,
+                         const AccCoords<Cfg>& co, uint8_t*, int lane) {
+        static_assert(Cfg::TN <= 8, "per-lane token columns");
+        const int V = ca.V, M = ca.M;
+        const bool partial = (r0 + Cfg::BM > V);
+#pragma unroll
+        for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < Cfg::TN; ++tn) {
+                float s = 0.0f;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    float e = tab[tab_index(f32_to_bf16_bits(acc[tm][tn][v] * scale))];
+                    if (partial) e = (r0 + co.row(tm, v) < V) ? e : 0.0f;
+                    s += e;
+                }
+                sum[tn] += s;
+            }
+        // sigma at candidate target columns that fall inside this wave's vocabulary rows (rare)
+        const int v_lo = r0 + co.wave_row0, v_hi = v_lo + Cfg::WTM;
+#pragma unroll
+        for (int tn = 0; tn < Cfg::TN; ++tn) {
+            int m = c0 + co.col(tn);
+            for (int c = 0; c <= ca.n_predict; ++c) {
+                int64_t t = (m < M) ? cand_target(ca, m, c) : -1;
+                bool hit = (t >= v_lo && t < v_hi && t < V);
+                if (__any(hit)) {
+                    int rl = hit ? (int)t - v_lo : -1;
+                    float got = 0.0f;
+                    bool mine = false;
+#pragma unroll
+                    for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            int r = co.row(tm, v) - co.wave_row0;
+                            if (r == rl) { got = acc[tm][tn][v]; mine = true; }
+                        }
+                    if (mine) saved_sigma[(int64_t)c * M + m] = softcap_sigma(round_to_bf16(got * scale), sc);
+                }
+            }
+        }
+    }
+
+    // Fold the lane sums of one finished (token tile, split) job into part[split][m].
+    template <class Cfg>
+    __device__ void job_end(int c0, int split, const AccCoords<Cfg>& co, uint8_t* scratch) {
+        float* red = (float*)scratch;                    // [WAVES_M][BN]
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int wr = wave / Cfg::WAVES_N;
+#pragma unroll
+        for (int tn = 0; tn < Cfg::TN; ++tn) {
+            float s = sum[tn] + __shfl_xor(sum[tn], 32, 64);
+            if (lane < 32) red[wr * Cfg::BN + co.col(tn)] = s;
+            sum[tn] = 0.0f;
+        }
+        __syncthreads();
+        for (int j = threadIdx.x; j < Cfg::BN; j += Cfg::THREADS) {
+            float s = 0.0f;
+#pragma unroll
+            for (int w = 0; w < Cfg::WAVES_M; ++w) s += red[w * Cfg::BN + j];
+            int m = c0 + j;
+            if (m < ca.M) part[(int64_t)split * ca.M + m] = s;
+        }
+    }
+};
+
+__global__ void ce_finalize_kernel(const float* __restrict__ part, const float* __restrict__ saved_sigma,
+                                   CandArgs ca, Softcap sc, float* __restrict__ losses, float* __restrict__ lse_out) {
+    int m = blockIdx.x * blockDim.x + threadIdx.x;
+    if (m >= ca.M) return;
+    float S = 0.0f;
+    for (int s = 0; s < CE_SPLITS; ++s) S += part[(int64_t)s * ca.M + m];
+    float lse = sc.A + logf(S);
+    float total = 0.0f;
+    for (int c = 0; c <= ca.n_predict; ++c) {
+        int64_t t = cand_target(ca, m, c);
+        if (t >= 0 && t < ca.V) total += cand_weight(ca, c) * (lse - sc.A * saved_sigma[(int64_t)c * ca.M + m]);
+    }
+    losses[m] = total;
+    lse_out[m] = lse;
+}
+
+// =====================================================================================================
+// Backward, recomputing the logits.  rowf[m] = coef * S_w[m] * exp(A - lse[m]).
+__global__ void ce_rowf_kernel(const float* __restrict__ lse, CandArgs ca, Softcap sc, float coef,
+                               float* __restrict__ rowf) {
+    int m = blockIdx.x * blockDim.x + threadIdx.x;
+    if (m >= ca.M) return;
+    rowf[m] = coef * (row_weight_sum(ca, m) * expf(sc.A - lse[m]));
+}
+
+// GEMM orientation: rows = tokens of the current chunk (A = x_f8), columns = vocabulary (B = w_f8).
+// Writes the e5m2 dlogits of the chunk row-major (dl [Mc, V]) and transposed (dl_t [V, Mc]).
+struct EpiDlStore {
+    static constexpr int EXTRA_LDS = TAB_BYTES;
+    const float* gtabD;
+    const float* rowf;     // already offset to the chunk's first row
+    uint8_t* dl;           // [Mc, V]
+    uint8_t* dl_t;         // [V, Mc]
+    int Mc, V;
+    float scale;
+    float* tab;
+
+    __device__ void begin(int, int, uint8_t* extra) {
+        tab = (float*)extra;
+        load_table(tab, gtabD);
+    }
+    __device__ void end(uint8_t*, int, int) {}
+    template <class Cfg>
+    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
+                         uint8_t* scratch, int lane) {
+        const int h = lane >> 5;
+        uint32_t pk[Cfg::TM][Cfg::TN][4];
+#pragma unroll
+        for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                int row = r0 + co.wave_row0 + tm * 32 + 8 * g + 4 * h;
+                v4f rf = (row + 4 <= Mc) ? *(const v4f*)(rowf + row) : (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int tn = 0; tn < Cfg::TN; ++tn) {
+                    float d[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        d[i] = rf[i] * tab[tab_index(f32_to_bf16_bits(acc[tm][tn][4 * g + i] * scale))];
+                    pk[tm][tn][g] = f32x4_to_e5m2_sat(d[0], d[1], d[2], d[3]);
+                }
+            }
+        // row-major copy: one 32-row strip per tm
+#pragma unroll
+        for (int tm = 0; tm < Cfg::TM; ++tm) {
+            uint32_t codes[Cfg::TN][16];
+#pragma unroll
+            for (int tn = 0; tn < Cfg::TN; ++tn)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) codes[tn][v] = (pk[tm][tn][v >> 2] >> (8 * (v & 3))) & 0xffu;
+            store_strip_rowmajor_u8<Cfg>(codes, scratch, lane, dl, V, r0 + co.wave_row0 + tm * 32,
+                                         c0 + co.wave_col0, Mc, V);
+        }
+        // transposed copy: one 32-column strip per tn
+#pragma unroll
+        for (int tn = 0; tn < Cfg::TN; ++tn) {
+            uint32_t packed[Cfg::TM][4];
+#pragma unroll
+            for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) packed[tm][g] = pk[tm][tn][g];
+            store_strip_transposed_u8<Cfg>(packed, scratch, lane, dl_t, Mc, r0 + co.wave_row0,
+                                           c0 + co.wave_col0 + tn * 32, Mc, V);
+        }
+    }
+};
+
+// Rewrites the (at most MAX_CAND) target columns of every row of the chunk with the exact gradient.
+__global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __restrict__ saved_sigma,
+                                 CandArgs ca, Softcap sc, float coef, int m_begin, int Mc,
+                                 uint8_t* __restrict__ dl, uint8_t* __restrict__ dl_t) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= Mc) return;
+    int m = m_begin + i;
+    float s_w = row_weight_sum(ca, m);
+    float p_scale = expf(sc.A - lse[m]);
+    for (int c = 0; c <= ca.n_predict; ++c) {
+        int64_t t = cand_target(ca, m, c);
+        if (t < 0 || t >= ca.V) continue;
+        float term2 = 0.0f;
+        for (int k = 0; k <= ca.n_predict; ++k)
+            if (cand_target(ca, m, k) == t) term2 += cand_weight(ca, k);
+        float sg = saved_sigma[(int64_t)c * ca.M + m];
+        float gz = s_w * (softcap_E(sg, sc) * p_scale) - term2;
+        float gx = coef * gz * sg * (1.0f - sg);
+        uint8_t code = (uint8_t)(f32x2_to_e5m2_sat(gx, gx) & 0xffu);
+        dl[(int64_t)i * ca.V + t] = code;
+        dl_t[(int64_t)t * Mc + i] = code;
+    }
+}
+
+int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
+               float scale, void* out, int64_t ldc, int out_kind, hipStream_t st);
+
+static Softcap make_softcap(float A, float B, float C) {
+    Softcap sc;
+    sc.A = A;
+    sc.inv_C = 1.0f / C;
+    sc.B_div_C = B * sc.inv_C;
+    return sc;
+}
+// grad_scale * (1/C * A) * (1/grad_s), in the reference's fp32 order
+static float make_coef(float A, float C, float grad_s, float grad_scale) {
+    return grad_scale * (1.0f / C * A) * (1.0f / grad_s);
+}
+
+static int check_cand(const char* who, const int64_t* targets, const float* mtp_weights, int n_predict) {
+    if (!targets || !mtp_weights) return fail(NGPT_EINVAL, "%s: targets / mtp_weights are required", who);
+    if (n_predict < 1 || n_predict > NGPT_MAX_PREDICT)
+        return fail(NGPT_ERANGE, "%s: n_predict=%d outside [1, %d]", who, n_predict, NGPT_MAX_PREDICT);
+    return NGPT_OK;
+}
+
+constexpr int BWD_CHUNK_ROWS = 16384;
+static int bwd_chunk_rows(int M) { return M < BWD_CHUNK_ROWS ? M : BWD_CHUNK_ROWS; }
+
+}  // namespace ngpt
+
+using namespace ngpt;
+
+// ------------------------------------------------------------------------------------------------
+extern "C" int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, const float* mtp_weights,
+                               const int64_t* prefix_targets, const float* prefix_weight,
+                               float* losses, void* grad_e5m2, int n_rows, int n_cols, int n_predict,
+                               float A, float B, float C, float grad_s, float grad_scale,
+                               void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!logits_bf16 || !losses || !grad_e5m2) return fail(NGPT_EINVAL, "ngpt_ce_fwd_bwd: null pointer");
+    if (int e = check_cand("ngpt_ce_fwd_bwd", targets, mtp_weights, n_predict)) return e;
+    if (n_rows <= 0 || n_cols <= 0) return fail(NGPT_EINVAL, "ngpt_ce_fwd_bwd: empty logits %d x %d", n_rows, n_cols);
+    if (n_cols % 8) return fail(NGPT_EALIGN, "ngpt_ce_fwd_bwd: n_cols=%d must be a multiple of 8", n_cols);
+    if (!workspace || workspace_bytes < 2 * TAB_BYTES)
+        return fail(NGPT_EWORKSPACE, "ngpt_ce_fwd_bwd: workspace %lld < %d bytes", (long long)workspace_bytes, 2 * TAB_BYTES);
+    hipStream_t st = (hipStream_t)stream;
+    Softcap sc = make_softcap(A, B, C);
+    float* tabE = (float*)workspace;
+    float* tabD = tabE + TAB_ENTRIES;
+    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
+    CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, n_rows, n_cols};
+    int grid = num_cus() * 2;
+    if (grid <= 0) return fail(NGPT_EINVAL, "no HIP device");
+    if (grid > n_rows) grid = n_rows;
+    ce_rows_kernel<<<grid, ROW_THREADS, 0, st>>>((const uint16_t*)logits_bf16, ca, losses, (uint8_t*)grad_e5m2,
+                                                 tabE, tabD, sc, make_coef(A, C, grad_s, grad_scale));
+    return check_launch("ce_rows_kernel");
+}
+
+extern "C" int64_t ngpt_ce_fwd_bwd_workspace_bytes(void) { return 2 * TAB_BYTES; }
+
+// ------------------------------------------------------------------------------------------------
+// forward workspace: tabE | tabD | part [CE_SPLITS][M] | (IN_OUT only) nothing extra: the transposed
+// quantiser writes w_f8_vk directly.
+extern "C" int64_t ngpt_lmhead_ce_fwd_workspace_bytes(int M, int K, int V, int w_layout) {
+    (void)K; (void)V; (void)w_layout;
+    return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)CE_SPLITS * M * 4, 256);
+}
+
+extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const int64_t* targets,
+                                  const float* mtp_weights, int n_predict,
+                                  const int64_t* prefix_targets, const float* prefix_weight,
+                                  int M, int K, int V, float x_s, float w_s, float A, float B, float C,
+                                  float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
+                                  int w_layout, void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!x_bf16 || !w_bf16 || !losses || !lse || !saved_sigma || !x_f8 || !w_f8_vk || !workspace)
+        return fail(NGPT_EINVAL, "ngpt_lmhead_ce_fwd: null pointer");
+    if (int e = check_cand("ngpt_lmhead_ce_fwd", targets, mtp_weights, n_predict)) return e;
+    if (M <= 0 || K <= 0 || V <= 0) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_fwd: empty problem M=%d K=%d V=%d", M, K, V);
+    if (K % 128 || M % 16 || V % 16)
+        return fail(NGPT_EALIGN, "ngpt_lmhead_ce_fwd: need K %% 128 == 0, M %% 16 == 0, V %% 16 == 0 (M=%d K=%d V=%d)", M, K, V);
+    if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_fwd: w_layout=%d", w_layout);
+    int64_t need = ngpt_lmhead_ce_fwd_workspace_bytes(M, K, V, w_layout);
+    if (workspace_bytes < need)
+        return fail(NGPT_EWORKSPACE, "ngpt_lmhead_ce_fwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
+    hipStream_t st = (hipStream_t)stream;
+    uint8_t* ws = (uint8_t*)workspace;
+    float* tabE = (float*)ws;
+    float* tabD = tabE + TAB_ENTRIES;
+    float* part = (float*)(ws + align_up(2 * TAB_BYTES, 256));
+
+    Softcap sc = make_softcap(A, B, C);
+    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
+    // a vocabulary split can be empty for a tiny V; its partial sums must read as zero
+    fill_f32_kernel<<<(CE_SPLITS * M + 255) / 256, 256, 0, st>>>(part, (int64_t)CE_SPLITS * M, 0.0f);
+    if (int e = ngpt_quant_fp8(x_bf16, x_f8, (int64_t)M * K, x_s, NGPT_FMT_E4M3, stream)) return e;
+    if (w_layout == NGPT_W_OUT_IN) {
+        if (int e = ngpt_quant_fp8(w_bf16, w_f8_vk, (int64_t)V * K, w_s, NGPT_FMT_E4M3, stream)) return e;
+    } else {
+        if (int e = ngpt_quant_fp8_2d(w_bf16, K, V, w_s, NGPT_FMT_E4M3, nullptr, w_f8_vk, stream)) return e;
+    }
+
+    using Cfg = MainCfg;
+    GemmOperands g{(const uint8_t*)w_f8_vk, (const uint8_t*)x_f8, K, K, V, M, K};
+    EpiCEFwd epi{};
+    epi.gtabE = tabE;
+    epi.part = part;
+    epi.saved_sigma = saved_sigma;
+    epi.ca = CandArgs{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
+    epi.sc = sc;
+    epi.scale = x_s * w_s;
+    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, EpiCEFwd, CEJobIter>;
+    constexpr int LDS = Cfg::SMEM_BYTES + EpiCEFwd::EXTRA_LDS;
+    static bool configured = false;
+    if (!configured) {
+        if (int e = allow_lds(kernel, LDS)) return e;
+        configured = true;
+    }
+    int cus = num_cus();
+    if (cus < CE_SPLITS) return fail(NGPT_EINVAL, "no HIP device");
+    int tiles_m = (M + Cfg::BN - 1) / Cfg::BN;
+    int slots = cus / CE_SPLITS < tiles_m ? cus / CE_SPLITS : tiles_m;
+    kernel<<<slots * CE_SPLITS, Cfg::THREADS, LDS, st>>>(g, epi);
+    if (int e = check_launch("lm_head CE forward")) return e;
+    ce_finalize_kernel<<<(M + 255) / 256, 256, 0, st>>>(part, saved_sigma, epi.ca, sc, losses, lse);
+    return check_launch("ce_finalize_kernel");
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward workspace: tabE | tabD | rowf [M] | x_f8^T [K, M] | w_f8^T [K, V] | dl [Mc, V] | dl^T [V, Mc]
+extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
+    (void)w_layout;
+    int64_t Mc = bwd_chunk_rows(M);
+    return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)M * 4, 256) + align_up((int64_t)K * M, 256) +
+           align_up((int64_t)K * V, 256) + 2 * align_up(Mc * V, 256);
+}
+
+extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const int64_t* targets,
+                                  const float* mtp_weights, int n_predict,
+                                  const int64_t* prefix_targets, const float* prefix_weight,
+                                  const float* lse, const float* saved_sigma, int M, int K, int V,
+                                  float x_s, float w_s, float grad_s, float grad_scale,
+                                  float A, float B, float C, void* dx_bf16, void* dw_f32, int w_layout,
+                                  void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!x_f8 || !w_f8_vk || !lse || !saved_sigma || !dx_bf16 || !dw_f32 || !workspace)
+        return fail(NGPT_EINVAL, "ngpt_lmhead_ce_bwd: null pointer");
+    if (int e = check_cand("ngpt_lmhead_ce_bwd", targets, mtp_weights, n_predict)) return e;
+    if (M <= 0 || K <= 0 || V <= 0) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_bwd: empty problem M=%d K=%d V=%d", M, K, V);
+    if (K % 128 || M % 128 || V % 128)
+        return fail(NGPT_EALIGN, "ngpt_lmhead_ce_bwd: need M, K, V multiples of 128 (M=%d K=%d V=%d)", M, K, V);
+    if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_bwd: w_layout=%d", w_layout);
+    int64_t need = ngpt_lmhead_ce_bwd_workspace_bytes(M, K, V, w_layout);
+    if (workspace_bytes < need)
+        return fail(NGPT_EWORKSPACE, "ngpt_lmhead_ce_bwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
+    hipStream_t st = (hipStream_t)stream;
+    const int Mc_max = bwd_chunk_rows(M);
+    uint8_t* ws = (uint8_t*)workspace;
+    float* tabE = (float*)ws;
+    float* tabD = tabE + TAB_ENTRIES;
+    ws += align_up(2 * TAB_BYTES, 256);
+    float* rowf = (float*)ws;
+    ws += align_up((int64_t)M * 4, 256);
+    uint8_t* x_t = ws;
+    ws += align_up((int64_t)K * M, 256);
+    uint8_t* w_t = ws;
+    ws += align_up((int64_t)K * V, 256);
+    uint8_t* dl = ws;
+    ws += align_up((int64_t)Mc_max * V, 256);
+    uint8_t* dl_t = ws;
+
+    Softcap sc = make_softcap(A, B, C);
+    const float coef = make_coef(A, C, grad_s, grad_scale);
+    CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
+    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
+    ce_rowf_kernel<<<(M + 255) / 256, 256, 0, st>>>(lse, ca, sc, coef, rowf);
+    if (int e = check_launch("ce_rowf_kernel")) return e;
+    if (int e = ngpt_transpose_u8(x_f8, M, K, x_t, stream)) return e;
+    if (int e = ngpt_transpose_u8(w_f8_vk, V, K, w_t, stream)) return e;
+
+    using Cfg = MainCfg;
+    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, EpiDlStore, GridIter>;
+    constexpr int LDS = Cfg::SMEM_BYTES + EpiDlStore::EXTRA_LDS;
+    static bool configured = false;
+    if (!configured) {
+        if (int e = allow_lds(kernel, LDS)) return e;
+        configured = true;
+    }
+    const int cus = num_cus();
+    if (cus <= 0) return fail(NGPT_EINVAL, "no HIP device");
+    for (int m0 = 0; m0 < M; m0 += Mc_max) {
+        const int Mc = (M - m0 < Mc_max) ? (M - m0) : Mc_max;
+        // 1. recompute the chunk's logits and turn them into e5m2 dlogits (both layouts)
+        GemmOperands g{(const uint8_t*)x_f8 + (int64_t)m0 * K, (const uint8_t*)w_f8_vk, K, K, Mc, V, K};
+        EpiDlStore epi{};
+        epi.gtabD = tabD;
+        epi.rowf = rowf + m0;
+        epi.dl = dl;
+        epi.dl_t = dl_t;
+        epi.Mc = Mc;
+        epi.V = V;
+        epi.scale = x_s * w_s;
+        int tiles = ((Mc + Cfg::BM - 1) / Cfg::BM) * ((V + Cfg::BN - 1) / Cfg::BN);
+        kernel<<<tiles < cus ? tiles : cus, Cfg::THREADS, LDS, st>>>(g, epi);
+        if (int e = check_launch("lm_head CE backward (dlogits)")) return e;
+        // 2. exact gradient at the target columns
+        ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, dl, dl_t);
+        if (int e = check_launch("ce_dl_fix_kernel")) return e;
+        // 3. dx[chunk] = dl [Mc, V] . (w^T [K, V])^T
+        if (int e = gemm_store(dl, FMT_E5M2, V, w_t, FMT_E4M3, V, Mc, K, V, grad_s * w_s,
+                               (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, 0, st)) return e;
+        // 4. dw += over the chunk's tokens
+        const int kind = m0 == 0 ? 1 : 2;
+        if (w_layout == NGPT_W_OUT_IN) {   // dw [V, K] = dl^T [V, Mc] . (x^T [K, Mc])^T
+            if (int e = gemm_store(dl_t, FMT_E5M2, Mc, x_t + m0, FMT_E4M3, M, V, K, Mc, x_s * grad_s,
+                                   dw_f32, K, kind, st)) return e;
+        } else {                           // dw [K, V] = x^T [K, Mc] . (dl^T [V, Mc])^T
+            if (int e = gemm_store(x_t + m0, FMT_E4M3, M, dl_t, FMT_E5M2, Mc, K, V, Mc, x_s * grad_s,
+                                   dw_f32, V, kind, st)) return e;
+        }
+    }
+    return NGPT_OK;
+}

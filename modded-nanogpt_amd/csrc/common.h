@@ -1,0 +1,109 @@
+// Device-side helpers shared by every kernel of the FP8 contraction path (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ngpt {
+
+typedef int   v2i  __attribute__((ext_vector_type(2)));
+typedef int   v4i  __attribute__((ext_vector_type(4)));
+typedef int   v8i  __attribute__((ext_vector_type(8)));
+typedef float v4f  __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+enum : int { FMT_E4M3 = 0, FMT_E5M2 = 1 };
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------- bf16 <-> f32
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// round-to-nearest-even; NaN stays NaN
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint32_t r = u + 0x7fffu + ((u >> 16) & 1u);
+    r = (f != f) ? (u | 0x00400000u) : r;
+    return r >> 16;
+}
+
+__device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// ---------------------------------------------------------------- f32 -> fp8 (OCP)
+// The hardware converter (v_cvt_pk_fp8_f32 / v_cvt_pk_bf8_f32) rounds to nearest even and keeps
+// subnormals.  What it does above the largest finite value depends on a mode bit, so overflow
+// and NaN are decided here and only in-range magnitudes reach the converter.
+
+// torch.float8_e4m3fn cast: |v| > 464 (the tie at 464 rounds down to 448) -> NaN code, no saturation.
+__device__ __forceinline__ uint32_t f32_to_e4m3_torch(float v) {
+    float a = fabsf(v);
+    uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
+    bool bad = !(a <= 464.0f);                       // overflow, inf or NaN
+    float c = bad ? 0.0f : v;
+    uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xffu;
+    return bad ? (sign | 0x7fu) : code;
+}
+
+// torch.float8_e5m2 cast: |v| >= 61440 -> +-inf (the tie rounds to the even code, which is inf).
+__device__ __forceinline__ uint32_t f32_to_e5m2_torch(float v) {
+    float a = fabsf(v);
+    uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
+    bool isnan_ = (v != v);
+    bool ovf = (a >= 61440.0f);
+    float c = (isnan_ || ovf) ? 0.0f : v;
+    uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(c, c, 0, false) & 0xffu;
+    code = ovf ? (sign | 0x7cu) : code;
+    return isnan_ ? (sign | 0x7fu) : code;
+}
+
+// Saturating e5m2 of two values (the cross-entropy gradient store): finite values clamp to +-57344.
+__device__ __forceinline__ uint32_t f32x2_to_e5m2_sat(float a, float b) {
+    a = __builtin_fminf(__builtin_fmaxf(a, -57344.0f), 57344.0f);
+    b = __builtin_fminf(__builtin_fmaxf(b, -57344.0f), 57344.0f);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false) & 0xffffu;
+}
+
+__device__ __forceinline__ uint32_t f32x4_to_e5m2_sat(float a, float b, float c, float d) {
+    a = __builtin_fminf(__builtin_fmaxf(a, -57344.0f), 57344.0f);
+    b = __builtin_fminf(__builtin_fmaxf(b, -57344.0f), 57344.0f);
+    c = __builtin_fminf(__builtin_fmaxf(c, -57344.0f), 57344.0f);
+    d = __builtin_fminf(__builtin_fmaxf(d, -57344.0f), 57344.0f);
+    int r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+    r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
+    return (uint32_t)r;
+}
+
+// Saturating e4m3 of one value, input already clamped to <= 448 by the caller or here.
+__device__ __forceinline__ uint32_t f32_to_e4m3_sat(float v) {
+    v = __builtin_fminf(__builtin_fmaxf(v, -448.0f), 448.0f);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v, v, 0, false) & 0xffu;
+}
+
+// ---------------------------------------------------------------- wave helpers
+__device__ __forceinline__ int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// 16-byte global -> LDS copy that bypasses registers.  `lds_wave_base` must be the same for all
+// lanes of the wave; lane l's 16 bytes land at lds_wave_base + 16*l.
+__device__ __forceinline__ void global_to_lds16(const void* gptr, void* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void*)gptr,
+        (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+__device__ __forceinline__ void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+}  // namespace ngpt

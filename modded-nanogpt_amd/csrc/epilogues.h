@@ -1,0 +1,196 @@
+// Epilogues for gemm_tn_kernel: what happens to a finished BM x BN fp32 accumulator tile.
+#pragma once
+#include "gemm_tn.h"
+
+namespace ngpt {
+
+// ---------------------------------------------------------------------------------------------
+// Staged byte stores.  An fp8 result tile cannot be written straight from the MFMA register
+// layout (a lane owns one column and scattered rows: 1-byte or 4-byte pieces per row), so the
+// wave parks a strip in its private LDS scratch and writes it back out in 16-byte pieces.
+
+// Strip = 32 rows x WTN columns of bytes, stored row-major in global memory (leading dim ld).
+// `codes[tn][v]` holds the byte for accumulator element (tn, v) of one tm.
+template <class Cfg>
+__device__ __forceinline__ void store_strip_rowmajor_u8(
+    const uint32_t (&codes)[Cfg::TN][16], uint8_t* scratch, int lane,
+    uint8_t* out, int64_t ld, int grow0 /* global row of strip row 0 */, int gcol0, int R, int C) {
+    constexpr int STRIDE = Cfg::WTN + 16;
+    const int h = lane >> 5, j = lane & 31;
+#pragma unroll
+    for (int tn = 0; tn < Cfg::TN; ++tn)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            int rl = 8 * (v >> 2) + 4 * h + (v & 3);
+            scratch[rl * STRIDE + tn * 32 + j] = (uint8_t)codes[tn][v];
+        }
+    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the wave's own LDS writes have landed
+    constexpr int CH_PER_ROW = Cfg::WTN / 16;
+#pragma unroll
+    for (int p = 0; p < Cfg::WTN / 32; ++p) {
+        int id = p * 64 + lane;
+        int rl = id / CH_PER_ROW, ch = id % CH_PER_ROW;
+        v4i val = *(const v4i*)(scratch + rl * STRIDE + ch * 16);
+        int gr = grow0 + rl, gc = gcol0 + ch * 16;
+        if (gr < R && gc + 16 <= C) *(v4i*)(out + (int64_t)gr * ld + gc) = val;
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+}
+
+// Strip = 32 columns x WTM rows, stored transposed: out[col][row], leading dim ld.
+// `packed[tm][g]` holds four consecutive rows (8g + 4h .. +3 of tm) as one little-endian word.
+template <class Cfg>
+__device__ __forceinline__ void store_strip_transposed_u8(
+    const uint32_t (&packed)[Cfg::TM][4], uint8_t* scratch, int lane,
+    uint8_t* out, int64_t ld, int grow0, int gcol0 /* global col of strip col 0 */, int R, int C) {
+    constexpr int STRIDE = Cfg::WTM + 16;
+    const int h = lane >> 5, j = lane & 31;
+#pragma unroll
+    for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            *(uint32_t*)(scratch + j * STRIDE + tm * 32 + 8 * g + 4 * h) = packed[tm][g];
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    constexpr int CH_PER_ROW = Cfg::WTM / 16;
+    constexpr int PASSES = (32 * CH_PER_ROW + 63) / 64;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+        int id = p * 64 + lane;
+        int cl = id / CH_PER_ROW, ch = id % CH_PER_ROW;
+        if (cl < 32) {
+            v4i val = *(const v4i*)(scratch + cl * STRIDE + ch * 16);
+            int gc = gcol0 + cl, gr = grow0 + ch * 16;
+            if (gc < C && gr + 16 <= R) *(v4i*)(out + (int64_t)gc * ld + gr) = val;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[r, c] = bf16(acc * scale)
+struct EpiStoreBf16 {
+    uint16_t* out;
+    int64_t ld;
+    float scale;
+    int R, C;
+    static constexpr int EXTRA_LDS = 0;
+    __device__ void begin(int, int, uint8_t*) {}
+    __device__ void end(uint8_t*, int, int) {}
+    template <class Cfg>
+    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
+                         uint8_t*, int) {
+#pragma unroll
+        for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < Cfg::TN; ++tn) {
+                int c = c0 + co.col(tn);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int r = r0 + co.row(tm, v);
+                    if (r < R && c < C) out[(int64_t)r * ld + c] = (uint16_t)f32_to_bf16_bits(acc[tm][tn][v] * scale);
+                }
+            }
+    }
+};
+
+// out[r, c] (+)= acc * scale in fp32
+struct EpiStoreF32 {
+    float* out;
+    int64_t ld;
+    float scale;
+    int R, C;
+    int accumulate;
+    static constexpr int EXTRA_LDS = 0;
+    __device__ void begin(int, int, uint8_t*) {}
+    __device__ void end(uint8_t*, int, int) {}
+    template <class Cfg>
+    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
+                         uint8_t*, int) {
+#pragma unroll
+        for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < Cfg::TN; ++tn) {
+                int c = c0 + co.col(tn);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int r = r0 + co.row(tm, v);
+                    if (r < R && c < C) {
+                        float* p = out + (int64_t)r * ld + c;
+                        float val = acc[tm][tn][v] * scale;
+                        *p = accumulate ? (*p + val) : val;
+                    }
+                }
+            }
+    }
+};
+
+// post = bf16(max(bf16(acc * *dequant), 0)^2); optionally post_f8 = e4m3(min(post / act_scale, 448))
+// and a per-workgroup running max of post written to partial_amax[bid].
+struct EpiRelu2 {
+    uint16_t* post;
+    int64_t ld;
+    const float* dequant;        // 1-element device tensor
+    uint8_t* post_f8;            // nullable
+    int64_t ld_f8;
+    const float* act_scale;      // 1-element device tensor, required with post_f8
+    float* partial_amax;         // nullable; n_partials entries
+    int n_partials;
+    int R, C;
+    float scale, inv_act, amax;
+    static constexpr int EXTRA_LDS = 0;
+    template <class Cfg>
+    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+    __device__ void begin(int, int, uint8_t*) {
+        scale = *dequant;
+        inv_act = post_f8 ? 1.0f / *act_scale : 0.0f;
+        amax = 0.0f;
+    }
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
+                         uint8_t* scratch, int lane) {
+#pragma unroll
+        for (int tm = 0; tm < Cfg::TM; ++tm) {
+            uint32_t codes[Cfg::TN][16];
+#pragma unroll
+            for (int tn = 0; tn < Cfg::TN; ++tn) {
+                int c = c0 + co.col(tn);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int r = r0 + co.row(tm, v);
+                    float pre = round_to_bf16(acc[tm][tn][v] * scale);
+                    pre = fmaxf(pre, 0.0f);
+                    float p = round_to_bf16(pre * pre);
+                    bool ok = (r < R && c < C);
+                    if (ok) post[(int64_t)r * ld + c] = (uint16_t)(__float_as_uint(p) >> 16);
+                    if (post_f8) {
+                        codes[tn][v] = f32_to_e4m3_sat(fminf(p * inv_act, 448.0f));
+                        amax = ok ? fmaxf(amax, p) : amax;
+                    }
+                }
+            }
+            if (post_f8)
+                store_strip_rowmajor_u8<Cfg>(codes, scratch, lane, post_f8, ld_f8,
+                                             r0 + co.wave_row0 + tm * 32, c0 + co.wave_col0, R, C);
+        }
+    }
+    __device__ void end(uint8_t* smem, int bid, int G) {
+        if (!partial_amax) return;
+        float m = wave_max(amax);
+        float* red = (float*)smem;
+        int wave = threadIdx.x >> 6;
+        if ((threadIdx.x & 63) == 0) red[wave] = m;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float t = 0.0f;
+            for (int w = 0; w < (int)(blockDim.x >> 6); ++w) t = fmaxf(t, red[w]);
+            partial_amax[bid] = t;
+            for (int i = bid + G; i < n_partials; i += G) partial_amax[i] = 0.0f;
+        }
+    }
+};
+
+}  // namespace ngpt

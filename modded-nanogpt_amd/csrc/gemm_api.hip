@@ -1,0 +1,160 @@
+// C-ABI entry points built on the persistent FP8 TN GEMM: the raw GEMM, nanogpt::mm(_t)
+// forward/backward and the fused up-projection + ReLU^2.
+#include "epilogues.h"
+#include "host_util.h"
+#include "launch.h"
+
+namespace ngpt {
+
+static char g_err[512];
+char* last_error_buf() {
+    static thread_local char buf[512];
+    (void)g_err;
+    return buf;
+}
+
+int num_cus() {
+    static int cached = -1;
+    if (cached < 0) {
+        int dev = 0;
+        hipDeviceProp_t p;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        cached = p.multiProcessorCount;
+    }
+    return cached;
+}
+
+static int check_gemm_dims(const char* who, int R, int C, int K, int64_t lda, int64_t ldb) {
+    if (R <= 0 || C <= 0 || K <= 0) return fail(NGPT_EINVAL, "%s: empty problem R=%d C=%d K=%d", who, R, C, K);
+    if (K % 128) return fail(NGPT_EALIGN, "%s: contraction length %d must be a multiple of 128", who, K);
+    if (lda % 16 || ldb % 16 || lda < K || ldb < K)
+        return fail(NGPT_EALIGN, "%s: operand row strides (%lld, %lld) must be multiples of 16 and >= K",
+                    who, (long long)lda, (long long)ldb);
+    return NGPT_OK;
+}
+
+int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
+               float scale, void* out, int64_t ldc, int out_kind, hipStream_t st) {
+    if (int e = check_gemm_dims("gemm_fp8_tn", R, C, K, lda, ldb)) return e;
+    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K};
+    if (out_kind == 0) {
+        EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C};
+        return launch_gemm<MainCfg>(g, fa, fb, epi, st);
+    }
+    EpiStoreF32 epi{(float*)out, ldc, scale, R, C, out_kind == 2};
+    return launch_gemm<MainCfg>(g, fa, fb, epi, st);
+}
+
+}  // namespace ngpt
+
+using namespace ngpt;
+
+extern "C" int ngpt_abi_version(void) { return 1; }
+extern "C" const char* ngpt_last_error(void) { return last_error_buf(); }
+extern "C" int ngpt_num_cus(void) { return num_cus(); }
+
+extern "C" int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const void* B, int fmt_b, int64_t ldb,
+                                int R, int C, int K, float scale, void* out, int64_t ldc, int out_kind,
+                                void* stream) {
+    if (!A || !B || !out) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: null pointer");
+    if ((fmt_a | fmt_b) & ~1) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: fmt_a=%d fmt_b=%d", fmt_a, fmt_b);
+    if (out_kind < 0 || out_kind > 2) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: out_kind=%d", out_kind);
+    if (ldc < C) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: ldc=%lld < C=%d", (long long)ldc, C);
+    return gemm_store(A, fmt_a, lda, B, fmt_b, ldb, R, C, K, scale, out, ldc, out_kind, (hipStream_t)stream);
+}
+
+// ------------------------------------------------------------------------------------------ mm forward
+extern "C" int64_t ngpt_mm_fwd_workspace_bytes(int M, int N, int K, int w_layout) {
+    (void)M;
+    return w_layout == NGPT_W_IN_OUT ? align_up((int64_t)N * K, 256) : 0;
+}
+
+extern "C" int ngpt_mm_fwd(const void* x_bf16, const void* w_bf16, int M, int N, int K, float x_s, float w_s,
+                           void* out_bf16, void* x_f8, void* w_f8, int w_layout,
+                           void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!x_bf16 || !w_bf16 || !out_bf16 || !x_f8 || !w_f8) return fail(NGPT_EINVAL, "ngpt_mm_fwd: null pointer");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(NGPT_EINVAL, "ngpt_mm_fwd: empty problem M=%d N=%d K=%d", M, N, K);
+    if (K % 128 || M % 16 || N % 16)
+        return fail(NGPT_EALIGN, "ngpt_mm_fwd: need K %% 128 == 0, M %% 16 == 0, N %% 16 == 0 (M=%d N=%d K=%d)", M, N, K);
+    if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "ngpt_mm_fwd: w_layout=%d", w_layout);
+    int64_t need = ngpt_mm_fwd_workspace_bytes(M, N, K, w_layout);
+    if (need > 0 && (!workspace || workspace_bytes < need))
+        return fail(NGPT_EWORKSPACE, "ngpt_mm_fwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
+    hipStream_t st = (hipStream_t)stream;
+    if (int e = ngpt_quant_fp8(x_bf16, x_f8, (int64_t)M * K, x_s, NGPT_FMT_E4M3, stream)) return e;
+    const void* w_nk = w_f8;
+    if (w_layout == NGPT_W_OUT_IN) {
+        if (int e = ngpt_quant_fp8(w_bf16, w_f8, (int64_t)N * K, w_s, NGPT_FMT_E4M3, stream)) return e;
+    } else {
+        // w is [K, N]: one pass writes w_f8 [K, N] and the [N, K] copy the GEMM reads
+        if (int e = ngpt_quant_fp8_2d(w_bf16, K, N, w_s, NGPT_FMT_E4M3, w_f8, workspace, stream)) return e;
+        w_nk = workspace;
+    }
+    return gemm_store(x_f8, FMT_E4M3, K, w_nk, FMT_E4M3, K, M, N, K, x_s * w_s, out_bf16, N, 0, st);
+}
+
+// ------------------------------------------------------------------------------------------ mm backward
+// workspace: g_f8 [M,N] | g_f8^T [N,M] | x_f8^T [K,M] | (OUT_IN only) w_f8^T [K,N]
+extern "C" int64_t ngpt_mm_bwd_workspace_bytes(int M, int N, int K, int w_layout) {
+    int64_t b = 2 * align_up((int64_t)M * N, 256) + align_up((int64_t)K * M, 256);
+    if (w_layout == NGPT_W_OUT_IN) b += align_up((int64_t)K * N, 256);
+    return b;
+}
+
+extern "C" int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f8, int M, int N, int K,
+                           float x_s, float w_s, float grad_s, void* dx_bf16, void* dw_kn_f32, int w_layout,
+                           void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!g_bf16 || !x_f8 || !w_f8 || !dx_bf16 || !dw_kn_f32 || !workspace) return fail(NGPT_EINVAL, "ngpt_mm_bwd: null pointer");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(NGPT_EINVAL, "ngpt_mm_bwd: empty problem M=%d N=%d K=%d", M, N, K);
+    if (M % 128 || N % 128 || K % 16)
+        return fail(NGPT_EALIGN, "ngpt_mm_bwd: need M %% 128 == 0, N %% 128 == 0, K %% 16 == 0 (M=%d N=%d K=%d)", M, N, K);
+    if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "ngpt_mm_bwd: w_layout=%d", w_layout);
+    int64_t need = ngpt_mm_bwd_workspace_bytes(M, N, K, w_layout);
+    if (workspace_bytes < need)
+        return fail(NGPT_EWORKSPACE, "ngpt_mm_bwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
+    hipStream_t st = (hipStream_t)stream;
+    uint8_t* ws = (uint8_t*)workspace;
+    uint8_t* g_f8 = ws;
+    uint8_t* g_f8_t = g_f8 + align_up((int64_t)M * N, 256);
+    uint8_t* x_f8_t = g_f8_t + align_up((int64_t)M * N, 256);
+    uint8_t* w_f8_t = x_f8_t + align_up((int64_t)K * M, 256);
+    if (int e = ngpt_quant_fp8_2d(g_bf16, M, N, grad_s, NGPT_FMT_E5M2, g_f8, g_f8_t, stream)) return e;
+    if (int e = ngpt_transpose_u8(x_f8, M, K, x_f8_t, stream)) return e;
+    const void* w_kn = w_f8;
+    if (w_layout == NGPT_W_OUT_IN) {
+        if (int e = ngpt_transpose_u8(w_f8, N, K, w_f8_t, stream)) return e;
+        w_kn = w_f8_t;
+    }
+    // dx [M,K] = g_f8 [M,N] . (w [K,N])^T, contraction over N
+    if (int e = gemm_store(g_f8, FMT_E5M2, N, w_kn, FMT_E4M3, N, M, K, N, grad_s * w_s, dx_bf16, K, 0, st)) return e;
+    // dw [K,N] = x_f8^T [K,M] . (g_f8^T [N,M])^T, contraction over M
+    return gemm_store(x_f8_t, FMT_E4M3, M, g_f8_t, FMT_E5M2, M, K, N, M, x_s * grad_s, dw_kn_f32, N, 1, st);
+}
+
+// ------------------------------------------------------------------------------------------ fc + relu^2
+extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, int M, int N, int K,
+                                 void* post_bf16, void* post_f8, const float* act_scale,
+                                 float* partial_amax, int n_partials, void* stream) {
+    if (!x_f8 || !w_f8 || !dequant || !post_bf16) return fail(NGPT_EINVAL, "ngpt_fc_relu2_fwd: null pointer");
+    if (post_f8 && (!act_scale || !partial_amax || n_partials <= 0))
+        return fail(NGPT_EINVAL, "ngpt_fc_relu2_fwd: post_f8 needs act_scale and partial_amax");
+    if (int e = check_gemm_dims("ngpt_fc_relu2_fwd", M, N, K, K, K)) return e;
+    if (N % 16) return fail(NGPT_EALIGN, "ngpt_fc_relu2_fwd: N=%d must be a multiple of 16", N);
+    GemmOperands g{(const uint8_t*)x_f8, (const uint8_t*)w_f8, K, K, M, N, K};
+    EpiRelu2 epi{};
+    epi.post = (uint16_t*)post_bf16;
+    epi.ld = N;
+    epi.dequant = dequant;
+    epi.post_f8 = (uint8_t*)post_f8;
+    epi.ld_f8 = N;
+    epi.act_scale = act_scale;
+    epi.partial_amax = post_f8 ? partial_amax : nullptr;
+    epi.n_partials = n_partials;
+    epi.R = M;
+    epi.C = N;
+    int max_grid = post_f8 ? n_partials : 0;   // one partial-amax slot per persistent workgroup
+    return launch_gemm<MainCfg>(g, FMT_E4M3, FMT_E4M3, epi, (hipStream_t)stream, max_grid);
+}

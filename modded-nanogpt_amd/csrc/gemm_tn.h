@@ -1,0 +1,264 @@
+// Persistent FP8 "TN" GEMM core for gfx950:  C[r, c] = sum_k A[r, k] * B[c, k]
+//
+// Both operands are fp8 bytes with the contraction index contiguous.  One workgroup owns a
+// BM x BN tile at a time and walks a list of tiles; the k-loop of consecutive tiles is one
+// continuous software pipeline, so the first operand slab of the next tile is already in flight
+// while the current tile's epilogue runs.
+//
+// Data path per k-step (BK = 128 bytes of contraction):
+//   HBM/L2 --global_load_lds_dwordx4--> LDS (two stages, no register staging)
+//   LDS --ds_read_b128--> MFMA operand registers --v_mfma_f32_32x32x64_f8f6f4--> fp32 accumulators
+//
+// LDS layout of an operand slab: rows of 128 bytes; the eight 16-byte chunks of row r are stored
+// at chunk position q ^ ((r >> 1) & 7).  A direct-to-LDS load writes 1 KiB (8 rows) per wave
+// instruction with lane l at byte 16*l, so the swizzle is applied on the global-address side.
+// With it, the 16 lanes that a ds_read_b128 serves together (16 consecutive rows, same chunk) hit
+// 16 distinct 16-byte bank groups.
+//
+// MFMA 32x32x64 f8f6f4 register layouts used here (lane l, h = l / 32):
+//   A operand: row  i = l % 32, 32 contraction bytes  [64*ks + 32*h, +32)
+//   B operand: col  j = l % 32, the same 32 contraction bytes
+//   D (16 fp32): col j = l % 32, row i = 8*(v/4) + 4*h + (v%4) for register v
+// Any permutation of the contraction bytes is harmless as long as A and B use the same one.
+#pragma once
+#include "common.h"
+
+namespace ngpt {
+
+struct GemmOperands {
+    const uint8_t* A;   // [R, K] fp8, row stride lda bytes
+    const uint8_t* B;   // [C, K] fp8, row stride ldb bytes
+    int64_t lda, ldb;
+    int R, C, K;        // K % 128 == 0
+};
+
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_>
+struct TileCfg {
+    static constexpr int BM = BM_, BN = BN_, BK = 128;
+    static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int NWAVES = WAVES_M * WAVES_N;
+    static constexpr int THREADS = NWAVES * 64;
+    static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;   // wave tile
+    static constexpr int TM = WTM / 32, TN = WTN / 32;             // MFMA tiles per wave
+    static constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int SMEM_BYTES = 2 * STAGE_BYTES;
+    static constexpr int A_LOADS = BM / 8 / NWAVES;                // wave-level 1 KiB loads per k-step
+    static constexpr int B_LOADS = BN / 8 / NWAVES;
+    static constexpr int WAVE_SCRATCH = STAGE_BYTES / NWAVES;      // epilogue staging per wave
+    static_assert(BM % (8 * NWAVES) == 0 && BN % (8 * NWAVES) == 0, "tile rows must split over waves");
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be made of 32x32 MFMA tiles");
+};
+
+// Tile order: groups of 4 tile-rows, column-major inside a group, so 32 consecutive sequence
+// numbers form a 4 x 8 block of tiles that shares 4 A panels and 8 B panels.  Workgroups are
+// dealt to the 8 XCDs round-robin by the dispatcher (workgroup b runs on XCD b % 8); giving
+// XCD x the sequence numbers [32x, 32x+32) of every batch of 256 keeps such a block inside one
+// XCD's L2.
+struct TileOrder {
+    int tiles_r, tiles_c, total;
+    __device__ TileOrder(int R, int C, int BM, int BN)
+        : tiles_r((R + BM - 1) / BM), tiles_c((C + BN - 1) / BN), total(tiles_r * tiles_c) {}
+    __device__ void coords(int seq, int& tr, int& tc) const {
+        constexpr int GROUP = 4;
+        int per_group = GROUP * tiles_c;
+        int grp = seq / per_group;
+        int first = grp * GROUP;
+        int gsz = min(tiles_r - first, GROUP);
+        int rem = seq - grp * per_group;
+        tr = first + rem % gsz;
+        tc = rem / gsz;
+    }
+    // sequence number handled by workgroup `bid` of `G` in its `it`-th turn
+    static __device__ int seq_of(int it, int bid, int G) {
+        if ((G & 7) == 0) return it * G + (bid & 7) * (G >> 3) + (bid >> 3);
+        return it * G + bid;
+    }
+};
+
+template <class Cfg, int AFMT, int BFMT>
+struct TileMainloop {
+    const uint8_t* a_ptr[Cfg::A_LOADS];
+    const uint8_t* b_ptr[Cfg::B_LOADS];
+    int frag_a[Cfg::TM];     // LDS byte offset of this lane's first 16-byte chunk, stage 0, ks 0
+    int frag_b[Cfg::TN];
+    int wave, lane, wr, wc;
+
+    __device__ void init() {
+        int tid = threadIdx.x;
+        lane = tid & 63;
+        wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        wr = wave / Cfg::WAVES_N;
+        wc = wave % Cfg::WAVES_N;
+        int h = lane >> 5;
+#pragma unroll
+        for (int t = 0; t < Cfg::TM; ++t) {
+            int row = wr * Cfg::WTM + t * 32 + (lane & 31);
+            frag_a[t] = row * 128 + ((((h * 2) ^ (row >> 1)) & 7) << 4);
+        }
+#pragma unroll
+        for (int t = 0; t < Cfg::TN; ++t) {
+            int row = wc * Cfg::WTN + t * 32 + (lane & 31);
+            frag_b[t] = Cfg::A_BYTES + row * 128 + ((((h * 2) ^ (row >> 1)) & 7) << 4);
+        }
+    }
+
+    // Point the per-lane global pointers at tile (r0, c0).  Rows past the end are clamped to the
+    // last row: they are loaded (valid memory) and their results discarded by the epilogue.
+    __device__ void set_tile(const GemmOperands& g, int r0, int c0) {
+        int lrow = lane >> 3, lchunk = lane & 7;
+#pragma unroll
+        for (int i = 0; i < Cfg::A_LOADS; ++i) {
+            int R = (wave + i * Cfg::NWAVES) * 8 + lrow;
+            int q = lchunk ^ ((R >> 1) & 7);
+            int gr = min(r0 + R, g.R - 1);
+            a_ptr[i] = g.A + (int64_t)gr * g.lda + q * 16;
+        }
+#pragma unroll
+        for (int i = 0; i < Cfg::B_LOADS; ++i) {
+            int R = (wave + i * Cfg::NWAVES) * 8 + lrow;
+            int q = lchunk ^ ((R >> 1) & 7);
+            int gc = min(c0 + R, g.C - 1);
+            b_ptr[i] = g.B + (int64_t)gc * g.ldb + q * 16;
+        }
+    }
+
+    __device__ void issue_loads(uint8_t* smem, int stage, int kt) {
+        uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
+        int koff = kt * Cfg::BK;
+#pragma unroll
+        for (int i = 0; i < Cfg::A_LOADS; ++i)
+            global_to_lds16(a_ptr[i] + koff, s + (wave + i * Cfg::NWAVES) * 1024);
+#pragma unroll
+        for (int i = 0; i < Cfg::B_LOADS; ++i)
+            global_to_lds16(b_ptr[i] + koff, s + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
+    }
+
+    __device__ void compute(const uint8_t* smem, int stage, v16f (&acc)[Cfg::TM][Cfg::TN]) {
+        const uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            v8i a[Cfg::TM], b[Cfg::TN];
+#pragma unroll
+            for (int t = 0; t < Cfg::TM; ++t) {
+                int o = frag_a[t] ^ (ks * 64);
+                v4i lo = *(const v4i*)(s + o);
+                v4i hi = *(const v4i*)(s + (o ^ 16));
+                a[t] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            }
+#pragma unroll
+            for (int t = 0; t < Cfg::TN; ++t) {
+                int o = frag_b[t] ^ (ks * 64);
+                v4i lo = *(const v4i*)(s + o);
+                v4i hi = *(const v4i*)(s + (o ^ 16));
+                b[t] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            }
+#pragma unroll
+            for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < Cfg::TN; ++tn)
+                    acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                        a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
+        }
+    }
+};
+
+// Coordinates of accumulator element (tm, tn, v) of this lane inside the workgroup tile.
+template <class Cfg>
+struct AccCoords {
+    int wave_row0, wave_col0;   // origin of this wave's sub-tile
+    int row_base, col_base;     // this lane's element for tm = tn = 0, v = 0
+    __device__ AccCoords(int wr, int wc, int lane)
+        : wave_row0(wr * Cfg::WTM), wave_col0(wc * Cfg::WTN),
+          row_base(wr * Cfg::WTM + 4 * (lane >> 5)), col_base(wc * Cfg::WTN + (lane & 31)) {}
+    __device__ int row(int tm, int v) const { return row_base + tm * 32 + 8 * (v >> 2) + (v & 3); }
+    __device__ int col(int tn) const { return col_base + tn * 32; }
+};
+
+// Default tile walk: every tile of the R x C grid once, in TileOrder.
+struct GridIter {
+    TileOrder order;
+    int it, bid, G, seq, tr_, tc_;
+    __device__ GridIter(const GemmOperands& g, int BM, int BN, int bid_, int G_)
+        : order(g.R, g.C, BM, BN), it(0), bid(bid_), G(G_), tr_(0), tc_(0) {
+        seq = TileOrder::seq_of(0, bid, G);
+        if (valid()) order.coords(seq, tr_, tc_);
+    }
+    __device__ bool valid() const { return seq < order.total; }
+    __device__ int tr() const { return tr_; }
+    __device__ int tc() const { return tc_; }
+    __device__ bool job_end() const { return false; }
+    __device__ int job_id() const { return 0; }
+    __device__ void advance() {
+        ++it;
+        seq = TileOrder::seq_of(it, bid, G);
+        if (valid()) order.coords(seq, tr_, tc_);
+    }
+};
+
+// The generic persistent kernel.  `Iter` walks the tiles of this workgroup (see GridIter).  `Epi` supplies
+//   void begin(int bid, int nblocks)
+//   void tile(acc, r0, c0, coords, scratch /* wave-private LDS */, lane)
+//   void job_end(c0, job_id, coords, stage_scratch /* whole free LDS stage */)   -- only if Iter reports job ends
+//   void end(uint8_t* smem, int bid, int nblocks)
+// `tile` runs after a workgroup barrier, so the just-consumed LDS stage is free for staging.
+// Dynamic LDS: Cfg::SMEM_BYTES for the two operand stages, then Epi::EXTRA_LDS bytes that the
+// epilogue owns for the whole kernel (lookup tables).
+template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
+__global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel(GemmOperands g, Epi epi) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    TileMainloop<Cfg, AFMT, BFMT> ml;
+    ml.init();
+    const int bid = blockIdx.x, G = gridDim.x;
+    const int nk = g.K / Cfg::BK;
+    AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane);
+    Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
+    if (cur.valid()) {
+        ml.set_tile(g, cur.tr() * Cfg::BM, cur.tc() * Cfg::BN);
+        ml.issue_loads(smem, 0, 0);
+    }
+    epi.begin(bid, G, smem + Cfg::SMEM_BYTES);
+
+    v16f acc[Cfg::TM][Cfg::TN];
+#pragma unroll
+    for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    int stage = 0;
+    while (cur.valid()) {
+        const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
+        Iter nxt = cur;
+        nxt.advance();
+        for (int kt = 0; kt < nk; ++kt) {
+            wait_vmem_all();
+            __syncthreads();
+            // prefetch the next k-step (possibly the first one of the next tile)
+            if (kt + 1 < nk) {
+                ml.issue_loads(smem, stage ^ 1, kt + 1);
+            } else if (nxt.valid()) {
+                ml.set_tile(g, nxt.tr() * Cfg::BM, nxt.tc() * Cfg::BN);
+                ml.issue_loads(smem, stage ^ 1, 0);
+            }
+            ml.compute(smem, stage, acc);
+            stage ^= 1;
+        }
+        __syncthreads();   // every wave is done reading the last stage: reuse it as scratch
+        uint8_t* free_stage = smem + (stage ^ 1) * Cfg::STAGE_BYTES;
+        epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
+        if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
+#pragma unroll
+        for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+            for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        cur = nxt;
+    }
+    __syncthreads();
+    epi.end(smem, bid, G);
+}
+
+}  // namespace ngpt

@@ -1,0 +1,37 @@
+// Host-side launcher of gemm_tn_kernel: picks the fp8 format instantiation and the grid.
+#pragma once
+#include "gemm_tn.h"
+#include "host_util.h"
+
+namespace ngpt {
+
+// 256 x 256 tile, 8 waves as 4 (rows) x 2 (cols): each wave owns 64 x 128 = 2 x 4 MFMA tiles.
+using MainCfg = TileCfg<256, 256, 4, 2>;
+
+template <class Cfg, int FA, int FB, class Epi>
+int launch_gemm_fmt(const GemmOperands& g, const Epi& epi, hipStream_t st, int max_grid) {
+    auto kernel = gemm_tn_kernel<Cfg, FA, FB, Epi, GridIter>;
+    constexpr int LDS = Cfg::SMEM_BYTES + Epi::EXTRA_LDS;
+    static bool configured = false;
+    if (!configured) {
+        if (int e = allow_lds(kernel, LDS)) return e;
+        configured = true;
+    }
+    int tiles = ((g.R + Cfg::BM - 1) / Cfg::BM) * ((g.C + Cfg::BN - 1) / Cfg::BN);
+    int cus = num_cus();
+    if (cus <= 0) return fail(NGPT_EINVAL, "no HIP device");
+    int grid = tiles < cus ? tiles : cus;
+    if (max_grid > 0 && grid > max_grid) grid = max_grid;
+    kernel<<<grid, Cfg::THREADS, LDS, st>>>(g, epi);
+    return check_launch("gemm_tn_kernel");
+}
+
+template <class Cfg, class Epi>
+int launch_gemm(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {
+    if (fa == FMT_E4M3 && fb == FMT_E4M3) return launch_gemm_fmt<Cfg, FMT_E4M3, FMT_E4M3>(g, epi, st, max_grid);
+    if (fa == FMT_E5M2 && fb == FMT_E4M3) return launch_gemm_fmt<Cfg, FMT_E5M2, FMT_E4M3>(g, epi, st, max_grid);
+    if (fa == FMT_E4M3 && fb == FMT_E5M2) return launch_gemm_fmt<Cfg, FMT_E4M3, FMT_E5M2>(g, epi, st, max_grid);
+    return launch_gemm_fmt<Cfg, FMT_E5M2, FMT_E5M2>(g, epi, st, max_grid);
+}
+
+}  // namespace ngpt

@@ -1,0 +1,128 @@
+// bf16 -> fp8 quantisers and byte transposes (HBM-bound, one pass over the input).
+#include "common.h"
+#include "host_util.h"
+
+namespace ngpt {
+
+// fp8(bf16_rne(fp32(x) / s)): the division is IEEE fp32 and is rounded to bf16 before the cast.
+template <int FMT>
+__device__ __forceinline__ uint32_t quant_one(uint32_t bf16_bits, float s) {
+    float q = round_to_bf16(__fdiv_rn(bf16_bits_to_f32(bf16_bits), s));
+    return FMT == FMT_E4M3 ? f32_to_e4m3_torch(q) : f32_to_e5m2_torch(q);
+}
+
+template <int FMT>
+__device__ __forceinline__ v2i quant8(v4i in, float s) {
+    uint32_t w[4] = {(uint32_t)in.x, (uint32_t)in.y, (uint32_t)in.z, (uint32_t)in.w};
+    uint32_t c[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        c[2 * i] = quant_one<FMT>(w[i] & 0xffffu, s);
+        c[2 * i + 1] = quant_one<FMT>(w[i] >> 16, s);
+    }
+    v2i o;
+    o.x = (int)(c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24));
+    o.y = (int)(c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24));
+    return o;
+}
+
+template <int FMT>
+__global__ __launch_bounds__(256) void quant_kernel(const v4i* __restrict__ in, v2i* __restrict__ out,
+                                                    int64_t n8, float s) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * 256;
+    for (; i < n8; i += stride) out[i] = quant8<FMT>(in[i], s);
+}
+
+// 64 x 64 tile: quantise, write the row-major bytes, and write the transposed bytes via LDS.
+// IN_BYTES = 2: bf16 input quantised with scale s.  IN_BYTES = 1: plain byte transpose.
+template <int FMT, int IN_BYTES>
+__global__ __launch_bounds__(256) void tile_transpose_kernel(const uint8_t* __restrict__ in, int rows, int cols,
+                                                             float s, uint8_t* __restrict__ out,
+                                                             uint8_t* __restrict__ out_t) {
+    __shared__ uint8_t tile[64][64 + 4];   // [col][row]
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int t = threadIdx.x;
+    // phase 1: each thread handles 8 consecutive columns of one row; 8 threads per row, 32 rows per pass
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        int rl = p * 32 + (t >> 3), cl = (t & 7) * 8;
+        int r = r0 + rl, c = c0 + cl;
+        v2i q = {0, 0};
+        if (r < rows && c < cols) {
+            if (IN_BYTES == 2) {
+                v4i v = *(const v4i*)(in + ((int64_t)r * cols + c) * 2);
+                q = quant8<FMT>(v, s);
+                if (out) *(v2i*)(out + (int64_t)r * cols + c) = q;
+            } else {
+                q = *(const v2i*)(in + (int64_t)r * cols + c);
+            }
+        }
+        uint32_t lo = (uint32_t)q.x, hi = (uint32_t)q.y;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            tile[cl + i][rl] = (uint8_t)(lo >> (8 * i));
+            tile[cl + 4 + i][rl] = (uint8_t)(hi >> (8 * i));
+        }
+    }
+    __syncthreads();
+    // phase 2: 64 transposed rows of 64 bytes = 256 pieces of 16 bytes
+    if (out_t) {
+        int cl = t >> 2, ch = (t & 3) * 16;
+        int c = c0 + cl, r = r0 + ch;
+        if (c < cols && r < rows) {
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w[i] = *(const uint32_t*)&tile[cl][ch + 4 * i];
+            *(v4i*)(out_t + (int64_t)c * rows + r) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+        }
+    }
+}
+
+}  // namespace ngpt
+
+using namespace ngpt;
+
+extern "C" int ngpt_quant_fp8(const void* in_bf16, void* out_f8, int64_t n, float scale, int fmt, void* stream) {
+    if (!in_bf16 || !out_f8 || n < 0) return fail(NGPT_EINVAL, "ngpt_quant_fp8: null pointer or negative size");
+    if (n % 8) return fail(NGPT_EALIGN, "ngpt_quant_fp8: n=%lld must be a multiple of 8", (long long)n);
+    if (fmt != NGPT_FMT_E4M3 && fmt != NGPT_FMT_E5M2) return fail(NGPT_EINVAL, "ngpt_quant_fp8: fmt=%d", fmt);
+    if (n == 0) return NGPT_OK;
+    int64_t n8 = n / 8;
+    int grid = (int)((n8 + 255) / 256 < (int64_t)num_cus() * 16 ? (n8 + 255) / 256 : (int64_t)num_cus() * 16);
+    hipStream_t st = (hipStream_t)stream;
+    if (fmt == NGPT_FMT_E4M3)
+        quant_kernel<FMT_E4M3><<<grid, 256, 0, st>>>((const v4i*)in_bf16, (v2i*)out_f8, n8, scale);
+    else
+        quant_kernel<FMT_E5M2><<<grid, 256, 0, st>>>((const v4i*)in_bf16, (v2i*)out_f8, n8, scale);
+    return check_launch("quant_kernel");
+}
+
+extern "C" int ngpt_quant_fp8_2d(const void* in_bf16, int rows, int cols, float scale, int fmt,
+                                 void* out_f8, void* out_f8_t, void* stream) {
+    if (!in_bf16 || rows <= 0 || cols <= 0 || (!out_f8 && !out_f8_t))
+        return fail(NGPT_EINVAL, "ngpt_quant_fp8_2d: null pointer or empty matrix");
+    if (rows % 16 || cols % 16)
+        return fail(NGPT_EALIGN, "ngpt_quant_fp8_2d: rows=%d and cols=%d must be multiples of 16", rows, cols);
+    if (fmt != NGPT_FMT_E4M3 && fmt != NGPT_FMT_E5M2) return fail(NGPT_EINVAL, "ngpt_quant_fp8_2d: fmt=%d", fmt);
+    hipStream_t st = (hipStream_t)stream;
+    if (!out_f8_t) return ngpt_quant_fp8(in_bf16, out_f8, (int64_t)rows * cols, scale, fmt, stream);
+    dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+    if (fmt == NGPT_FMT_E4M3)
+        tile_transpose_kernel<FMT_E4M3, 2><<<grid, 256, 0, st>>>((const uint8_t*)in_bf16, rows, cols, scale,
+                                                                (uint8_t*)out_f8, (uint8_t*)out_f8_t);
+    else
+        tile_transpose_kernel<FMT_E5M2, 2><<<grid, 256, 0, st>>>((const uint8_t*)in_bf16, rows, cols, scale,
+                                                                (uint8_t*)out_f8, (uint8_t*)out_f8_t);
+    return check_launch("tile_transpose_kernel(quant)");
+}
+
+extern "C" int ngpt_transpose_u8(const void* in, int rows, int cols, void* out, void* stream) {
+    if (!in || !out || rows <= 0 || cols <= 0) return fail(NGPT_EINVAL, "ngpt_transpose_u8: null pointer or empty matrix");
+    if (rows % 16 || cols % 16)
+        return fail(NGPT_EALIGN, "ngpt_transpose_u8: rows=%d and cols=%d must be multiples of 16", rows, cols);
+    dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+    tile_transpose_kernel<FMT_E4M3, 1><<<grid, 256, 0, (hipStream_t)stream>>>((const uint8_t*)in, rows, cols, 1.0f,
+                                                                             nullptr, (uint8_t*)out);
+    return check_launch("tile_transpose_kernel(u8)");
+}

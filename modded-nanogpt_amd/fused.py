@@ -1,0 +1,148 @@
+"""The two autograd functions the reference model calls, with identical `apply` signatures:
+
+    FusedLinearReLUSquareFunction   reference triton_kernels.py:667-729 (alias ReLUSqrdMLP, train_gpt.py:48)
+    FusedSoftcappedCrossEntropy     reference triton_kernels.py:1208-1292
+
+plus the launch wrappers the reference exports beside them (`linear_relu_square`,
+`transpose_copy`).  `train_gpt.py:42` imports these names from a module called
+`triton_kernels`; this module exports the same names.
+"""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from . import _lib, ops
+
+E4M3 = torch.float8_e4m3fn
+
+
+def transpose_copy(src: Tensor, dst: Tensor) -> None:
+    """dst (N, M) = src (M, N).T for 1-byte element types -- reference triton_kernels.py:819-841."""
+    assert src.ndim == 2 and dst.ndim == 2
+    M, N = src.shape
+    assert dst.shape == (N, M), f"Expected dst shape ({N}, {M}), got {dst.shape}"
+    assert src.is_contiguous() and dst.is_contiguous() and src.element_size() == 1 and dst.element_size() == 1
+    ops._gpu(src, dst)
+    _lib.check(_lib.load().ngpt_transpose_u8(src.data_ptr(), M, N, dst.data_ptr(), ops._stream(src)),
+               "ngpt_transpose_u8")
+
+
+def linear_relu_square(a, b, aux=None, a_f8=None, b_f8=None, dequant_scale_ptr=None,
+                       activation_scale=None, partial_amax=None):
+    """Reference launcher triton_kernels.py:576-665.
+
+    Forward (aux is None): post = relu(a @ b.T)^2.  With b_f8: the contraction runs on the e4m3
+    copies and is scaled by the 1-element device tensor `dequant_scale_ptr`; with
+    `activation_scale` an e4m3 copy of post and per-workgroup amax partials are produced too.
+    Backward (aux = post): dpre = 2 * (a @ b.T) * sqrt(post), all bf16."""
+    M, K = a.shape
+    N, K2 = b.shape
+    assert K == K2
+    use_fp8 = b_f8 is not None
+    emit_fp8 = activation_scale is not None
+    if aux is None:
+        if use_fp8:
+            assert dequant_scale_ptr is not None and a_f8 is not None
+            if emit_fp8:
+                assert partial_amax is not None
+                return ops.fc_relu2_fwd_emit(a_f8, b_f8, dequant_scale_ptr, activation_scale, partial_amax)
+            return ops.fc_relu2_fwd(a_f8, b_f8, dequant_scale_ptr)
+        c = a @ b.T                                     # bf16 GEMM (hipBLASLt), fp32 accumulate
+        r = torch.clamp_min(c, 0)
+        return r * r
+    c = a @ b.T
+    return (2 * c.float() * torch.sqrt(aux.float())).to(a.dtype)
+
+
+class FusedLinearReLUSquareFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, W1, W2, W1_f8=None, dequant_scale=None, x_f8=None, W2_f8=None, W2_scale=None,
+                activation_scale=None, partial_amax=None):
+        # Forward stores only post = relu(x @ W1.T)^2; `pre` is never materialised.
+        x_flat = x.view((-1, x.shape[-1]))
+        post_f8 = None
+        if W1_f8 is not None:
+            assert x_f8 is not None and dequant_scale is not None
+            x_f8 = x_f8.view((-1, x_f8.shape[-1]))
+            if W2_f8 is not None:
+                assert W2_scale is not None and activation_scale is not None
+                assert partial_amax is not None
+                post, post_f8 = linear_relu_square(x_flat, W1, a_f8=x_f8, b_f8=W1_f8,
+                                                   dequant_scale_ptr=dequant_scale,
+                                                   activation_scale=activation_scale,
+                                                   partial_amax=partial_amax)
+            else:
+                post = linear_relu_square(x_flat, W1, a_f8=x_f8, b_f8=W1_f8, dequant_scale_ptr=dequant_scale)
+        else:
+            post = linear_relu_square(x_flat, W1)
+        if W2_f8 is not None:
+            # W2_f8 is the (H, D) view of a (D, H) row-major e4m3 buffer: the contraction index H
+            # is contiguous on both sides, which is what the TN GEMM reads.  The two scales are
+            # 1-element device tensors; their product is taken on the device, no host sync.
+            w2_dh = W2_f8.T
+            assert w2_dh.is_contiguous()
+            x3 = ops.gemm_fp8_tn(post_f8, w2_dh, 1.0, out_dtype=torch.float32)
+            x3 = (x3 * (activation_scale * W2_scale)).to(torch.bfloat16)
+        else:
+            x3 = post @ W2
+        # Backward stays BF16: it consumes `post` (and W2), not their FP8 copies.
+        ctx.save_for_backward(x, W1, W2, post)
+        return x3.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, W1, W2, post = ctx.saved_tensors
+        x_flat = x.view((-1, x.shape[-1]))
+        g = grad_output.reshape((-1, grad_output.shape[-1]))
+        dW2 = post.T @ g
+        dpre = linear_relu_square(g, W2, aux=post)
+        dW1 = dpre.T @ x_flat
+        dx = dpre @ W1
+        return dx.view(x.shape), dW1, dW2, None, None, None, None, None, None, None
+
+
+ReLUSqrdMLP = FusedLinearReLUSquareFunction.apply
+
+
+class FusedSoftcappedCrossEntropy(torch.autograd.Function):
+    """lm_head GEMM + 23*sigmoid((l+5)/7.5) softcap + cross-entropy, forward and backward, with the
+    [M, V] logits never written to HBM.  `lm_head_weight` is (in, out) as at the reference's HEAD
+    (`w_layout="in_out"`); pass `w_layout="out_in"` as a keyword-free 14th argument for the
+    (out, in) convention of `nanogpt::mm`."""
+
+    @staticmethod
+    def forward(ctx, x, targets, mtp_weights, prefix_targets, prefix_weight, lm_head_weight,
+                x_s, w_s, grad_s, grad_scale, A=23.0, B=5.0, C=7.5, w_layout="in_out"):
+        assert w_layout in ("in_out", "out_in")
+        w_in_out = w_layout == "in_out"
+        n_rows = x.shape[0]
+        dev = x.device
+        if mtp_weights is None:
+            mtp_weights = torch.tensor([1.0], device=dev, dtype=torch.float32)
+        mtp_weights = mtp_weights.to(torch.float32).contiguous()
+        targets = targets.contiguous()
+        if prefix_targets is None:
+            prefix_targets = torch.full((n_rows,), -1, dtype=torch.int64, device=dev)
+        prefix_targets = prefix_targets.contiguous()
+        if prefix_weight is None:
+            prefix_weight = torch.zeros(1, dtype=torch.float32, device=dev)
+        prefix_weight = prefix_weight.reshape(1).to(torch.float32).contiguous()
+
+        losses, lse, saved_sigma, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(
+            x.contiguous(), lm_head_weight.contiguous(), targets, mtp_weights, prefix_targets, prefix_weight,
+            x_s, w_s, A, B, C, w_in_out)
+        ctx.save_for_backward(targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma, x_f8, w_f8)
+        ctx.params = (A, B, C, x_s, w_s, grad_s, grad_scale, w_in_out)
+        return losses
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        # grad_output is ignored: grad_scale is folded into the gradient, as in the reference
+        # (triton_kernels.py:1117, 1262).
+        targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma, x_f8, w_f8 = ctx.saved_tensors
+        A, B, C, x_s, w_s, grad_s, grad_scale, w_in_out = ctx.params
+        grad_x, grad_w = torch.ops.nanogpt.lmhead_ce_bwd(
+            x_f8, w_f8, targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma,
+            x_s, w_s, grad_s, grad_scale, A, B, C, w_in_out)
+        return grad_x, None, None, None, None, grad_w, None, None, None, None, None, None, None, None

@@ -1,0 +1,376 @@
+"""`torch.library` operators of the FP8 contraction path, under the reference's own names and
+schemas, backed by libngpt_fp8.so (hand-written HIP for gfx950) through its C ABI.
+
+    nanogpt::mm, nanogpt::mm_backward          reference train_gpt_medium.py:40-116
+    nanogpt::mm_t, nanogpt::mm_t_backward      reference train_gpt.py:70-162
+    nanogpt::ce_fwd_bwd                        reference triton_kernels.py:1182-1206
+    nanogpt::lmhead_ce_fwd / _bwd              the fused lm_head + softcapped CE behind
+                                               FusedSoftcappedCrossEntropy (no reference op: the
+                                               reference materialises the logits instead)
+    nanogpt::fc_relu2_fwd                      linear_relu_square(..., a_f8=, b_f8=), triton_kernels.py:576-665
+
+Scales are Python floats in the schema (graph constants under torch.compile), every op has a
+fake implementation reproducing shapes, dtypes and strides, and `mm` / `mm_t` carry the
+reference's autograd contract (saved x_f8 / w_f8, `set_materialize_grads(False)`).
+All tensors must live on the GPU: there is no CPU implementation behind these ops.
+"""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+E4M3 = torch.float8_e4m3fn
+E5M2 = torch.float8_e5m2
+MAX_PREDICT = _lib.MAX_PREDICT
+
+
+def _gpu(*tensors: Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("nanogpt FP8 ops run on the GPU only (got a CPU tensor); "
+                               "there is no CPU fallback")
+
+
+def _p(t: Tensor | None):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _workspace(nbytes: int, device) -> Tensor:
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+# ------------------------------------------------------------------------------------------------
+# nanogpt::mm  (weight stored (out, in))
+
+@torch.library.custom_op("nanogpt::mm", mutates_args=())
+def mm_op(x: Tensor, w: Tensor, x_s: float, w_s: float, grad_s: float) -> tuple[Tensor, Tensor, Tensor]:
+    assert x.is_contiguous() and w.is_contiguous()
+    assert x.ndim == w.ndim == 2 and x.shape[1] == w.shape[1]
+    assert x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    _gpu(x, w)
+    lib = _lib.load()
+    M, K = x.shape
+    N = w.shape[0]
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    x_f8 = torch.empty((M, K), dtype=E4M3, device=x.device)
+    w_f8 = torch.empty((N, K), dtype=E4M3, device=x.device)
+    _lib.check(lib.ngpt_mm_fwd(_p(x), _p(w), M, N, K, x_s, w_s, _p(out), _p(x_f8), _p(w_f8),
+                               _lib.W_OUT_IN, None, 0, _stream(x)), "ngpt_mm_fwd")
+    return out, x_f8, w_f8
+
+
+@mm_op.register_fake
+def _(x: Tensor, w: Tensor, *_):
+    assert x.ndim == w.ndim == 2
+    assert x.shape[1] == w.shape[1]
+    assert x.device == w.device
+    assert x.is_contiguous() and w.is_contiguous()
+    return x @ w.T, x.to(E4M3), w.to(E4M3)
+
+
+@torch.library.custom_op("nanogpt::mm_backward", mutates_args=())
+def mm_backward_op(g: Tensor, x_f8: Tensor, w_f8: Tensor, x_s: float, w_s: float, grad_s: float) -> tuple[Tensor, Tensor]:
+    assert g.is_contiguous()
+    _gpu(g, x_f8, w_f8)
+    lib = _lib.load()
+    M, N = g.shape
+    K = x_f8.shape[1]
+    assert x_f8.shape == (M, K) and w_f8.shape == (N, K)
+    dx = torch.empty((M, K), dtype=torch.bfloat16, device=g.device)
+    dw_kn = torch.empty((K, N), dtype=torch.float32, device=g.device)
+    ws = _workspace(lib.ngpt_mm_bwd_workspace_bytes(M, N, K, _lib.W_OUT_IN), g.device)
+    _lib.check(lib.ngpt_mm_bwd(_p(g), _p(x_f8.contiguous()), _p(w_f8.contiguous()), M, N, K, x_s, w_s, grad_s,
+                               _p(dx), _p(dw_kn), _lib.W_OUT_IN, _p(ws), ws.numel(), _stream(g)), "ngpt_mm_bwd")
+    return dx, dw_kn.T
+
+
+@mm_backward_op.register_fake
+def _(g: Tensor, x_f8: Tensor, w_f8: Tensor, *_):
+    return x_f8.to(torch.bfloat16), w_f8.T.contiguous().T.to(torch.float32)
+
+
+def _mm_backward(ctx, grad_out: Tensor, *_):
+    x_f8, w_f8 = ctx.saved_tensors
+    x_s, w_s, grad_s = ctx.scales
+    grad_x, grad_w = torch.ops.nanogpt.mm_backward(grad_out, x_f8, w_f8, x_s, w_s, grad_s)
+    return grad_x, grad_w, None, None, None
+
+
+def _mm_setup_context(ctx: torch.autograd.function.FunctionCtx, inputs, output):
+    *_, x_s, w_s, grad_s = inputs
+    _, x_f8, w_f8 = output
+    ctx.save_for_backward(x_f8, w_f8)
+    ctx.scales = x_s, w_s, grad_s
+    ctx.set_materialize_grads(False)
+
+
+mm_op.register_autograd(_mm_backward, setup_context=_mm_setup_context)
+
+
+# ------------------------------------------------------------------------------------------------
+# nanogpt::mm_t  (weight stored (in, out))
+
+@torch.library.custom_op("nanogpt::mm_t", mutates_args=())
+def mm_t_op(x: Tensor, w: Tensor, x_s: float, w_s: float, grad_s: float) -> tuple[Tensor, Tensor, Tensor]:
+    """Computes y = x @ w with F8 weights stored as (in_features, out_features)."""
+    assert x.is_contiguous() and w.is_contiguous()
+    assert x.ndim == w.ndim == 2 and x.shape[1] == w.shape[0]
+    assert x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    _gpu(x, w)
+    lib = _lib.load()
+    M, K = x.shape
+    N = w.shape[1]
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    x_f8 = torch.empty((M, K), dtype=E4M3, device=x.device)
+    w_f8 = torch.empty((K, N), dtype=E4M3, device=x.device)
+    ws = _workspace(lib.ngpt_mm_fwd_workspace_bytes(M, N, K, _lib.W_IN_OUT), x.device)
+    _lib.check(lib.ngpt_mm_fwd(_p(x), _p(w), M, N, K, x_s, w_s, _p(out), _p(x_f8), _p(w_f8),
+                               _lib.W_IN_OUT, _p(ws), ws.numel(), _stream(x)), "ngpt_mm_fwd")
+    return out, x_f8, w_f8
+
+
+@mm_t_op.register_fake
+def _(x: Tensor, w: Tensor, *_):
+    assert x.ndim == w.ndim == 2
+    assert x.shape[1] == w.shape[0]
+    assert x.device == w.device
+    assert x.is_contiguous() and w.is_contiguous()
+    return x @ w, x.to(E4M3), w.to(E4M3)
+
+
+@torch.library.custom_op("nanogpt::mm_t_backward", mutates_args=())
+def mm_t_backward_op(g: Tensor, x_f8: Tensor, w_f8: Tensor, x_s: float, w_s: float, grad_s: float) -> tuple[Tensor, Tensor]:
+    assert g.is_contiguous()
+    _gpu(g, x_f8, w_f8)
+    lib = _lib.load()
+    M, N = g.shape
+    K = x_f8.shape[1]
+    assert x_f8.shape == (M, K) and w_f8.shape == (K, N)
+    dx = torch.empty((M, K), dtype=torch.bfloat16, device=g.device)
+    dw = torch.empty((K, N), dtype=torch.float32, device=g.device)
+    ws = _workspace(lib.ngpt_mm_bwd_workspace_bytes(M, N, K, _lib.W_IN_OUT), g.device)
+    _lib.check(lib.ngpt_mm_bwd(_p(g), _p(x_f8.contiguous()), _p(w_f8.contiguous()), M, N, K, x_s, w_s, grad_s,
+                               _p(dx), _p(dw), _lib.W_IN_OUT, _p(ws), ws.numel(), _stream(g)), "ngpt_mm_bwd")
+    return dx, dw
+
+
+@mm_t_backward_op.register_fake
+def _(g: Tensor, x_f8: Tensor, w_f8: Tensor, *_):
+    return x_f8.to(torch.bfloat16), w_f8.to(torch.float32)
+
+
+def _mm_t_backward(ctx, grad_out: Tensor, *_):
+    x_f8, w_f8 = ctx.saved_tensors
+    x_s, w_s, grad_s = ctx.scales
+    grad_x, grad_w = torch.ops.nanogpt.mm_t_backward(grad_out, x_f8, w_f8, x_s, w_s, grad_s)
+    return grad_x, grad_w, None, None, None
+
+
+mm_t_op.register_autograd(_mm_t_backward, setup_context=_mm_setup_context)
+
+
+# ------------------------------------------------------------------------------------------------
+# nanogpt::ce_fwd_bwd  (logits materialised by the caller)
+
+@torch.library.custom_op("nanogpt::ce_fwd_bwd", mutates_args={"losses", "grad_input"})
+def ce_fwd_bwd(
+    logits: Tensor,
+    targets: Tensor,
+    mtp_weights: Tensor,
+    prefix_targets: Tensor,
+    prefix_weight: Tensor,
+    losses: Tensor,
+    grad_input: Tensor,
+    n_rows: int,
+    n_predict: int,
+    A: float,
+    B: float,
+    C: float,
+    grad_s: float,
+    grad_scale: float,
+) -> None:
+    _gpu(logits, targets, mtp_weights, prefix_targets, prefix_weight, losses, grad_input)
+    assert logits.dtype == torch.bfloat16 and logits.is_contiguous() and logits.ndim == 2
+    assert logits.shape[0] == n_rows and grad_input.shape == logits.shape
+    assert targets.dtype == torch.int64 and prefix_targets.dtype == torch.int64
+    assert mtp_weights.dtype == torch.float32 and mtp_weights.numel() >= n_predict
+    assert losses.dtype == torch.float32 and grad_input.dtype == E5M2 and grad_input.is_contiguous()
+    lib = _lib.load()
+    ws = _workspace(lib.ngpt_ce_fwd_bwd_workspace_bytes(), logits.device)
+    _lib.check(lib.ngpt_ce_fwd_bwd(_p(logits), _p(targets), _p(mtp_weights), _p(prefix_targets),
+                                   _p(prefix_weight), _p(losses), _p(grad_input), n_rows, logits.shape[1],
+                                   n_predict, A, B, C, grad_s, grad_scale, _p(ws), ws.numel(),
+                                   _stream(logits)), "ngpt_ce_fwd_bwd")
+
+
+@ce_fwd_bwd.register_fake
+def _(logits, targets, mtp_weights, prefix_targets, prefix_weight, losses, grad_input, *_):
+    return None
+
+
+# ------------------------------------------------------------------------------------------------
+# Fused lm_head + softcapped CE (the logits are never stored)
+
+@torch.library.custom_op("nanogpt::lmhead_ce_fwd", mutates_args=())
+def lmhead_ce_fwd(x: Tensor, w: Tensor, targets: Tensor, mtp_weights: Tensor, prefix_targets: Tensor,
+                  prefix_weight: Tensor, x_s: float, w_s: float, A: float, B: float, C: float,
+                  w_in_out: bool) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
+    """-> (losses [M] f32, lse [M] f32, saved_sigma [MAX_PREDICT+1, M] f32, x_f8 [M,K], w_f8 [V,K])."""
+    _gpu(x, w, targets, mtp_weights, prefix_targets, prefix_weight)
+    assert x.is_contiguous() and w.is_contiguous() and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    assert targets.dtype == torch.int64 and prefix_targets.dtype == torch.int64
+    lib = _lib.load()
+    M, K = x.shape
+    V = w.shape[1] if w_in_out else w.shape[0]
+    assert (w.shape[0] if w_in_out else w.shape[1]) == K
+    n_predict = mtp_weights.shape[0]
+    dev = x.device
+    losses = torch.empty(M, dtype=torch.float32, device=dev)
+    lse = torch.empty(M, dtype=torch.float32, device=dev)
+    saved_sigma = torch.zeros((MAX_PREDICT + 1, M), dtype=torch.float32, device=dev)
+    x_f8 = torch.empty((M, K), dtype=E4M3, device=dev)
+    w_f8 = torch.empty((V, K), dtype=E4M3, device=dev)
+    layout = _lib.W_IN_OUT if w_in_out else _lib.W_OUT_IN
+    ws = _workspace(lib.ngpt_lmhead_ce_fwd_workspace_bytes(M, K, V, layout), dev)
+    _lib.check(lib.ngpt_lmhead_ce_fwd(_p(x), _p(w), _p(targets), _p(mtp_weights), n_predict,
+                                      _p(prefix_targets), _p(prefix_weight), M, K, V, x_s, w_s, A, B, C,
+                                      _p(losses), _p(lse), _p(saved_sigma), _p(x_f8), _p(w_f8), layout,
+                                      _p(ws), ws.numel(), _stream(x)), "ngpt_lmhead_ce_fwd")
+    return losses, lse, saved_sigma, x_f8, w_f8
+
+
+@lmhead_ce_fwd.register_fake
+def _(x, w, targets, mtp_weights, prefix_targets, prefix_weight, x_s, w_s, A, B, C, w_in_out):
+    M, K = x.shape
+    V = w.shape[1] if w_in_out else w.shape[0]
+    f32 = dict(dtype=torch.float32, device=x.device)
+    return (torch.empty(M, **f32), torch.empty(M, **f32), torch.empty((MAX_PREDICT + 1, M), **f32),
+            torch.empty((M, K), dtype=E4M3, device=x.device), torch.empty((V, K), dtype=E4M3, device=x.device))
+
+
+@torch.library.custom_op("nanogpt::lmhead_ce_bwd", mutates_args=())
+def lmhead_ce_bwd(x_f8: Tensor, w_f8: Tensor, targets: Tensor, mtp_weights: Tensor, prefix_targets: Tensor,
+                  prefix_weight: Tensor, lse: Tensor, saved_sigma: Tensor, x_s: float, w_s: float,
+                  grad_s: float, grad_scale: float, A: float, B: float, C: float,
+                  w_in_out: bool) -> tuple[Tensor, Tensor]:
+    """-> (dx [M,K] bf16, dW fp32 in the weight's layout)."""
+    _gpu(x_f8, w_f8, targets, lse, saved_sigma)
+    lib = _lib.load()
+    M, K = x_f8.shape
+    V = w_f8.shape[0]
+    dev = x_f8.device
+    dx = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
+    dw = torch.empty((K, V) if w_in_out else (V, K), dtype=torch.float32, device=dev)
+    layout = _lib.W_IN_OUT if w_in_out else _lib.W_OUT_IN
+    ws = _workspace(lib.ngpt_lmhead_ce_bwd_workspace_bytes(M, K, V, layout), dev)
+    _lib.check(lib.ngpt_lmhead_ce_bwd(_p(x_f8), _p(w_f8), _p(targets), _p(mtp_weights), mtp_weights.shape[0],
+                                      _p(prefix_targets), _p(prefix_weight), _p(lse), _p(saved_sigma),
+                                      M, K, V, x_s, w_s, grad_s, grad_scale, A, B, C, _p(dx), _p(dw), layout,
+                                      _p(ws), ws.numel(), _stream(x_f8)), "ngpt_lmhead_ce_bwd")
+    return dx, dw
+
+
+@lmhead_ce_bwd.register_fake
+def _(x_f8, w_f8, targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma,
+      x_s, w_s, grad_s, grad_scale, A, B, C, w_in_out):
+    M, K = x_f8.shape
+    V = w_f8.shape[0]
+    return (torch.empty((M, K), dtype=torch.bfloat16, device=x_f8.device),
+            torch.empty((K, V) if w_in_out else (V, K), dtype=torch.float32, device=x_f8.device))
+
+
+# ------------------------------------------------------------------------------------------------
+# FP8 up-projection + ReLU^2
+
+@torch.library.custom_op("nanogpt::fc_relu2_fwd", mutates_args=())
+def fc_relu2_fwd(x_f8: Tensor, w_f8: Tensor, dequant_scale: Tensor) -> Tensor:
+    """post [M,N] bf16 = relu(bf16(x_f8 . w_f8^T * dequant))^2."""
+    _gpu(x_f8, w_f8, dequant_scale)
+    assert x_f8.is_contiguous() and w_f8.is_contiguous() and x_f8.dtype == E4M3 and w_f8.dtype == E4M3
+    assert dequant_scale.dtype == torch.float32 and dequant_scale.numel() >= 1
+    lib = _lib.load()
+    M, K = x_f8.shape
+    N = w_f8.shape[0]
+    post = torch.empty((M, N), dtype=torch.bfloat16, device=x_f8.device)
+    _lib.check(lib.ngpt_fc_relu2_fwd(_p(x_f8), _p(w_f8), _p(dequant_scale), M, N, K, _p(post), None, None,
+                                     None, 0, _stream(x_f8)), "ngpt_fc_relu2_fwd")
+    return post
+
+
+@fc_relu2_fwd.register_fake
+def _(x_f8, w_f8, dequant_scale):
+    return torch.empty((x_f8.shape[0], w_f8.shape[0]), dtype=torch.bfloat16, device=x_f8.device)
+
+
+@torch.library.custom_op("nanogpt::fc_relu2_fwd_emit", mutates_args={"partial_amax"})
+def fc_relu2_fwd_emit(x_f8: Tensor, w_f8: Tensor, dequant_scale: Tensor, activation_scale: Tensor,
+                      partial_amax: Tensor) -> tuple[Tensor, Tensor]:
+    """As fc_relu2_fwd, plus post_f8 = e4m3(min(post / activation_scale, 448)) and the
+    per-workgroup running max of post in partial_amax."""
+    _gpu(x_f8, w_f8, dequant_scale, activation_scale, partial_amax)
+    assert x_f8.is_contiguous() and w_f8.is_contiguous() and partial_amax.is_contiguous()
+    assert partial_amax.dtype == torch.float32 and activation_scale.dtype == torch.float32
+    lib = _lib.load()
+    M, K = x_f8.shape
+    N = w_f8.shape[0]
+    post = torch.empty((M, N), dtype=torch.bfloat16, device=x_f8.device)
+    post_f8 = torch.empty((M, N), dtype=E4M3, device=x_f8.device)
+    _lib.check(lib.ngpt_fc_relu2_fwd(_p(x_f8), _p(w_f8), _p(dequant_scale), M, N, K, _p(post), _p(post_f8),
+                                     _p(activation_scale), _p(partial_amax), partial_amax.numel(),
+                                     _stream(x_f8)), "ngpt_fc_relu2_fwd")
+    return post, post_f8
+
+
+@fc_relu2_fwd_emit.register_fake
+def _(x_f8, w_f8, dequant_scale, activation_scale, partial_amax):
+    M, N = x_f8.shape[0], w_f8.shape[0]
+    return (torch.empty((M, N), dtype=torch.bfloat16, device=x_f8.device),
+            torch.empty((M, N), dtype=E4M3, device=x_f8.device))
+
+
+# ------------------------------------------------------------------------------------------------
+# Building blocks exposed for callers and tests (plain functions, not registered ops)
+
+def quant_fp8(x: Tensor, scale: float, dtype: torch.dtype = E4M3) -> Tensor:
+    """`x.div(scale).to(dtype)` for a contiguous bf16 tensor, on the GPU."""
+    _gpu(x)
+    assert x.dtype == torch.bfloat16 and x.is_contiguous()
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    fmt = _lib.E4M3 if dtype == E4M3 else _lib.E5M2
+    _lib.check(_lib.load().ngpt_quant_fp8(_p(x), _p(out), x.numel(), scale, fmt, _stream(x)), "ngpt_quant_fp8")
+    return out
+
+
+def quant_fp8_2d(x: Tensor, scale: float, dtype: torch.dtype = E4M3, want_rowmajor=True, want_transposed=True):
+    _gpu(x)
+    assert x.dtype == torch.bfloat16 and x.is_contiguous() and x.ndim == 2
+    R, C = x.shape
+    out = torch.empty((R, C), dtype=dtype, device=x.device) if want_rowmajor else None
+    out_t = torch.empty((C, R), dtype=dtype, device=x.device) if want_transposed else None
+    fmt = _lib.E4M3 if dtype == E4M3 else _lib.E5M2
+    _lib.check(_lib.load().ngpt_quant_fp8_2d(_p(x), R, C, scale, fmt, _p(out), _p(out_t), _stream(x)),
+               "ngpt_quant_fp8_2d")
+    return out, out_t
+
+
+def gemm_fp8_tn(a: Tensor, b: Tensor, scale: float, out_dtype=torch.bfloat16, out: Tensor | None = None,
+                accumulate: bool = False) -> Tensor:
+    """C[r,c] = scale * sum_k a[r,k] b[c,k] for fp8 a [R,K], b [C,K] (contraction contiguous)."""
+    _gpu(a, b)
+    fmt = {E4M3: _lib.E4M3, E5M2: _lib.E5M2}
+    R, K = a.shape
+    Cn = b.shape[0]
+    assert b.shape[1] == K and a.stride(1) == 1 and b.stride(1) == 1
+    if out is None:
+        out = torch.empty((R, Cn), dtype=out_dtype, device=a.device)
+    kind = 0 if out.dtype == torch.bfloat16 else (2 if accumulate else 1)
+    _lib.check(_lib.load().ngpt_gemm_fp8_tn(_p(a), fmt[a.dtype], a.stride(0), _p(b), fmt[b.dtype], b.stride(0),
+                                            R, Cn, K, scale, _p(out), out.stride(0), kind, _stream(a)),
+               "ngpt_gemm_fp8_tn")
+    return out
