@@ -1,0 +1,155 @@
+"""Benchmark of the FP8 lm_head + fused softcapped cross-entropy, forward + backward, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload: BASELINE config 3 -- x bf16 [49152, 768] ~ N(0,1), W bf16 [50304, 768] ~ N(0, 1/768),
+lm_head scales x_s = 100/448, w_s = 1.6/448, grad_s = 0.75/448, int64 targets uniform in [0, 50257),
+outputs per-token losses, dx bf16, dW fp32.  One "step" = one forward + one backward of the path
+with all inputs already resident in HBM.  Algorithmic work per step: 6*M*K*V FLOP (three GEMMs;
+the logits recomputed in the backward are not counted).
+
+Prints one JSON line.  Besides the whole-step throughput it carries
+  roofline      for the kernel that takes the most time, timed with HIP events on its stream,
+  cpu_baseline  the CPU oracle (PyTorch eager restatement) on a bounded row sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import torch
+
+PEAK_FP8_TFLOPS = 5033.0      # MI355X dense FP8 MFMA (published)
+M, K, V = 49152, 768, 50304
+SLOT_NAMES = ["lm_head_ce_fwd", "dlogits_recompute", "dx_gemm", "dw_gemm", "other_gemm"]
+
+
+def profile_read(lib):
+    out = {}
+    for slot, name in enumerate(SLOT_NAMES):
+        ms, n = ctypes.c_double(0), ctypes.c_int(0)
+        lib.ngpt_profile_read(slot, ctypes.byref(ms), ctypes.byref(n))
+        out[name] = (ms.value, n.value)
+    return out
+
+
+def cpu_baseline(oracle, x, w, t, sc, budget_s=20.0):
+    """Oracle forward+backward on the first rows of the same inputs; ~budget_s seconds of CPU work."""
+    threads = torch.get_num_threads()
+    rows_per_chunk = 1024
+    oracle.lm_head_ce_chunked(x, t, w, **sc, rows_per_chunk=rows_per_chunk, max_rows=rows_per_chunk)   # warm-up
+    t0 = time.perf_counter()
+    oracle.lm_head_ce_chunked(x, t, w, **sc, rows_per_chunk=rows_per_chunk, max_rows=rows_per_chunk)
+    per_chunk = time.perf_counter() - t0
+    n_chunks = max(1, min(M // rows_per_chunk, int(budget_s / max(per_chunk, 1e-3))))
+    rows = n_chunks * rows_per_chunk
+    t0 = time.perf_counter()
+    _, _, _, done = oracle.lm_head_ce_chunked(x, t, w, **sc, rows_per_chunk=rows_per_chunk, max_rows=rows)
+    dt = time.perf_counter() - t0
+    return {
+        "value": done / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
+        "sample": f"first {done} of {M} rows, K={K}, V={V}, forward+backward in {rows_per_chunk}-row chunks, "
+                  f"{dt:.1f} s of PyTorch-eager fp32 on the host CPU",
+        "tflops": 6.0 * done * K * V / dt / 1e12,
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is built and measured on ONE GPU (the kernel on one GPU's share of the "
+              "batch, M=49152); runs with more than one GPU are not part of this build.", file=sys.stderr)
+        return 2
+
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import modded_nanogpt_amd as amd
+    from oracle import nanogpt_fp8_oracle as oracle
+
+    lib = amd._lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    x, w, t, sc = oracle.make_cfg3(seed=0)
+    xd, wd, td = x.to(dev), w.to(dev), t.to(dev)
+    mtp = torch.tensor([1.0], device=dev)
+    pt = torch.full((M,), -1, dtype=torch.int64, device=dev)
+    pw = torch.zeros(1, device=dev)
+
+    def step():
+        losses, lse, sig, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(
+            xd, wd, td, mtp, pt, pw, sc["x_s"], sc["w_s"], sc["A"], sc["B"], sc["C"], False)
+        dx, dw = torch.ops.nanogpt.lmhead_ce_bwd(
+            x_f8, w_f8, td, mtp, pt, pw, lse, sig, sc["x_s"], sc["w_s"], sc["grad_s"], sc["grad_scale"],
+            sc["A"], sc["B"], sc["C"], False)
+        return losses, dx, dw
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.ngpt_profile_enable(1)
+    profile_read(lib)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    prof = profile_read(lib)
+    lib.ngpt_profile_enable(0)
+
+    ms_per_step = dt / args.steps * 1e3
+    flops_step = 6.0 * M * K * V
+    tflops = flops_step / (ms_per_step * 1e-3) / 1e12
+    mean_loss = float(out[0].mean())
+
+    # roofline of the kernel with the largest share of the step
+    flops_per_launch = {   # algorithmic FLOP of one launch of each kernel at this workload
+        "lm_head_ce_fwd": 2.0 * M * K * V,
+        "dlogits_recompute": None,      # recompute: executed 2*Mc*K*V per launch, algorithmic share 0
+        "dx_gemm": None, "dw_gemm": None, "other_gemm": None,
+    }
+    kernels = {}
+    for name, (ms, n) in prof.items():
+        if n:
+            kernels[name] = {"launches_per_step": n / args.steps, "avg_ms": ms / n, "ms_per_step": ms / args.steps}
+    for name in ("dlogits_recompute", "dx_gemm", "dw_gemm"):
+        if name in kernels:
+            flops_per_launch[name] = 2.0 * M * K * V / kernels[name]["launches_per_step"]
+    dominant = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
+    dom = kernels[dominant]
+    achieved = flops_per_launch[dominant] / (dom["avg_ms"] * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+        "frac": achieved / PEAK_FP8_TFLOPS, "traffic": None,
+        "avg_launch_ms": dom["avg_ms"], "flop_per_launch": flops_per_launch[dominant],
+        "note": "executed 2*rows*K*V FLOP per launch of each GEMM-shaped kernel / its HIP-event duration",
+    }
+
+    result = {
+        "metric": "lm_head+CE fwd+bwd tokens/s at M=49152 (FP8 TFLOP/s and fraction of dense FP8 peak alongside)",
+        "value": M / (ms_per_step * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8", "data": "synthetic",
+        "config": {"workload": "config 3: FP8 lm_head + fused softcapped cross-entropy, forward+backward, "
+                               "M=49152 K=768 V=50304, (out,in) weight, n_predict=1"},
+        "tflops": tflops, "frac_fp8_peak": tflops / PEAK_FP8_TFLOPS, "peak_fp8_tflops": PEAK_FP8_TFLOPS,
+        "flop_per_step": flops_step, "mean_loss": mean_loss,
+        "kernels": kernels, "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(oracle, x, w, t, sc)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

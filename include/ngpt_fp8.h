@@ -47,6 +47,15 @@ const char* ngpt_last_error(void);
 /* Number of compute units the persistent kernels size their grids to (0 if no device). */
 int ngpt_num_cus(void);
 
+/* ---- optional per-kernel timing ------------------------------------------------------------
+ * No counterpart in the reference (contributors patch torch.profiler in by hand).  When enabled,
+ * the heavy launches of the fused lm_head + CE path are bracketed by HIP events on their own
+ * stream.  Slots: 0 forward kernel, 1 dlogits recompute, 2 dx GEMM, 3 dW GEMM, 4 other GEMMs.
+ * ngpt_profile_read waits for the recorded launches of a slot, returns the sum of their
+ * durations and their count, and clears the slot. */
+int ngpt_profile_enable(int on);
+int ngpt_profile_read(int slot, double* total_ms, int* launches);
+
 /* ---- quantisers ---------------------------------------------------------------------------
  * out[i] = fp8(bf16_rne(fp32(in[i]) / scale)), round-to-nearest-even, NOT saturating
  * (e4m3fn overflow -> NaN code, e5m2 overflow -> +-inf): PyTorch-eager `x.div(s).to(fp8)`.

@@ -413,6 +413,12 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
 
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
                float scale, void* out, int64_t ldc, int out_kind, hipStream_t st);
+extern int g_gemm_slot;
+struct GemmSlot {   // books the plain GEMM launches inside a scope under a CE profile slot
+    int saved;
+    explicit GemmSlot(int s) : saved(g_gemm_slot) { g_gemm_slot = s; }
+    ~GemmSlot() { g_gemm_slot = saved; }
+};
 
 static Softcap make_softcap(float A, float B, float C) {
     Softcap sc;
@@ -529,7 +535,10 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
     if (cus < CE_SPLITS) return fail(NGPT_EINVAL, "no HIP device");
     int tiles_m = (M + Cfg::BN - 1) / Cfg::BN;
     int slots = cus / CE_SPLITS < tiles_m ? cus / CE_SPLITS : tiles_m;
-    kernel<<<slots * CE_SPLITS, Cfg::THREADS, LDS, st>>>(g, epi);
+    {
+        ProfileScope prof(PROF_CE_FWD, st);
+        kernel<<<slots * CE_SPLITS, Cfg::THREADS, LDS, st>>>(g, epi);
+    }
     if (int e = check_launch("lm_head CE forward")) return e;
     ce_finalize_kernel<<<(M + 255) / 256, 256, 0, st>>>(part, saved_sigma, epi.ca, sc, losses, lse);
     return check_launch("ce_finalize_kernel");
@@ -609,15 +618,22 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         epi.V = V;
         epi.scale = x_s * w_s;
         int tiles = ((Mc + Cfg::BM - 1) / Cfg::BM) * ((V + Cfg::BN - 1) / Cfg::BN);
-        kernel<<<tiles < cus ? tiles : cus, Cfg::THREADS, LDS, st>>>(g, epi);
+        {
+            ProfileScope prof(PROF_CE_DLOGITS, st);
+            kernel<<<tiles < cus ? tiles : cus, Cfg::THREADS, LDS, st>>>(g, epi);
+        }
         if (int e = check_launch("lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
         ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, dl, dl_t);
         if (int e = check_launch("ce_dl_fix_kernel")) return e;
         // 3. dx[chunk] = dl [Mc, V] . (w^T [K, V])^T
-        if (int e = gemm_store(dl, FMT_E5M2, V, w_t, FMT_E4M3, V, Mc, K, V, grad_s * w_s,
-                               (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, 0, st)) return e;
+        {
+            GemmSlot slot(PROF_CE_DX);
+            if (int e = gemm_store(dl, FMT_E5M2, V, w_t, FMT_E4M3, V, Mc, K, V, grad_s * w_s,
+                                   (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, 0, st)) return e;
+        }
         // 4. dw += over the chunk's tokens
+        GemmSlot slot(PROF_CE_DW);
         const int kind = m0 == 0 ? 1 : 2;
         if (w_layout == NGPT_W_OUT_IN) {   // dw [V, K] = dl^T [V, Mc] . (x^T [K, Mc])^T
             if (int e = gemm_store(dl_t, FMT_E5M2, Mc, x_t + m0, FMT_E4M3, M, V, K, Mc, x_s * grad_s,

@@ -3,8 +3,44 @@
 #include "epilogues.h"
 #include "host_util.h"
 #include "launch.h"
+#include <mutex>
+#include <vector>
 
 namespace ngpt {
+
+// ---------------------------------------------------------------- per-kernel event timing
+namespace {
+struct EventPair {
+    hipEvent_t a, b;
+};
+std::mutex g_prof_mu;
+bool g_prof_on = false;
+std::vector<EventPair> g_prof_pending[PROF_SLOTS];
+std::vector<EventPair> g_prof_free;
+hipEvent_t g_prof_open[PROF_SLOTS];
+}  // namespace
+
+bool profiling_on() { return g_prof_on; }
+
+void profile_begin(int slot, hipStream_t st) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    EventPair p;
+    if (!g_prof_free.empty()) {
+        p = g_prof_free.back();
+        g_prof_free.pop_back();
+    } else if (hipEventCreate(&p.a) != hipSuccess || hipEventCreate(&p.b) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    (void)hipEventRecord(p.a, st);
+    g_prof_pending[slot].push_back(p);
+    g_prof_open[slot] = p.b;
+}
+
+void profile_end(int slot, hipStream_t st) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    if (!g_prof_pending[slot].empty()) (void)hipEventRecord(g_prof_open[slot], st);
+}
 
 static char g_err[512];
 char* last_error_buf() {
@@ -36,10 +72,14 @@ static int check_gemm_dims(const char* who, int R, int C, int K, int64_t lda, in
     return NGPT_OK;
 }
 
+// Which profile slot the next gemm_store launches are booked under (set by the fused CE backward).
+int g_gemm_slot = PROF_GEMM;
+
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
                float scale, void* out, int64_t ldc, int out_kind, hipStream_t st) {
     if (int e = check_gemm_dims("gemm_fp8_tn", R, C, K, lda, ldb)) return e;
     GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K};
+    ProfileScope prof(g_gemm_slot, st);
     if (out_kind == 0) {
         EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
@@ -55,6 +95,35 @@ using namespace ngpt;
 extern "C" int ngpt_abi_version(void) { return 1; }
 extern "C" const char* ngpt_last_error(void) { return last_error_buf(); }
 extern "C" int ngpt_num_cus(void) { return num_cus(); }
+
+extern "C" int ngpt_profile_enable(int on) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof_on = on != 0;
+    return NGPT_OK;
+}
+
+// Waits for the recorded launches of `slot`, adds up their durations and forgets them.
+extern "C" int ngpt_profile_read(int slot, double* total_ms, int* launches) {
+    if (slot < 0 || slot >= PROF_SLOTS || !total_ms || !launches)
+        return fail(NGPT_EINVAL, "ngpt_profile_read: slot=%d", slot);
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    double sum = 0.0;
+    int n = 0;
+    for (EventPair& p : g_prof_pending[slot]) {
+        float ms = 0.0f;
+        if (hipEventSynchronize(p.b) == hipSuccess && hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
+            sum += ms;
+            ++n;
+        } else {
+            (void)hipGetLastError();
+        }
+        g_prof_free.push_back(p);
+    }
+    g_prof_pending[slot].clear();
+    *total_ms = sum;
+    *launches = n;
+    return NGPT_OK;
+}
 
 extern "C" int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const void* B, int fmt_b, int64_t ldb,
                                 int R, int C, int K, float scale, void* out, int64_t ldc, int out_kind,

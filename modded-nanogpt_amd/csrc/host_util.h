@@ -35,6 +35,32 @@ inline int allow_lds(K kernel, int bytes) {
     return NGPT_OK;
 }
 
+// Optional per-kernel timing with HIP events on the launch stream (off by default).
+// Slots name the heavy kernels of the fused lm_head + CE path.
+enum ProfileSlot : int {
+    PROF_CE_FWD = 0,      // lm_head GEMM + softcap + row statistics
+    PROF_CE_DLOGITS = 1,  // logits recompute + e5m2 dlogits
+    PROF_CE_DX = 2,       // dx GEMM
+    PROF_CE_DW = 3,       // dW GEMM
+    PROF_GEMM = 4,        // any other plain GEMM launch
+    PROF_SLOTS = 5
+};
+bool profiling_on();
+void profile_begin(int slot, hipStream_t st);
+void profile_end(int slot, hipStream_t st);
+
+struct ProfileScope {
+    int slot;
+    hipStream_t st;
+    bool on;
+    ProfileScope(int s, hipStream_t stream) : slot(s), st(stream), on(profiling_on()) {
+        if (on) profile_begin(slot, st);
+    }
+    ~ProfileScope() {
+        if (on) profile_end(slot, st);
+    }
+};
+
 inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace ngpt
