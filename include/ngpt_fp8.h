@@ -56,6 +56,10 @@ int ngpt_num_cus(void);
 int ngpt_profile_enable(int on);
 int ngpt_profile_read(int slot, double* total_ms, int* launches);
 
+/* Tuning aid, no counterpart in the reference: key 0 selects the GEMM tile configuration
+ * (0 = default), key 1 the number of persistent workgroups per compute unit. */
+int ngpt_tuning_set(int key, int value);
+
 /* ---- quantisers ---------------------------------------------------------------------------
  * out[i] = fp8(bf16_rne(fp32(in[i]) / scale)), round-to-nearest-even, NOT saturating
  * (e4m3fn overflow -> NaN code, e5m2 overflow -> +-inf): PyTorch-eager `x.div(s).to(fp8)`.
@@ -79,7 +83,7 @@ int ngpt_transpose_u8(const void* in, int rows, int cols, void* out, void* strea
  * index contiguous (row strides lda / ldb bytes).  What `torch._scaled_mm` does for the
  * reference (call sites train_gpt_medium.py:47,76,85; train_gpt.py:85,117,128;
  * triton_kernels.py:1217,1268,1283).  out_kind: 0 = bf16, 1 = fp32, 2 = fp32 accumulate
- * (C += ...).  ldc in elements.  K % 128 == 0, lda % 16 == 0, ldb % 16 == 0. */
+ * (C += ...), 3 = discard the result (times the contraction loop alone).  ldc in elements.  K % 128 == 0, lda % 16 == 0, ldb % 16 == 0. */
 int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const void* B, int fmt_b, int64_t ldb,
                      int R, int C, int K, float scale, void* out, int64_t ldc, int out_kind,
                      void* stream);

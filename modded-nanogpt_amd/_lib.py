@@ -19,6 +19,7 @@ SIGNATURES = {
     "ngpt_abi_version": (_I, []),
     "ngpt_last_error": (c_char_p, []),
     "ngpt_num_cus": (_I, []),
+    "ngpt_tuning_set": (_I, [_I, _I]),
     "ngpt_profile_enable": (_I, [_I]),
     "ngpt_profile_read": (_I, [_I, _P, _P]),
     "ngpt_quant_fp8": (_I, [_P, _P, _L, _F, _I, _P]),

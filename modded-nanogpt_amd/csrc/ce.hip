@@ -9,7 +9,7 @@
 // tables indexed by the logit's bit pattern replace all transcendental work in the hot loops:
 //   tabE[i] = exp(z - A)                     (forward: sum of exponentials, shifted by the cap A)
 //   tabD[i] = exp(z - A) * sigma * (1-sigma) (backward: dlogit = rowf[m] * tabD[i])
-// with rowf[m] = coef * S_w[m] * exp(A - lse[m]).  The tables cover |l| in [2^-16, 2^8) exactly
+// with rowf[m] = coef * S_w[m] * exp(A - lse[m]).  The tables cover |l| in [2^-12, 2^8) exactly
 // (128 mantissa steps per binade, both signs); smaller magnitudes share the entry of l = 0 and
 // larger ones the last entry, where sigma has saturated in bf16.
 #include "epilogues.h"
@@ -18,9 +18,10 @@
 
 namespace ngpt {
 
-constexpr int TAB_LO = 0x3780;            // bf16 bits of 2^-16
-constexpr int TAB_N = 0x4380 - 0x3780;    // 3072 entries per sign, up to 2^8
-constexpr int TAB_ENTRIES = 2 * TAB_N;
+constexpr int TAB_LO = 0x3980;            // bf16 bits of 2^-12
+constexpr int TAB_N = 0x4380 - 0x3980;    // 2560 entries per sign, up to 2^8
+constexpr int TAB_NEG = 4096;             // negative logits start here, so the sign is one index bit
+constexpr int TAB_ENTRIES = TAB_NEG + TAB_N;
 constexpr int TAB_BYTES = TAB_ENTRIES * 4;
 constexpr int MAX_CAND = NGPT_MAX_PREDICT + 1;   // shifted targets + the prefix target
 
@@ -31,7 +32,28 @@ struct Softcap {
 __device__ __forceinline__ int tab_index(uint32_t bf16_bits) {
     int t = (int)(bf16_bits & 0x7fffu) - TAB_LO;
     t = max(0, min(t, TAB_N - 1));
-    return t + (int)(bf16_bits >> 15) * TAB_N;
+    return t + (int)(bf16_bits >> 15) * TAB_NEG;
+}
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+
+// Two fp32 logits -> their bf16 bit patterns (round to nearest even) packed lo | hi << 16.
+__device__ __forceinline__ uint32_t pack_logits(float a, float b) {
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+// Byte offsets (4 * tab_index) of both packed logits, again packed lo | hi << 16; all 16-bit lane math.
+__device__ __forceinline__ uint32_t tab_offsets2(uint32_t pk) {
+    u16x2_t u = __builtin_bit_cast(u16x2_t, pk);
+    u16x2_t t = __builtin_elementwise_sub_sat(u & (u16x2_t){0x7fff, 0x7fff}, (u16x2_t){TAB_LO, TAB_LO});
+    t = __builtin_elementwise_min(t, (u16x2_t){TAB_N - 1, TAB_N - 1});
+    u16x2_t off = (t << (u16x2_t){2, 2}) | ((u >> (u16x2_t){1, 1}) & (u16x2_t){4 * TAB_NEG, 4 * TAB_NEG});
+    return __builtin_bit_cast(uint32_t, off);
+}
+__device__ __forceinline__ float tab_at(const float* tab, uint32_t byte_off) {
+    return *(const float*)((const uint8_t*)tab + byte_off);
 }
 
 // bf16(sigmoid(l * inv_C + B_div_C)) as an fp32 value; mul and add rounded separately.
@@ -45,7 +67,8 @@ __device__ __forceinline__ float softcap_E(float sigma, const Softcap& sc) { ret
 __global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= TAB_ENTRIES) return;
-    int t = i % TAB_N, neg = i / TAB_N;
+    int t = i % TAB_NEG, neg = i / TAB_NEG;
+    if (t >= TAB_N) { tabE[i] = 0.0f; tabD[i] = 0.0f; return; }   // unused gap
     uint32_t bits = t == 0 ? 0u : (uint32_t)(TAB_LO + t);
     float l = bf16_bits_to_f32(bits | (neg ? 0x8000u : 0u));
     float s = softcap_sigma(l, sc);
@@ -57,6 +80,13 @@ __global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc) {
 __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
+}
+
+// The lookup table of the GEMM-fused kernels lives in static LDS, so its address is a link-time
+// constant that folds into the offset field of every ds_read.
+__device__ __forceinline__ float* lds_table() {
+    __shared__ float table[TAB_ENTRIES];
+    return table;
 }
 
 __device__ __forceinline__ void load_table(float* lds_tab, const float* gtab) {
@@ -201,6 +231,7 @@ struct CEJobIter {
     __device__ bool valid() const { return slot + it * nslots < tiles_m; }
     __device__ int tr() const { return tr_; }
     __device__ int tc() const { return slot + it * nslots; }
+    __device__ bool job_begin() const { return tr_ == tiles_v * split / CE_SPLITS; }
     __device__ bool job_end() const { return tr_ + 1 == tr_end; }
     __device__ int job_id() const { return split; }
     __device__ void advance() {
@@ -211,64 +242,106 @@ struct CEJobIter {
     }
 };
 
+constexpr int CE_MAX_BN = 256;                                  // widest token tile of any config
+constexpr int CAND_LDS_BYTES = MAX_CAND * CE_MAX_BN * 4;
+constexpr int CE_FWD_EXTRA_LDS = (CAND_LDS_BYTES + 1023) / 1024 * 1024;
+
 struct EpiCEFwd {
-    static constexpr int EXTRA_LDS = TAB_BYTES;
+    static constexpr int EXTRA_LDS = CE_FWD_EXTRA_LDS;
     const float* gtabE;
     float* part;          // [CE_SPLITS][M] partial sums of exp(z - A)
     float* saved_sigma;   // [MAX_CAND][M] bf16-rounded sigma at each candidate target column
     CandArgs ca;
     Softcap sc;
     float scale;
-    float* tab;
+    int ncand;            // n_predict (+1 with prefix targets)
+    int* cand;            // LDS: [MAX_CAND][CE_MAX_BN] valid target column of the job's tokens, else -1
     float sum[8];
 
     __device__ void begin(int, int, uint8_t* extra) {
-        tab = (float*)extra;
-        load_table(tab, gtabE);
+        cand = (int*)extra;
+        load_table(lds_table(), gtabE);
 #pragma unroll
         for (int i = 0; i < 8; ++i) sum[i] = 0.0f;
     }
     __device__ void end(uint8_t*, int, int) {}
+
+    // A new (token tile, split) job: stage the candidate target columns of its tokens in LDS.
+    template <class Cfg>
+    __device__ void job_begin(int c0) {
+        static_assert(Cfg::BN <= CE_MAX_BN, "token tile too wide");
+        for (int i = threadIdx.x; i < ncand * Cfg::BN; i += Cfg::THREADS) {
+            int c = i / Cfg::BN, j = i % Cfg::BN;
+            int m = c0 + j;
+            int64_t t = (m < ca.M) ? cand_target(ca, m, c) : -1;
+            cand[c * CE_MAX_BN + j] = (t >= 0 && t < ca.V) ? (int)t : -1;
+        }
+    }
 
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0 /* vocab */, int c0 /* token */,
                          const AccCoords<Cfg>& co, uint8_t*, int lane) {
         static_assert(Cfg::TN <= 8, "per-lane token columns");
         const int V = ca.V, M = ca.M;
-        const bool partial = (r0 + Cfg::BM > V);
+        const float* tab = lds_table();
+        if (r0 + Cfg::BM <= V) {
 #pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm)
+            for (int tn = 0; tn < Cfg::TN; ++tn)
+#pragma unroll
+                for (int tm = 0; tm < Cfg::TM; ++tm) {
+                    float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2) {
+                        uint32_t off = tab_offsets2(pack_logits(acc[tm][tn][v] * scale, acc[tm][tn][v + 1] * scale));
+                        s0 += tab_at(tab, off & 0xffffu);
+                        s1 += tab_at(tab, off >> 16);
+                    }
+                    sum[tn] += s0 + s1;
+                    __builtin_amdgcn_sched_barrier(0);   // keep the table reads of one MFMA tile together
+                }
+        } else {   // last vocabulary tile: rows past V are clamped duplicates and must not count
+#pragma unroll
+            for (int tn = 0; tn < Cfg::TN; ++tn)
+#pragma unroll
+                for (int tm = 0; tm < Cfg::TM; ++tm) {
+                    float s0 = 0.0f;
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2) {
+                        uint32_t off = tab_offsets2(pack_logits(acc[tm][tn][v] * scale, acc[tm][tn][v + 1] * scale));
+                        float e0 = tab_at(tab, off & 0xffffu), e1 = tab_at(tab, off >> 16);
+                        s0 += (r0 + co.row(tm, v) < V) ? e0 : 0.0f;
+                        s0 += (r0 + co.row(tm, v + 1) < V) ? e1 : 0.0f;
+                    }
+                    sum[tn] += s0;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+        }
+        // sigma at candidate target columns that fall inside this wave's vocabulary rows
+        const int v_lo = r0 + co.wave_row0;
+        for (int c = 0; c < ncand; ++c) {
+            int rl[Cfg::TN];
+            bool any_hit = false;
 #pragma unroll
             for (int tn = 0; tn < Cfg::TN; ++tn) {
-                float s = 0.0f;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    float e = tab[tab_index(f32_to_bf16_bits(acc[tm][tn][v] * scale))];
-                    if (partial) e = (r0 + co.row(tm, v) < V) ? e : 0.0f;
-                    s += e;
-                }
-                sum[tn] += s;
+                int d = cand[c * CE_MAX_BN + co.col(tn)] - v_lo;
+                rl[tn] = ((unsigned)d < (unsigned)Cfg::WTM) ? d : -1;
+                any_hit |= rl[tn] >= 0;
             }
-        // sigma at candidate target columns that fall inside this wave's vocabulary rows (rare)
-        const int v_lo = r0 + co.wave_row0, v_hi = v_lo + Cfg::WTM;
+            if (!__any(any_hit)) continue;
 #pragma unroll
-        for (int tn = 0; tn < Cfg::TN; ++tn) {
-            int m = c0 + co.col(tn);
-            for (int c = 0; c <= ca.n_predict; ++c) {
-                int64_t t = (m < M) ? cand_target(ca, m, c) : -1;
-                bool hit = (t >= v_lo && t < v_hi && t < V);
-                if (__any(hit)) {
-                    int rl = hit ? (int)t - v_lo : -1;
-                    float got = 0.0f;
-                    bool mine = false;
+            for (int tn = 0; tn < Cfg::TN; ++tn) {
+                if (!__any(rl[tn] >= 0)) continue;
+                float got = 0.0f;
+                bool mine = false;
 #pragma unroll
-                    for (int tm = 0; tm < Cfg::TM; ++tm)
+                for (int tm = 0; tm < Cfg::TM; ++tm)
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            int r = co.row(tm, v) - co.wave_row0;
-                            if (r == rl) { got = acc[tm][tn][v]; mine = true; }
-                        }
-                    if (mine) saved_sigma[(int64_t)c * M + m] = softcap_sigma(round_to_bf16(got * scale), sc);
+                    for (int v = 0; v < 16; ++v)
+                        if (co.row(tm, v) - co.wave_row0 == rl[tn]) { got = acc[tm][tn][v]; mine = true; }
+                int m = c0 + co.col(tn);
+                if (mine && m < M) {
+                    float l = bf16_bits_to_f32(pack_logits(got * scale, 0.0f) & 0xffffu);
+                    saved_sigma[(int64_t)c * M + m] = softcap_sigma(l, sc);
                 }
             }
         }
@@ -325,19 +398,17 @@ __global__ void ce_rowf_kernel(const float* __restrict__ lse, CandArgs ca, Softc
 // GEMM orientation: rows = tokens of the current chunk (A = x_f8), columns = vocabulary (B = w_f8).
 // Writes the e5m2 dlogits of the chunk row-major (dl [Mc, V]) and transposed (dl_t [V, Mc]).
 struct EpiDlStore {
-    static constexpr int EXTRA_LDS = TAB_BYTES;
+    static constexpr int EXTRA_LDS = 0;
+    template <class Cfg>
+    __device__ void job_begin(int) {}
     const float* gtabD;
     const float* rowf;     // already offset to the chunk's first row
     uint8_t* dl;           // [Mc, V]
     uint8_t* dl_t;         // [V, Mc]
     int Mc, V;
     float scale;
-    float* tab;
 
-    __device__ void begin(int, int, uint8_t* extra) {
-        tab = (float*)extra;
-        load_table(tab, gtabD);
-    }
+    __device__ void begin(int, int, uint8_t*) { load_table(lds_table(), gtabD); }
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
     __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
@@ -346,6 +417,7 @@ struct EpiDlStore {
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t* scratch, int lane) {
         const int h = lane >> 5;
+        const float* tab = lds_table();
         uint32_t pk[Cfg::TM][Cfg::TN][4];
 #pragma unroll
         for (int tm = 0; tm < Cfg::TM; ++tm)
@@ -355,11 +427,11 @@ struct EpiDlStore {
                 v4f rf = (row + 4 <= Mc) ? *(const v4f*)(rowf + row) : (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int tn = 0; tn < Cfg::TN; ++tn) {
-                    float d[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        d[i] = rf[i] * tab[tab_index(f32_to_bf16_bits(acc[tm][tn][4 * g + i] * scale))];
-                    pk[tm][tn][g] = f32x4_to_e5m2_sat(d[0], d[1], d[2], d[3]);
+                    const v16f& a = acc[tm][tn];
+                    uint32_t o01 = tab_offsets2(pack_logits(a[4 * g] * scale, a[4 * g + 1] * scale));
+                    uint32_t o23 = tab_offsets2(pack_logits(a[4 * g + 2] * scale, a[4 * g + 3] * scale));
+                    pk[tm][tn][g] = f32x4_to_e5m2_sat(rf[0] * tab_at(tab, o01 & 0xffffu), rf[1] * tab_at(tab, o01 >> 16),
+                                                      rf[2] * tab_at(tab, o23 & 0xffffu), rf[3] * tab_at(tab, o23 >> 16));
                 }
             }
         // row-major copy: one 32-row strip per tm
@@ -524,8 +596,9 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
     epi.ca = CandArgs{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
     epi.sc = sc;
     epi.scale = x_s * w_s;
+    epi.ncand = prefix_targets ? n_predict + 1 : n_predict;
     auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, EpiCEFwd, CEJobIter>;
-    constexpr int LDS = Cfg::SMEM_BYTES + EpiCEFwd::EXTRA_LDS;
+    constexpr int LDS = Cfg::SMEM_BYTES + EpiCEFwd::EXTRA_LDS;   // dynamic part; the table is static LDS
     static bool configured = false;
     if (!configured) {
         if (int e = allow_lds(kernel, LDS)) return e;

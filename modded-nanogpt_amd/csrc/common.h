@@ -104,6 +104,4 @@ __device__ __forceinline__ void global_to_lds16(const void* gptr, void* lds_wave
         (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
-__device__ __forceinline__ void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
 }  // namespace ngpt

@@ -77,6 +77,8 @@ struct EpiStoreBf16 {
     __device__ void begin(int, int, uint8_t*) {}
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
+    __device__ void job_begin(int) {}
+    template <class Cfg>
     __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
@@ -95,6 +97,29 @@ struct EpiStoreBf16 {
     }
 };
 
+// Mainloop-only timing aid: keeps the accumulators alive but writes (practically) nothing.
+struct EpiDiscard {
+    float* out;
+    static constexpr int EXTRA_LDS = 0;
+    __device__ void begin(int, int, uint8_t*) {}
+    __device__ void end(uint8_t*, int, int) {}
+    template <class Cfg>
+    __device__ void job_begin(int) {}
+    template <class Cfg>
+    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int, int, const AccCoords<Cfg>&, uint8_t*, int) {
+        float s = 0.0f;
+#pragma unroll
+        for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < Cfg::TN; ++tn)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s += acc[tm][tn][v];
+        if (s == 1.2345678e30f) out[0] = s;
+    }
+};
+
 // out[r, c] (+)= acc * scale in fp32
 struct EpiStoreF32 {
     float* out;
@@ -105,6 +130,8 @@ struct EpiStoreF32 {
     static constexpr int EXTRA_LDS = 0;
     __device__ void begin(int, int, uint8_t*) {}
     __device__ void end(uint8_t*, int, int) {}
+    template <class Cfg>
+    __device__ void job_begin(int) {}
     template <class Cfg>
     __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
     template <class Cfg>
@@ -142,6 +169,8 @@ struct EpiRelu2 {
     int R, C;
     float scale, inv_act, amax;
     static constexpr int EXTRA_LDS = 0;
+    template <class Cfg>
+    __device__ void job_begin(int) {}
     template <class Cfg>
     __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
     __device__ void begin(int, int, uint8_t*) {

@@ -72,6 +72,8 @@ static int check_gemm_dims(const char* who, int R, int C, int K, int64_t lda, in
     return NGPT_OK;
 }
 
+int g_tuning[8] = {0, 1, 0, 0, 0, 0, 0, 0};
+
 // Which profile slot the next gemm_store launches are booked under (set by the fused CE backward).
 int g_gemm_slot = PROF_GEMM;
 
@@ -82,6 +84,10 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
     ProfileScope prof(g_gemm_slot, st);
     if (out_kind == 0) {
         EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C};
+        return launch_gemm<MainCfg>(g, fa, fb, epi, st);
+    }
+    if (out_kind == 3) {
+        EpiDiscard epi{(float*)out};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
     EpiStoreF32 epi{(float*)out, ldc, scale, R, C, out_kind == 2};
@@ -95,6 +101,12 @@ using namespace ngpt;
 extern "C" int ngpt_abi_version(void) { return 1; }
 extern "C" const char* ngpt_last_error(void) { return last_error_buf(); }
 extern "C" int ngpt_num_cus(void) { return num_cus(); }
+
+extern "C" int ngpt_tuning_set(int key, int value) {
+    if (key < 0 || key >= 8) return fail(NGPT_EINVAL, "ngpt_tuning_set: key=%d", key);
+    g_tuning[key] = value;
+    return NGPT_OK;
+}
 
 extern "C" int ngpt_profile_enable(int on) {
     std::lock_guard<std::mutex> lk(g_prof_mu);
@@ -130,7 +142,7 @@ extern "C" int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const voi
                                 void* stream) {
     if (!A || !B || !out) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: null pointer");
     if ((fmt_a | fmt_b) & ~1) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: fmt_a=%d fmt_b=%d", fmt_a, fmt_b);
-    if (out_kind < 0 || out_kind > 2) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: out_kind=%d", out_kind);
+    if (out_kind < 0 || out_kind > 3) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: out_kind=%d", out_kind);
     if (ldc < C) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: ldc=%lld < C=%d", (long long)ldc, C);
     return gemm_store(A, fmt_a, lda, B, fmt_b, ldb, R, C, K, scale, out, ldc, out_kind, (hipStream_t)stream);
 }

@@ -32,22 +32,32 @@ struct GemmOperands {
     int R, C, K;        // K % 128 == 0
 };
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2>
 struct TileCfg {
-    static constexpr int BM = BM_, BN = BN_, BK = 128;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, NSTAGES = NSTAGES_;
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int NWAVES = WAVES_M * WAVES_N;
     static constexpr int THREADS = NWAVES * 64;
     static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;   // wave tile
     static constexpr int TM = WTM / 32, TN = WTN / 32;             // MFMA tiles per wave
+    static constexpr int KSUB = BK / 64;                           // 64-byte MFMA contraction steps per k-step
+    static constexpr int CPR = BK / 16;                            // 16-byte chunks per LDS row
+    static constexpr int RPB = 256 / BK;                           // LDS rows per 256-byte bank row
+    static constexpr int ROWS_PER_LOAD = 1024 / BK;                // rows one wave-level 1 KiB load covers
     static constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    static constexpr int SMEM_BYTES = 2 * STAGE_BYTES;
-    static constexpr int A_LOADS = BM / 8 / NWAVES;                // wave-level 1 KiB loads per k-step
-    static constexpr int B_LOADS = BN / 8 / NWAVES;
+    static constexpr int SMEM_BYTES = NSTAGES * STAGE_BYTES;
+    static constexpr int A_LOADS = BM / ROWS_PER_LOAD / NWAVES;    // wave-level loads per k-step
+    static constexpr int B_LOADS = BN / ROWS_PER_LOAD / NWAVES;
+    static constexpr int LOADS = A_LOADS + B_LOADS;
     static constexpr int WAVE_SCRATCH = STAGE_BYTES / NWAVES;      // epilogue staging per wave
-    static_assert(BM % (8 * NWAVES) == 0 && BN % (8 * NWAVES) == 0, "tile rows must split over waves");
+    static_assert(BK == 64 || BK == 128, "BK is 64 or 128 bytes");
+    static_assert(NSTAGES >= 2 && NSTAGES <= 4, "2..4 LDS stages");
+    static_assert(BM % (ROWS_PER_LOAD * NWAVES) == 0 && BN % (ROWS_PER_LOAD * NWAVES) == 0,
+                  "tile rows must split over waves");
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be made of 32x32 MFMA tiles");
+    // LDS swizzle: chunk q of row r is stored at chunk position q ^ swz(r)
+    static __device__ __forceinline__ int swz(int r) { return (r / RPB) % CPR; }
 };
 
 // Tile order: groups of 4 tile-rows, column-major inside a group, so 32 consecutive sequence
@@ -76,11 +86,18 @@ struct TileOrder {
     }
 };
 
+template <int N>
+__device__ __forceinline__ void wait_vmem_le() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
 template <class Cfg, int AFMT, int BFMT>
 struct TileMainloop {
     const uint8_t* a_ptr[Cfg::A_LOADS];
     const uint8_t* b_ptr[Cfg::B_LOADS];
-    int frag_a[Cfg::TM];     // LDS byte offset of this lane's first 16-byte chunk, stage 0, ks 0
+    int frag_a[Cfg::TM];     // LDS byte offset of this lane's first 16-byte chunk, stage 0, ksub 0
     int frag_b[Cfg::TN];
     int wave, lane, wr, wc;
 
@@ -94,30 +111,30 @@ struct TileMainloop {
 #pragma unroll
         for (int t = 0; t < Cfg::TM; ++t) {
             int row = wr * Cfg::WTM + t * 32 + (lane & 31);
-            frag_a[t] = row * 128 + ((((h * 2) ^ (row >> 1)) & 7) << 4);
+            frag_a[t] = row * Cfg::BK + (((h * 2) ^ Cfg::swz(row)) << 4);
         }
 #pragma unroll
         for (int t = 0; t < Cfg::TN; ++t) {
             int row = wc * Cfg::WTN + t * 32 + (lane & 31);
-            frag_b[t] = Cfg::A_BYTES + row * 128 + ((((h * 2) ^ (row >> 1)) & 7) << 4);
+            frag_b[t] = Cfg::A_BYTES + row * Cfg::BK + (((h * 2) ^ Cfg::swz(row)) << 4);
         }
     }
 
     // Point the per-lane global pointers at tile (r0, c0).  Rows past the end are clamped to the
     // last row: they are loaded (valid memory) and their results discarded by the epilogue.
     __device__ void set_tile(const GemmOperands& g, int r0, int c0) {
-        int lrow = lane >> 3, lchunk = lane & 7;
+        int lrow = lane / Cfg::CPR, lchunk = lane % Cfg::CPR;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i) {
-            int R = (wave + i * Cfg::NWAVES) * 8 + lrow;
-            int q = lchunk ^ ((R >> 1) & 7);
+            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
+            int q = lchunk ^ Cfg::swz(R);
             int gr = min(r0 + R, g.R - 1);
             a_ptr[i] = g.A + (int64_t)gr * g.lda + q * 16;
         }
 #pragma unroll
         for (int i = 0; i < Cfg::B_LOADS; ++i) {
-            int R = (wave + i * Cfg::NWAVES) * 8 + lrow;
-            int q = lchunk ^ ((R >> 1) & 7);
+            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
+            int q = lchunk ^ Cfg::swz(R);
             int gc = min(c0 + R, g.C - 1);
             b_ptr[i] = g.B + (int64_t)gc * g.ldb + q * 16;
         }
@@ -137,7 +154,7 @@ struct TileMainloop {
     __device__ void compute(const uint8_t* smem, int stage, v16f (&acc)[Cfg::TM][Cfg::TN]) {
         const uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        for (int ks = 0; ks < Cfg::KSUB; ++ks) {
             v8i a[Cfg::TM], b[Cfg::TN];
 #pragma unroll
             for (int t = 0; t < Cfg::TM; ++t) {
@@ -187,6 +204,7 @@ struct GridIter {
     __device__ bool valid() const { return seq < order.total; }
     __device__ int tr() const { return tr_; }
     __device__ int tc() const { return tc_; }
+    __device__ bool job_begin() const { return false; }
     __device__ bool job_end() const { return false; }
     __device__ int job_id() const { return 0; }
     __device__ void advance() {
@@ -199,25 +217,57 @@ struct GridIter {
 // The generic persistent kernel.  `Iter` walks the tiles of this workgroup (see GridIter).  `Epi` supplies
 //   void begin(int bid, int nblocks)
 //   void tile(acc, r0, c0, coords, scratch /* wave-private LDS */, lane)
-//   void job_end(c0, job_id, coords, stage_scratch /* whole free LDS stage */)   -- only if Iter reports job ends
+//   void job_begin(c0) / job_end(c0, job_id, coords, stage_scratch /* whole free LDS stage */)
+//                                                              -- only if Iter reports job boundaries
 //   void end(uint8_t* smem, int bid, int nblocks)
 // `tile` runs after a workgroup barrier, so the just-consumed LDS stage is free for staging.
-// Dynamic LDS: Cfg::SMEM_BYTES for the two operand stages, then Epi::EXTRA_LDS bytes that the
-// epilogue owns for the whole kernel (lookup tables).
+// Dynamic LDS: Epi::EXTRA_LDS bytes that the epilogue owns for the whole kernel (lookup tables; at
+// offset 0 so their addresses fit the 16-bit offset field of LDS instructions), then
+// Cfg::SMEM_BYTES for the operand stages.
+// Walks (tile, k-step) pairs of one workgroup as one flat sequence, so the software pipeline of
+// operand loads runs ahead across tile boundaries.
+template <class Iter>
+struct StepCursor {
+    Iter it;
+    int kt;
+    __device__ StepCursor(const Iter& i) : it(i), kt(0) {}
+    __device__ bool valid() const { return it.valid(); }
+    __device__ void advance(int nk) {
+        if (++kt == nk) {
+            kt = 0;
+            it.advance();
+        }
+    }
+};
+
 template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
 __global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel(GemmOperands g, Epi epi) {
-    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem_all[];
+    static_assert(Epi::EXTRA_LDS % 1024 == 0, "epilogue LDS must keep the stages 1 KiB aligned");
+    uint8_t* const smem = smem_all + Epi::EXTRA_LDS;      // operand stages
+    constexpr int NS = Cfg::NSTAGES;
     TileMainloop<Cfg, AFMT, BFMT> ml;
     ml.init();
     const int bid = blockIdx.x, G = gridDim.x;
     const int nk = g.K / Cfg::BK;
     AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane);
     Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
-    if (cur.valid()) {
-        ml.set_tile(g, cur.tr() * Cfg::BM, cur.tc() * Cfg::BN);
-        ml.issue_loads(smem, 0, 0);
+
+    // prologue: put NS-1 k-steps in flight
+    StepCursor<Iter> pre(cur);
+    int pre_slot = 0;
+    bool pre_new_tile = true;
+#pragma unroll
+    for (int i = 0; i < NS - 1; ++i) {
+        if (pre.valid()) {
+            if (pre_new_tile) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
+            ml.issue_loads(smem, pre_slot, pre.kt);
+            pre.advance(nk);
+            pre_new_tile = (pre.kt == 0);
+        }
+        pre_slot = (pre_slot + 1 == NS) ? 0 : pre_slot + 1;
     }
-    epi.begin(bid, G, smem + Cfg::SMEM_BYTES);
+    epi.begin(bid, G, smem_all);
 
     v16f acc[Cfg::TM][Cfg::TN];
 #pragma unroll
@@ -227,26 +277,32 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel(GemmOperands g, E
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    int stage = 0;
+    int slot = 0;
     while (cur.valid()) {
         const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
-        Iter nxt = cur;
-        nxt.advance();
+        if (cur.job_begin()) epi.template job_begin<Cfg>(c0);   // made visible by the k-loop's barriers
         for (int kt = 0; kt < nk; ++kt) {
-            wait_vmem_all();
+            // The loads of this k-step are the oldest loads in flight and loads retire in order, so it
+            // is enough that at most the NS-2 newer load groups remain outstanding.  Stores issued by
+            // an epilogue share the counter and may retire in any order relative to loads; they only
+            // make this wait stricter, never too weak.  Near the end of the walk fewer groups were
+            // issued, so wait for everything.
+            if (pre.valid()) wait_vmem_le<(NS - 2) * Cfg::LOADS>();
+            else wait_vmem_le<0>();
             __syncthreads();
-            // prefetch the next k-step (possibly the first one of the next tile)
-            if (kt + 1 < nk) {
-                ml.issue_loads(smem, stage ^ 1, kt + 1);
-            } else if (nxt.valid()) {
-                ml.set_tile(g, nxt.tr() * Cfg::BM, nxt.tc() * Cfg::BN);
-                ml.issue_loads(smem, stage ^ 1, 0);
+            // refill the slot consumed in the previous step with the k-step NS-1 ahead
+            if (pre.valid()) {
+                if (pre_new_tile) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
+                ml.issue_loads(smem, pre_slot, pre.kt);
+                pre.advance(nk);
+                pre_new_tile = (pre.kt == 0);
+                pre_slot = (pre_slot + 1 == NS) ? 0 : pre_slot + 1;
             }
-            ml.compute(smem, stage, acc);
-            stage ^= 1;
+            ml.compute(smem, slot, acc);
+            slot = (slot + 1 == NS) ? 0 : slot + 1;
         }
-        __syncthreads();   // every wave is done reading the last stage: reuse it as scratch
-        uint8_t* free_stage = smem + (stage ^ 1) * Cfg::STAGE_BYTES;
+        __syncthreads();   // every wave is done reading the last slot: reuse it as scratch
+        uint8_t* free_stage = smem + (slot == 0 ? NS - 1 : slot - 1) * Cfg::STAGE_BYTES;
         epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
         if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
 #pragma unroll
@@ -255,7 +311,7 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel(GemmOperands g, E
             for (int j = 0; j < Cfg::TN; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-        cur = nxt;
+        cur.advance();
     }
     __syncthreads();
     epi.end(smem, bid, G);

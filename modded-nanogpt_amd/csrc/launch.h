@@ -6,7 +6,15 @@
 namespace ngpt {
 
 // 256 x 256 tile, 8 waves as 4 (rows) x 2 (cols): each wave owns 64 x 128 = 2 x 4 MFMA tiles.
-using MainCfg = TileCfg<256, 256, 4, 2>;
+using MainCfg = TileCfg<256, 256, 4, 2, 128, 2>;
+// Alternatives selectable at run time through ngpt_tuning_set(0, id) (tuning aid).
+using Cfg256x256k64s4 = TileCfg<256, 256, 4, 2, 64, 4>;     // id 1: four 32 KiB stages
+using Cfg256x128k64s3 = TileCfg<256, 128, 2, 2, 64, 3>;     // id 2: 4 waves, 72 KiB: two workgroups per CU
+using Cfg256x128k128s2 = TileCfg<256, 128, 2, 2, 128, 2>;   // id 3: 4 waves, 96 KiB
+using Cfg128x128k128s2 = TileCfg<128, 128, 2, 2, 128, 2>;   // id 4: 4 waves, 64 KiB: two workgroups per CU
+using Cfg256x128k64s2 = TileCfg<256, 128, 2, 2, 64, 2>;     // id 5: 4 waves, 48 KiB: three workgroups per CU
+
+extern int g_tuning[8];   // [0] GEMM tile config id, [1] workgroups per CU for the persistent grid
 
 template <class Cfg, int FA, int FB, class Epi>
 int launch_gemm_fmt(const GemmOperands& g, const Epi& epi, hipStream_t st, int max_grid) {
@@ -20,18 +28,34 @@ int launch_gemm_fmt(const GemmOperands& g, const Epi& epi, hipStream_t st, int m
     int tiles = ((g.R + Cfg::BM - 1) / Cfg::BM) * ((g.C + Cfg::BN - 1) / Cfg::BN);
     int cus = num_cus();
     if (cus <= 0) return fail(NGPT_EINVAL, "no HIP device");
-    int grid = tiles < cus ? tiles : cus;
+    int per_cu = g_tuning[1] > 0 ? g_tuning[1] : 1;
+    if ((int64_t)per_cu * (Cfg::SMEM_BYTES + Epi::EXTRA_LDS) > 160 * 1024) per_cu = 1;
+    int slots = cus * per_cu;
+    int grid = tiles < slots ? tiles : slots;
     if (max_grid > 0 && grid > max_grid) grid = max_grid;
     kernel<<<grid, Cfg::THREADS, LDS, st>>>(g, epi);
     return check_launch("gemm_tn_kernel");
 }
 
 template <class Cfg, class Epi>
-int launch_gemm(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {
+int launch_gemm_cfg(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {
     if (fa == FMT_E4M3 && fb == FMT_E4M3) return launch_gemm_fmt<Cfg, FMT_E4M3, FMT_E4M3>(g, epi, st, max_grid);
     if (fa == FMT_E5M2 && fb == FMT_E4M3) return launch_gemm_fmt<Cfg, FMT_E5M2, FMT_E4M3>(g, epi, st, max_grid);
     if (fa == FMT_E4M3 && fb == FMT_E5M2) return launch_gemm_fmt<Cfg, FMT_E4M3, FMT_E5M2>(g, epi, st, max_grid);
     return launch_gemm_fmt<Cfg, FMT_E5M2, FMT_E5M2>(g, epi, st, max_grid);
+}
+
+// Dispatch on the run-time tile configuration (default MainCfg).
+template <class Cfg /* default */, class Epi>
+int launch_gemm(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {
+    switch (g_tuning[0]) {
+        case 1: return launch_gemm_cfg<Cfg256x256k64s4>(g, fa, fb, epi, st, max_grid);
+        case 2: return launch_gemm_cfg<Cfg256x128k64s3>(g, fa, fb, epi, st, max_grid);
+        case 3: return launch_gemm_cfg<Cfg256x128k128s2>(g, fa, fb, epi, st, max_grid);
+        case 4: return launch_gemm_cfg<Cfg128x128k128s2>(g, fa, fb, epi, st, max_grid);
+        case 5: return launch_gemm_cfg<Cfg256x128k64s2>(g, fa, fb, epi, st, max_grid);
+        default: return launch_gemm_cfg<Cfg>(g, fa, fb, epi, st, max_grid);
+    }
 }
 
 }  // namespace ngpt
