@@ -231,6 +231,8 @@ struct CEJobIter {
     __device__ bool valid() const { return slot + it * nslots < tiles_m; }
     __device__ int tr() const { return tr_; }
     __device__ int tc() const { return slot + it * nslots; }
+    __device__ int kt_begin(int) const { return 0; }
+    __device__ int kt_end(int nk) const { return nk; }
     __device__ bool job_begin() const { return tr_ == tiles_v * split / CE_SPLITS; }
     __device__ bool job_end() const { return tr_ + 1 == tr_end; }
     __device__ int job_id() const { return split; }
@@ -248,6 +250,8 @@ constexpr int CE_FWD_EXTRA_LDS = (CAND_LDS_BYTES + 1023) / 1024 * 1024;
 
 struct EpiCEFwd {
     static constexpr int EXTRA_LDS = CE_FWD_EXTRA_LDS;
+    static constexpr bool NEEDS_SCRATCH = false;
+    static constexpr bool JOB_END_NEEDS_SCRATCH = true;    // job_end reduces through the stage
     const float* gtabE;
     float* part;          // [CE_SPLITS][M] partial sums of exp(z - A)
     float* saved_sigma;   // [MAX_CAND][M] bf16-rounded sigma at each candidate target column
@@ -359,7 +363,7 @@ struct EpiCEFwd {
             if (lane < 32) red[wr * Cfg::BN + co.col(tn)] = s;
             sum[tn] = 0.0f;
         }
-        __syncthreads();
+        wg_barrier();
         for (int j = threadIdx.x; j < Cfg::BN; j += Cfg::THREADS) {
             float s = 0.0f;
 #pragma unroll
@@ -399,6 +403,8 @@ __global__ void ce_rowf_kernel(const float* __restrict__ lse, CandArgs ca, Softc
 // Writes the e5m2 dlogits of the chunk row-major (dl [Mc, V]) and transposed (dl_t [V, Mc]).
 struct EpiDlStore {
     static constexpr int EXTRA_LDS = 0;
+    static constexpr bool NEEDS_SCRATCH = true;
+    static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     template <class Cfg>
     __device__ void job_begin(int) {}
     const float* gtabD;
@@ -484,7 +490,17 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
 }
 
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
-               float scale, void* out, int64_t ldc, int out_kind, hipStream_t st);
+               float scale, void* out, int64_t ldc, int out_kind, hipStream_t st, int splits);
+int pick_splits(int tiles, int ksteps);
+
+// out[i] = bf16(in[i]), eight elements per thread
+__global__ void f32_to_bf16_kernel(const float* __restrict__ in, uint16_t* __restrict__ out, int64_t n8) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    v4f a = *(const v4f*)(in + i * 8), b = *(const v4f*)(in + i * 8 + 4);
+    v4i o = {(int)cvt_pk_bf16(a[0], a[1]), (int)cvt_pk_bf16(a[2], a[3]), (int)cvt_pk_bf16(b[0], b[1]), (int)cvt_pk_bf16(b[2], b[3])};
+    *(v4i*)(out + i * 8) = o;
+}
 extern int g_gemm_slot;
 struct GemmSlot {   // books the plain GEMM launches inside a scope under a CE profile slot
     int saved;
@@ -509,6 +525,49 @@ static int check_cand(const char* who, const int64_t* targets, const float* mtp_
     if (n_predict < 1 || n_predict > NGPT_MAX_PREDICT)
         return fail(NGPT_ERANGE, "%s: n_predict=%d outside [1, %d]", who, n_predict, NGPT_MAX_PREDICT);
     return NGPT_OK;
+}
+
+// One launch of the fused forward kernel for tile configuration Cfg.
+template <class Cfg>
+static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwd& epi, hipStream_t st) {
+    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, EpiCEFwd, CEJobIter>;
+    constexpr int LDS = Cfg::SMEM_BYTES + EpiCEFwd::EXTRA_LDS;   // dynamic part; the table is static LDS
+    static bool configured = false;
+    if (!configured) {
+        if (int e = allow_lds(kernel, LDS)) return e;
+        configured = true;
+    }
+    int cus = num_cus();
+    if (cus < CE_SPLITS) return fail(NGPT_EINVAL, "no HIP device");
+    int tiles_m = (g.C + Cfg::BN - 1) / Cfg::BN;
+    int slots_max = cus * Cfg::WGS_PER_CU / CE_SPLITS;
+    int slots = slots_max < tiles_m ? slots_max : tiles_m;
+    {
+        ProfileScope prof(PROF_CE_FWD, st);
+        kernel<<<slots * CE_SPLITS, Cfg::THREADS, LDS, st>>>(g, epi);
+    }
+    return check_launch("lm_head CE forward");
+}
+
+template <class Cfg, class Epi>
+static int launch_grid_kernel(const GemmOperands& g, const Epi& epi, hipStream_t st, int slot, const char* what) {
+    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, Epi, GridIter>;
+    constexpr int LDS = Cfg::SMEM_BYTES + Epi::EXTRA_LDS;
+    static bool configured = false;
+    if (!configured) {
+        if (int e = allow_lds(kernel, LDS)) return e;
+        configured = true;
+    }
+    const int cus = num_cus();
+    if (cus <= 0) return fail(NGPT_EINVAL, "no HIP device");
+    int tiles = ((g.R + Cfg::BM - 1) / Cfg::BM) * ((g.C + Cfg::BN - 1) / Cfg::BN);
+    int per_cu = Cfg::WGS_PER_CU > 1 ? Cfg::WGS_PER_CU : 1;
+    int grid = tiles < cus * per_cu ? tiles : cus * per_cu;
+    {
+        ProfileScope prof(slot, st);
+        kernel<<<grid, Cfg::THREADS, LDS, st>>>(g, epi);
+    }
+    return check_launch(what);
 }
 
 constexpr int BWD_CHUNK_ROWS = 16384;
@@ -587,8 +646,7 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
         if (int e = ngpt_quant_fp8_2d(w_bf16, K, V, w_s, NGPT_FMT_E4M3, nullptr, w_f8_vk, stream)) return e;
     }
 
-    using Cfg = MainCfg;
-    GemmOperands g{(const uint8_t*)w_f8_vk, (const uint8_t*)x_f8, K, K, V, M, K};
+    GemmOperands g{(const uint8_t*)w_f8_vk, (const uint8_t*)x_f8, K, K, V, M, K, 1, 0};
     EpiCEFwd epi{};
     epi.gtabE = tabE;
     epi.part = part;
@@ -597,33 +655,18 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
     epi.sc = sc;
     epi.scale = x_s * w_s;
     epi.ncand = prefix_targets ? n_predict + 1 : n_predict;
-    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, EpiCEFwd, CEJobIter>;
-    constexpr int LDS = Cfg::SMEM_BYTES + EpiCEFwd::EXTRA_LDS;   // dynamic part; the table is static LDS
-    static bool configured = false;
-    if (!configured) {
-        if (int e = allow_lds(kernel, LDS)) return e;
-        configured = true;
-    }
-    int cus = num_cus();
-    if (cus < CE_SPLITS) return fail(NGPT_EINVAL, "no HIP device");
-    int tiles_m = (M + Cfg::BN - 1) / Cfg::BN;
-    int slots = cus / CE_SPLITS < tiles_m ? cus / CE_SPLITS : tiles_m;
-    {
-        ProfileScope prof(PROF_CE_FWD, st);
-        kernel<<<slots * CE_SPLITS, Cfg::THREADS, LDS, st>>>(g, epi);
-    }
-    if (int e = check_launch("lm_head CE forward")) return e;
+    if (int e = g_tuning[5] ? launch_ce_fwd<Cfg256x128k64s2>(g, epi, st) : launch_ce_fwd<MainCfg>(g, epi, st)) return e;
     ce_finalize_kernel<<<(M + 255) / 256, 256, 0, st>>>(part, saved_sigma, epi.ca, sc, losses, lse);
     return check_launch("ce_finalize_kernel");
 }
 
 // ------------------------------------------------------------------------------------------------
-// backward workspace: tabE | tabD | rowf [M] | x_f8^T [K, M] | w_f8^T [K, V] | dl [Mc, V] | dl^T [V, Mc]
+// backward workspace: tabE | tabD | rowf [M] | x_f8^T [K, M] | w_f8^T [K, V] | dl [Mc, V] | dl^T [V, Mc] | dx fp32 [Mc, K]
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
     int64_t Mc = bwd_chunk_rows(M);
     return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)M * 4, 256) + align_up((int64_t)K * M, 256) +
-           align_up((int64_t)K * V, 256) + 2 * align_up(Mc * V, 256);
+           align_up((int64_t)K * V, 256) + 2 * align_up(Mc * V, 256) + align_up(Mc * K * 4, 256);
 }
 
 extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const int64_t* targets,
@@ -658,6 +701,8 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     uint8_t* dl = ws;
     ws += align_up((int64_t)Mc_max * V, 256);
     uint8_t* dl_t = ws;
+    ws += align_up((int64_t)Mc_max * V, 256);
+    float* dx32 = (float*)ws;
 
     Softcap sc = make_softcap(A, B, C);
     const float coef = make_coef(A, C, grad_s, grad_scale);
@@ -667,21 +712,14 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     if (int e = check_launch("ce_rowf_kernel")) return e;
     if (int e = ngpt_transpose_u8(x_f8, M, K, x_t, stream)) return e;
     if (int e = ngpt_transpose_u8(w_f8_vk, V, K, w_t, stream)) return e;
+    const bool split_k = g_tuning[6] != 0;
+    if (split_k) fill_f32_kernel<<<(int)(((int64_t)V * K + 255) / 256), 256, 0, st>>>((float*)dw_f32, (int64_t)V * K, 0.0f);
 
     using Cfg = MainCfg;
-    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, EpiDlStore, GridIter>;
-    constexpr int LDS = Cfg::SMEM_BYTES + EpiDlStore::EXTRA_LDS;
-    static bool configured = false;
-    if (!configured) {
-        if (int e = allow_lds(kernel, LDS)) return e;
-        configured = true;
-    }
-    const int cus = num_cus();
-    if (cus <= 0) return fail(NGPT_EINVAL, "no HIP device");
     for (int m0 = 0; m0 < M; m0 += Mc_max) {
         const int Mc = (M - m0 < Mc_max) ? (M - m0) : Mc_max;
         // 1. recompute the chunk's logits and turn them into e5m2 dlogits (both layouts)
-        GemmOperands g{(const uint8_t*)x_f8 + (int64_t)m0 * K, (const uint8_t*)w_f8_vk, K, K, Mc, V, K};
+        GemmOperands g{(const uint8_t*)x_f8 + (int64_t)m0 * K, (const uint8_t*)w_f8_vk, K, K, Mc, V, K, 1, 0};
         EpiDlStore epi{};
         epi.gtabD = tabD;
         epi.rowf = rowf + m0;
@@ -690,30 +728,40 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         epi.Mc = Mc;
         epi.V = V;
         epi.scale = x_s * w_s;
-        int tiles = ((Mc + Cfg::BM - 1) / Cfg::BM) * ((V + Cfg::BN - 1) / Cfg::BN);
-        {
-            ProfileScope prof(PROF_CE_DLOGITS, st);
-            kernel<<<tiles < cus ? tiles : cus, Cfg::THREADS, LDS, st>>>(g, epi);
-        }
-        if (int e = check_launch("lm_head CE backward (dlogits)")) return e;
+        if (int e = g_tuning[5] ? launch_grid_kernel<Cfg256x128k64s2>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")
+                                : launch_grid_kernel<MainCfg>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
         ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, dl, dl_t);
         if (int e = check_launch("ce_dl_fix_kernel")) return e;
-        // 3. dx[chunk] = dl [Mc, V] . (w^T [K, V])^T
+        // 3. dx[chunk] = dl [Mc, V] . (w^T [K, V])^T.  The output has only K/256 tile columns, so the
+        //    contraction over V is split across jobs that add into an fp32 staging buffer.
         {
             GemmSlot slot(PROF_CE_DX);
-            if (int e = gemm_store(dl, FMT_E5M2, V, w_t, FMT_E4M3, V, Mc, K, V, grad_s * w_s,
-                                   (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, 0, st)) return e;
+            const int tiles = ((Mc + Cfg::BM - 1) / Cfg::BM) * ((K + Cfg::BN - 1) / Cfg::BN);
+            const int splits = pick_splits(tiles, V / Cfg::BK);
+            if (splits > 1) {
+                fill_f32_kernel<<<(int)(((int64_t)Mc * K + 255) / 256), 256, 0, st>>>(dx32, (int64_t)Mc * K, 0.0f);
+                if (int e = gemm_store(dl, FMT_E5M2, V, w_t, FMT_E4M3, V, Mc, K, V, grad_s * w_s, dx32, K, 2, st, splits)) return e;
+                int64_t n8 = (int64_t)Mc * K / 8;
+                f32_to_bf16_kernel<<<(int)((n8 + 255) / 256), 256, 0, st>>>(dx32, (uint16_t*)dx_bf16 + (int64_t)m0 * K, n8);
+                if (int e = check_launch("f32_to_bf16_kernel")) return e;
+            } else {
+                if (int e = gemm_store(dl, FMT_E5M2, V, w_t, FMT_E4M3, V, Mc, K, V, grad_s * w_s,
+                                       (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, 0, st, 1)) return e;
+            }
         }
-        // 4. dw += over the chunk's tokens
+        // 4. dw: the first chunk stores, later chunks add (fp32 atomics); with split-K every chunk adds
+        //    into the zeroed output
         GemmSlot slot(PROF_CE_DW);
-        const int kind = m0 == 0 ? 1 : 2;
+        const int kind = (split_k || m0 > 0) ? 2 : 1;
         if (w_layout == NGPT_W_OUT_IN) {   // dw [V, K] = dl^T [V, Mc] . (x^T [K, Mc])^T
+            const int tiles = ((V + Cfg::BM - 1) / Cfg::BM) * ((K + Cfg::BN - 1) / Cfg::BN);
             if (int e = gemm_store(dl_t, FMT_E5M2, Mc, x_t + m0, FMT_E4M3, M, V, K, Mc, x_s * grad_s,
-                                   dw_f32, K, kind, st)) return e;
+                                   dw_f32, K, kind, st, pick_splits(tiles, Mc / Cfg::BK))) return e;
         } else {                           // dw [K, V] = x^T [K, Mc] . (dl^T [V, Mc])^T
+            const int tiles = ((K + Cfg::BM - 1) / Cfg::BM) * ((V + Cfg::BN - 1) / Cfg::BN);
             if (int e = gemm_store(x_t + m0, FMT_E4M3, M, dl_t, FMT_E5M2, Mc, K, V, Mc, x_s * grad_s,
-                                   dw_f32, V, kind, st)) return e;
+                                   dw_f32, V, kind, st, pick_splits(tiles, Mc / Cfg::BK))) return e;
         }
     }
     return NGPT_OK;

@@ -32,6 +32,15 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
 }
 
+// Two fp32 values -> bf16 bit patterns packed lo | hi << 16 with the hardware converter
+// (v_cvt_pk_bf16_f32, round to nearest even).
+typedef __bf16 hw_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float hw_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
+    hw_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, hw_bf16x2));
+}
+
 // ---------------------------------------------------------------- f32 -> fp8 (OCP)
 // The hardware converter (v_cvt_pk_fp8_f32 / v_cvt_pk_bf8_f32) rounds to nearest even and keeps
 // subnormals.  What it does above the largest finite value depends on a mode bit, so overflow
@@ -103,5 +112,11 @@ __device__ __forceinline__ void global_to_lds16(const void* gptr, void* lds_wave
         (const __attribute__((address_space(1))) void*)gptr,
         (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
+
+// Workgroup barrier WITHOUT the implicit "wait for all outstanding memory operations" that
+// __syncthreads() carries: the caller states which waits it needs (wait_vmem_le / wait_lds) so
+// that operand loads of later pipeline stages can stay in flight across the barrier.
+__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void wg_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 }  // namespace ngpt

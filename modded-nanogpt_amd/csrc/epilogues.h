@@ -74,6 +74,8 @@ struct EpiStoreBf16 {
     float scale;
     int R, C;
     static constexpr int EXTRA_LDS = 0;
+    static constexpr bool NEEDS_SCRATCH = false;
+    static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     __device__ void begin(int, int, uint8_t*) {}
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
@@ -83,26 +85,46 @@ struct EpiStoreBf16 {
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t*, int) {
+        // address = wave-uniform pointer (tile origin + the element's fixed position inside the wave
+        // tile, all scalar) + ONE per-lane 32-bit offset, so no per-element address registers exist
+        uint16_t* origin = out + ((int64_t)r0 * ld + c0);
+        const uint32_t lane_off = (uint32_t)co.row_base * (uint32_t)ld + (uint32_t)co.col_base;
+        const int rlim = R - r0 - co.row_base, clim = C - c0 - co.col_base;   // lane's element (dr, dc) exists iff dr < rlim && dc < clim
+        const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
 #pragma unroll
         for (int tm = 0; tm < Cfg::TM; ++tm)
 #pragma unroll
             for (int tn = 0; tn < Cfg::TN; ++tn) {
-                int c = c0 + co.col(tn);
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    int r = r0 + co.row(tm, v);
-                    if (r < R && c < C) out[(int64_t)r * ld + c] = (uint16_t)f32_to_bf16_bits(acc[tm][tn][v] * scale);
+                for (int v = 0; v < 16; v += 2) {
+                    const int dr = tm * 32 + 8 * (v >> 2) + (v & 3), dc = tn * 32;
+                    uint16_t* pu = origin + ((int64_t)dr * ld + dc);
+                    uint32_t pk = cvt_pk_bf16(acc[tm][tn][v] * scale, acc[tm][tn][v + 1] * scale);
+                    if (full || (dr < rlim && dc < clim)) pu[lane_off] = (uint16_t)pk;
+                    if (full || (dr + 1 < rlim && dc < clim)) pu[lane_off + (uint32_t)ld] = (uint16_t)(pk >> 16);
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
     }
 };
 
 // Mainloop-only timing aid: keeps the accumulators alive but writes (practically) nothing.
 struct EpiDiscard {
-    float* out;
+    float* out;   // >= 4 floats; workgroup 0 leaves its shader-clock and 100 MHz wall-clock tick counts in out[2], out[3]
     static constexpr int EXTRA_LDS = 0;
-    __device__ void begin(int, int, uint8_t*) {}
-    __device__ void end(uint8_t*, int, int) {}
+    static constexpr bool NEEDS_SCRATCH = false;
+    static constexpr bool JOB_END_NEEDS_SCRATCH = false;
+    long long t_clk, t_wall;
+    __device__ void begin(int, int, uint8_t*) {
+        t_clk = clock64();
+        t_wall = wall_clock64();
+    }
+    __device__ void end(uint8_t*, int bid, int) {
+        if (bid == 0 && threadIdx.x == 0) {
+            out[2] = (float)(clock64() - t_clk);
+            out[3] = (float)(wall_clock64() - t_wall);
+        }
+    }
     template <class Cfg>
     __device__ void job_begin(int) {}
     template <class Cfg>
@@ -120,14 +142,16 @@ struct EpiDiscard {
     }
 };
 
-// out[r, c] (+)= acc * scale in fp32
+// out[r, c] (+)= acc * scale in fp32 (the += form uses floating-point atomics)
+template <bool ACCUMULATE>
 struct EpiStoreF32 {
     float* out;
     int64_t ld;
     float scale;
     int R, C;
-    int accumulate;
     static constexpr int EXTRA_LDS = 0;
+    static constexpr bool NEEDS_SCRATCH = false;
+    static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     __device__ void begin(int, int, uint8_t*) {}
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
@@ -137,20 +161,30 @@ struct EpiStoreF32 {
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t*, int) {
+        float* origin = out + ((int64_t)r0 * ld + c0);
+        const uint32_t lane_off = (uint32_t)co.row_base * (uint32_t)ld + (uint32_t)co.col_base;
+        const int rlim = R - r0 - co.row_base, clim = C - c0 - co.col_base;
+        const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
 #pragma unroll
         for (int tm = 0; tm < Cfg::TM; ++tm)
 #pragma unroll
             for (int tn = 0; tn < Cfg::TN; ++tn) {
-                int c = c0 + co.col(tn);
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    int r = r0 + co.row(tm, v);
-                    if (r < R && c < C) {
-                        float* p = out + (int64_t)r * ld + c;
-                        float val = acc[tm][tn][v] * scale;
-                        *p = accumulate ? (*p + val) : val;
+                for (int v = 0; v < 16; v += 2) {
+                    const int dr = tm * 32 + 8 * (v >> 2) + (v & 3), dc = tn * 32;
+                    float* pu = origin + ((int64_t)dr * ld + dc);
+                    float v0 = acc[tm][tn][v] * scale, v1 = acc[tm][tn][v + 1] * scale;
+                    // accumulation is a fire-and-forget L2 atomic: no read-modify-write through registers
+                    if (full || (dr < rlim && dc < clim)) {
+                        if constexpr (ACCUMULATE) (void)__hip_atomic_fetch_add(&pu[lane_off], v0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        else pu[lane_off] = v0;
+                    }
+                    if (full || (dr + 1 < rlim && dc < clim)) {
+                        if constexpr (ACCUMULATE) (void)__hip_atomic_fetch_add(&pu[lane_off + (uint32_t)ld], v1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        else pu[lane_off + (uint32_t)ld] = v1;
                     }
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
     }
 };
@@ -169,6 +203,8 @@ struct EpiRelu2 {
     int R, C;
     float scale, inv_act, amax;
     static constexpr int EXTRA_LDS = 0;
+    static constexpr bool NEEDS_SCRATCH = true;
+    static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     template <class Cfg>
     __device__ void job_begin(int) {}
     template <class Cfg>
@@ -212,7 +248,7 @@ struct EpiRelu2 {
         float* red = (float*)smem;
         int wave = threadIdx.x >> 6;
         if ((threadIdx.x & 63) == 0) red[wave] = m;
-        __syncthreads();
+        wg_barrier();
         if (threadIdx.x == 0) {
             float t = 0.0f;
             for (int w = 0; w < (int)(blockDim.x >> 6); ++w) t = fmaxf(t, red[w]);

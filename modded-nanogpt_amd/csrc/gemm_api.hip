@@ -72,25 +72,54 @@ static int check_gemm_dims(const char* who, int R, int C, int K, int64_t lda, in
     return NGPT_OK;
 }
 
-int g_tuning[8] = {0, 1, 0, 0, 0, 0, 0, 0};
+int g_tuning[8] = {0, 2, 0, 0, 1, 0, 0, 0};
 
 // Which profile slot the next gemm_store launches are booked under (set by the fused CE backward).
 int g_gemm_slot = PROF_GEMM;
 
+// Smallest split-K factor (<= 8) whose job count fills the persistent grid to >= 94 %, or else the
+// best one found.  One job must keep at least 8 k-steps.
+int pick_splits(int tiles, int ksteps) {
+    // Measured on MI355X: the skinny backward GEMMs are bound by their strided operand loads, not by
+    // grid occupancy, so splitting the contraction buys nothing; it stays opt-in (tuning key 6).
+    if (!g_tuning[6]) return 1;
+    int cus = num_cus();
+    if (cus <= 0 || tiles <= 0) return 1;
+    int best = 1;
+    double best_eff = 0.0;
+    for (int s = 1; s <= 8 && ksteps / s >= 8; ++s) {
+        int jobs = tiles * s;
+        int rounds = (jobs + cus - 1) / cus;
+        double eff = (double)jobs / ((double)rounds * cus);
+        if (eff > best_eff + 1e-9) { best_eff = eff; best = s; }
+        if (eff >= 0.94) break;
+    }
+    return best;
+}
+
+// out_kind: 0 bf16, 1 fp32, 2 fp32 accumulate (atomic), 3 discard.  splits > 1 cuts each tile's
+// contraction into that many jobs and needs out_kind 2 on a buffer the caller has zeroed or wants added to.
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
-               float scale, void* out, int64_t ldc, int out_kind, hipStream_t st) {
+               float scale, void* out, int64_t ldc, int out_kind, hipStream_t st, int splits) {
     if (int e = check_gemm_dims("gemm_fp8_tn", R, C, K, lda, ldb)) return e;
-    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K};
+    if (splits < 1) splits = 1;
+    if (splits > K / 128) splits = K / 128;
+    if (splits > 1 && out_kind != 2) return fail(NGPT_EINVAL, "gemm_fp8_tn: split-K needs the accumulating fp32 output");
+    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, splits, g_tuning[2]};
     ProfileScope prof(g_gemm_slot, st);
     if (out_kind == 0) {
         EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
     if (out_kind == 3) {
-        EpiDiscard epi{(float*)out};
+        EpiDiscard epi{(float*)out, 0, 0};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
-    EpiStoreF32 epi{(float*)out, ldc, scale, R, C, out_kind == 2};
+    if (out_kind == 2) {
+        EpiStoreF32<true> epi{(float*)out, ldc, scale, R, C};
+        return launch_gemm<MainCfg>(g, fa, fb, epi, st);
+    }
+    EpiStoreF32<false> epi{(float*)out, ldc, scale, R, C};
     return launch_gemm<MainCfg>(g, fa, fb, epi, st);
 }
 
@@ -144,7 +173,7 @@ extern "C" int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const voi
     if ((fmt_a | fmt_b) & ~1) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: fmt_a=%d fmt_b=%d", fmt_a, fmt_b);
     if (out_kind < 0 || out_kind > 3) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: out_kind=%d", out_kind);
     if (ldc < C) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: ldc=%lld < C=%d", (long long)ldc, C);
-    return gemm_store(A, fmt_a, lda, B, fmt_b, ldb, R, C, K, scale, out, ldc, out_kind, (hipStream_t)stream);
+    return gemm_store(A, fmt_a, lda, B, fmt_b, ldb, R, C, K, scale, out, ldc, out_kind, (hipStream_t)stream, g_tuning[4]);
 }
 
 // ------------------------------------------------------------------------------------------ mm forward
@@ -174,7 +203,7 @@ extern "C" int ngpt_mm_fwd(const void* x_bf16, const void* w_bf16, int M, int N,
         if (int e = ngpt_quant_fp8_2d(w_bf16, K, N, w_s, NGPT_FMT_E4M3, w_f8, workspace, stream)) return e;
         w_nk = workspace;
     }
-    return gemm_store(x_f8, FMT_E4M3, K, w_nk, FMT_E4M3, K, M, N, K, x_s * w_s, out_bf16, N, 0, st);
+    return gemm_store(x_f8, FMT_E4M3, K, w_nk, FMT_E4M3, K, M, N, K, x_s * w_s, out_bf16, N, 0, st, 1);
 }
 
 // ------------------------------------------------------------------------------------------ mm backward
@@ -210,9 +239,9 @@ extern "C" int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f
         w_kn = w_f8_t;
     }
     // dx [M,K] = g_f8 [M,N] . (w [K,N])^T, contraction over N
-    if (int e = gemm_store(g_f8, FMT_E5M2, N, w_kn, FMT_E4M3, N, M, K, N, grad_s * w_s, dx_bf16, K, 0, st)) return e;
+    if (int e = gemm_store(g_f8, FMT_E5M2, N, w_kn, FMT_E4M3, N, M, K, N, grad_s * w_s, dx_bf16, K, 0, st, 1)) return e;
     // dw [K,N] = x_f8^T [K,M] . (g_f8^T [N,M])^T, contraction over M
-    return gemm_store(x_f8_t, FMT_E4M3, M, g_f8_t, FMT_E5M2, M, K, N, M, x_s * grad_s, dw_kn_f32, N, 1, st);
+    return gemm_store(x_f8_t, FMT_E4M3, M, g_f8_t, FMT_E5M2, M, K, N, M, x_s * grad_s, dw_kn_f32, N, 1, st, 1);
 }
 
 // ------------------------------------------------------------------------------------------ fc + relu^2
@@ -224,7 +253,7 @@ extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float
         return fail(NGPT_EINVAL, "ngpt_fc_relu2_fwd: post_f8 needs act_scale and partial_amax");
     if (int e = check_gemm_dims("ngpt_fc_relu2_fwd", M, N, K, K, K)) return e;
     if (N % 16) return fail(NGPT_EALIGN, "ngpt_fc_relu2_fwd: N=%d must be a multiple of 16", N);
-    GemmOperands g{(const uint8_t*)x_f8, (const uint8_t*)w_f8, K, K, M, N, K};
+    GemmOperands g{(const uint8_t*)x_f8, (const uint8_t*)w_f8, K, K, M, N, K, 1, 0};
     EpiRelu2 epi{};
     epi.post = (uint16_t*)post_bf16;
     epi.ld = N;

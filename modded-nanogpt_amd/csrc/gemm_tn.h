@@ -30,11 +30,14 @@ struct GemmOperands {
     const uint8_t* B;   // [C, K] fp8, row stride ldb bytes
     int64_t lda, ldb;
     int R, C, K;        // K % 128 == 0
+    int splits;         // split-K: each tile's contraction is cut into this many jobs (>= 1); needs an accumulating epilogue if > 1
+    int ablate;         // timing aid: bit 0 = issue no operand loads after the first, bit 1 = no MFMA work, bit 2 = no k-loop barrier
 };
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1>
 struct TileCfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, NSTAGES = NSTAGES_;
+    static constexpr int WGS_PER_CU = WGS_PER_CU_;                 // co-resident workgroups the register budget allows
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int NWAVES = WAVES_M * WAVES_N;
     static constexpr int THREADS = NWAVES * 64;
@@ -93,10 +96,35 @@ __device__ __forceinline__ void wait_vmem_le() {
     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// Operand addresses are a wave-uniform 64-bit base (SGPRs) plus a 32-bit per-lane offset, which keeps
+// the k-loop free of 64-bit VGPR pointer arithmetic; a tile's operand slab must span < 4 GiB.
+template <class Cfg>
+struct LaneOffsets {
+    uint32_t a_off[Cfg::A_LOADS], b_off[Cfg::B_LOADS];   // byte offset of this lane's chunk from the tile's first row
+    __device__ void init(const GemmOperands& g, int wave, int lane, int r0, int c0) {
+        int lrow = lane / Cfg::CPR, lchunk = lane % Cfg::CPR;
+#pragma unroll
+        for (int i = 0; i < Cfg::A_LOADS; ++i) {
+            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
+            int q = lchunk ^ Cfg::swz(R);
+            int rr = min(R, g.R - 1 - r0);                       // clamp rows past the end
+            a_off[i] = (uint32_t)((int64_t)rr * g.lda + q * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < Cfg::B_LOADS; ++i) {
+            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
+            int q = lchunk ^ Cfg::swz(R);
+            int rr = min(R, g.C - 1 - c0);
+            b_off[i] = (uint32_t)((int64_t)rr * g.ldb + q * 16);
+        }
+    }
+};
+
 template <class Cfg, int AFMT, int BFMT>
 struct TileMainloop {
-    const uint8_t* a_ptr[Cfg::A_LOADS];
-    const uint8_t* b_ptr[Cfg::B_LOADS];
+    LaneOffsets<Cfg> lo;
+    const uint8_t* a_base;   // wave-uniform: first row of the tile
+    const uint8_t* b_base;
     int frag_a[Cfg::TM];     // LDS byte offset of this lane's first 16-byte chunk, stage 0, ksub 0
     int frag_b[Cfg::TN];
     int wave, lane, wr, wc;
@@ -120,37 +148,29 @@ struct TileMainloop {
         }
     }
 
-    // Point the per-lane global pointers at tile (r0, c0).  Rows past the end are clamped to the
-    // last row: they are loaded (valid memory) and their results discarded by the epilogue.
+    // Point the loads at tile (r0, c0).  Rows past the end are clamped to the last row: they are
+    // loaded (valid memory) and their results discarded by the epilogue.
     __device__ void set_tile(const GemmOperands& g, int r0, int c0) {
-        int lrow = lane / Cfg::CPR, lchunk = lane % Cfg::CPR;
-#pragma unroll
-        for (int i = 0; i < Cfg::A_LOADS; ++i) {
-            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
-            int q = lchunk ^ Cfg::swz(R);
-            int gr = min(r0 + R, g.R - 1);
-            a_ptr[i] = g.A + (int64_t)gr * g.lda + q * 16;
-        }
-#pragma unroll
-        for (int i = 0; i < Cfg::B_LOADS; ++i) {
-            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
-            int q = lchunk ^ Cfg::swz(R);
-            int gc = min(c0 + R, g.C - 1);
-            b_ptr[i] = g.B + (int64_t)gc * g.ldb + q * 16;
-        }
+        a_base = g.A + (int64_t)r0 * g.lda;
+        b_base = g.B + (int64_t)c0 * g.ldb;
+        lo.init(g, wave, lane, r0, c0);
     }
 
     __device__ void issue_loads(uint8_t* smem, int stage, int kt) {
         uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
-        int koff = kt * Cfg::BK;
+        const uint8_t* ab = a_base + kt * Cfg::BK;
+        const uint8_t* bb = b_base + kt * Cfg::BK;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i)
-            global_to_lds16(a_ptr[i] + koff, s + (wave + i * Cfg::NWAVES) * 1024);
+            global_to_lds16(ab + lo.a_off[i], s + (wave + i * Cfg::NWAVES) * 1024);
 #pragma unroll
         for (int i = 0; i < Cfg::B_LOADS; ++i)
-            global_to_lds16(b_ptr[i] + koff, s + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
+            global_to_lds16(bb + lo.b_off[i], s + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
     }
 
+    // One k-step of MFMAs.  FIRST: this is the first k-step of a tile, so its first sub-step starts the
+    // accumulators from the constant 0 (the C operand of the MFMA) instead of from zeroed registers.
+    template <bool FIRST>
     __device__ void compute(const uint8_t* smem, int stage, v16f (&acc)[Cfg::TM][Cfg::TN]) {
         const uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
 #pragma unroll
@@ -173,9 +193,16 @@ struct TileMainloop {
 #pragma unroll
             for (int tm = 0; tm < Cfg::TM; ++tm)
 #pragma unroll
-                for (int tn = 0; tn < Cfg::TN; ++tn)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                        a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
+                for (int tn = 0; tn < Cfg::TN; ++tn) {
+                    if (FIRST && ks == 0) {
+                        const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                        acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            a[tm], b[tn], zero, AFMT, BFMT, 0, 0, 0, 0);
+                    } else {
+                        acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
+                    }
+                }
         }
     }
 };
@@ -192,25 +219,37 @@ struct AccCoords {
     __device__ int col(int tn) const { return col_base + tn * 32; }
 };
 
-// Default tile walk: every tile of the R x C grid once, in TileOrder.
+// Default job walk: every (tile, contraction split) of the R x C grid once.  Jobs are numbered
+// split-major (all tiles of split 0 in TileOrder, then split 1, ...), so the workgroups that run
+// together work on neighbouring tiles of the same split.
 struct GridIter {
     TileOrder order;
-    int it, bid, G, seq, tr_, tc_;
+    int it, bid, G, seq, tr_, tc_, split_, splits, jobs;
     __device__ GridIter(const GemmOperands& g, int BM, int BN, int bid_, int G_)
-        : order(g.R, g.C, BM, BN), it(0), bid(bid_), G(G_), tr_(0), tc_(0) {
+        : order(g.R, g.C, BM, BN), it(0), bid(bid_), G(G_), tr_(0), tc_(0), split_(0),
+          splits(g.splits < 1 ? 1 : g.splits) {
+        jobs = order.total * splits;
         seq = TileOrder::seq_of(0, bid, G);
-        if (valid()) order.coords(seq, tr_, tc_);
+        locate();
     }
-    __device__ bool valid() const { return seq < order.total; }
+    __device__ void locate() {
+        if (seq < jobs) {
+            split_ = seq / order.total;
+            order.coords(seq - split_ * order.total, tr_, tc_);
+        }
+    }
+    __device__ bool valid() const { return seq < jobs; }
     __device__ int tr() const { return tr_; }
     __device__ int tc() const { return tc_; }
+    __device__ int kt_begin(int nk) const { return (int)((int64_t)nk * split_ / splits); }
+    __device__ int kt_end(int nk) const { return (int)((int64_t)nk * (split_ + 1) / splits); }
     __device__ bool job_begin() const { return false; }
     __device__ bool job_end() const { return false; }
     __device__ int job_id() const { return 0; }
     __device__ void advance() {
         ++it;
         seq = TileOrder::seq_of(it, bid, G);
-        if (valid()) order.coords(seq, tr_, tc_);
+        locate();
     }
 };
 
@@ -229,19 +268,22 @@ struct GridIter {
 template <class Iter>
 struct StepCursor {
     Iter it;
-    int kt;
-    __device__ StepCursor(const Iter& i) : it(i), kt(0) {}
+    int kt, nk;
+    __device__ StepCursor(const Iter& i, int nk_) : it(i), kt(0), nk(nk_) {
+        if (it.valid()) kt = it.kt_begin(nk);
+    }
     __device__ bool valid() const { return it.valid(); }
-    __device__ void advance(int nk) {
-        if (++kt == nk) {
-            kt = 0;
+    __device__ bool at_job_start() const { return kt == it.kt_begin(nk); }
+    __device__ void advance() {
+        if (++kt == it.kt_end(nk)) {
             it.advance();
+            kt = it.valid() ? it.kt_begin(nk) : 0;
         }
     }
 };
 
 template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
-__global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel(GemmOperands g, Epi epi) {
+__global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(GemmOperands g, Epi epi) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_all[];
     static_assert(Epi::EXTRA_LDS % 1024 == 0, "epilogue LDS must keep the stages 1 KiB aligned");
     uint8_t* const smem = smem_all + Epi::EXTRA_LDS;      // operand stages
@@ -254,16 +296,14 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel(GemmOperands g, E
     Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
 
     // prologue: put NS-1 k-steps in flight
-    StepCursor<Iter> pre(cur);
+    StepCursor<Iter> pre(cur, nk);
     int pre_slot = 0;
-    bool pre_new_tile = true;
 #pragma unroll
     for (int i = 0; i < NS - 1; ++i) {
         if (pre.valid()) {
-            if (pre_new_tile) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
+            if (pre.at_job_start()) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
             ml.issue_loads(smem, pre_slot, pre.kt);
-            pre.advance(nk);
-            pre_new_tile = (pre.kt == 0);
+            pre.advance();
         }
         pre_slot = (pre_slot + 1 == NS) ? 0 : pre_slot + 1;
     }
@@ -281,7 +321,8 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel(GemmOperands g, E
     while (cur.valid()) {
         const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
         if (cur.job_begin()) epi.template job_begin<Cfg>(c0);   // made visible by the k-loop's barriers
-        for (int kt = 0; kt < nk; ++kt) {
+        const int kt0 = cur.kt_begin(nk), kt1 = cur.kt_end(nk);
+        for (int kt = kt0; kt < kt1; ++kt) {
             // The loads of this k-step are the oldest loads in flight and loads retire in order, so it
             // is enough that at most the NS-2 newer load groups remain outstanding.  Stores issued by
             // an epilogue share the counter and may retire in any order relative to loads; they only
@@ -289,19 +330,18 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel(GemmOperands g, E
             // issued, so wait for everything.
             if (pre.valid()) wait_vmem_le<(NS - 2) * Cfg::LOADS>();
             else wait_vmem_le<0>();
-            __syncthreads();
+            if (!(g.ablate & 4)) wg_barrier();
             // refill the slot consumed in the previous step with the k-step NS-1 ahead
             if (pre.valid()) {
-                if (pre_new_tile) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
-                ml.issue_loads(smem, pre_slot, pre.kt);
-                pre.advance(nk);
-                pre_new_tile = (pre.kt == 0);
+                if (pre.at_job_start()) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
+                if (!(g.ablate & 1)) ml.issue_loads(smem, pre_slot, pre.kt);
+                pre.advance();
                 pre_slot = (pre_slot + 1 == NS) ? 0 : pre_slot + 1;
             }
-            ml.compute(smem, slot, acc);
+            if (!(g.ablate & 2)) ml.template compute<false>(smem, slot, acc);
             slot = (slot + 1 == NS) ? 0 : slot + 1;
         }
-        __syncthreads();   // every wave is done reading the last slot: reuse it as scratch
+        wg_barrier();   // every wave is done reading the last slot: reuse it as scratch
         uint8_t* free_stage = smem + (slot == 0 ? NS - 1 : slot - 1) * Cfg::STAGE_BYTES;
         epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
         if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
@@ -313,7 +353,198 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel(GemmOperands g, E
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
         cur.advance();
     }
-    __syncthreads();
+    wg_barrier();
+    epi.end(smem, bid, G);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Software-pipelined variant (two LDS stages, BK = 128), meant for 4 waves per workgroup so that
+// each wave owns a whole SIMD: 128 x 128 per wave, 256 accumulator registers (AGPRs) and room for
+// double-buffered operand fragments.
+//
+// In gemm_tn_kernel every wave leaves the per-k-step barrier at the same moment, reads its operand
+// fragments from LDS, waits, and only then issues MFMAs, so LDS reads and MFMAs do not overlap.
+// Here each wave keeps its MFMA pipe fed:
+//   * fragments are prefetched on a rolling basis: as soon as the MFMAs that consume b[tn] of the
+//     current 64-byte contraction sub-step are issued, the same registers are reloaded with b[tn]
+//     of the next sub-step (A fragments use one spare set);
+//   * the workgroup barrier sits between the two contraction sub-steps of a k-step.  By then all LDS
+//     reads of the current stage are done, so the stage is refilled right after the barrier and the
+//     first fragments of the next k-step are read under the second sub-step's MFMAs.
+// Epilogues that stage data through LDS (Epi::NEEDS_SCRATCH for every tile, Epi::JOB_END_NEEDS_SCRATCH
+// for job ends only) get the current stage as scratch; for them the refill of that stage is issued
+// after the epilogue instead of before it.
+//
+template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
+__global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel_v2(GemmOperands g, Epi epi) {
+    static_assert(Cfg::NSTAGES == 2 && Cfg::KSUB == 2, "pipelined kernel: two stages of 128 contraction bytes");
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem_all[];
+    static_assert(Epi::EXTRA_LDS % 1024 == 0, "epilogue LDS must keep the stages 1 KiB aligned");
+    uint8_t* const smem = smem_all + Epi::EXTRA_LDS;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave / Cfg::WAVES_N, wc = wave % Cfg::WAVES_N;
+    const int bid = blockIdx.x, G = gridDim.x;
+    const int nk = g.K / Cfg::BK;
+    AccCoords<Cfg> coords(wr, wc, lane);
+    Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
+    if (!cur.valid()) return;
+
+    // LDS byte offsets of this lane's first fragment chunk (stage 0, sub-step 0)
+    int frag_a[TM], frag_b[TN];
+    {
+        int h = lane >> 5;
+#pragma unroll
+        for (int t = 0; t < TM; ++t) {
+            int row = wr * Cfg::WTM + t * 32 + (lane & 31);
+            frag_a[t] = row * Cfg::BK + (((h * 2) ^ Cfg::swz(row)) << 4);
+        }
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+            int row = wc * Cfg::WTN + t * 32 + (lane & 31);
+            frag_b[t] = Cfg::A_BYTES + row * Cfg::BK + (((h * 2) ^ Cfg::swz(row)) << 4);
+        }
+    }
+    auto read_frag = [&](int slot, int ks, int frag_off) -> v8i {
+        const uint8_t* sp = smem + slot * Cfg::STAGE_BYTES;
+        int o = frag_off ^ (ks * 64);
+        v4i lo = *(const v4i*)(sp + o);
+        v4i hi = *(const v4i*)(sp + (o ^ 16));
+        return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    };
+
+    // operand load state: uniform tile bases + per-lane 32-bit offsets
+    LaneOffsets<Cfg> lo;
+    const uint8_t* a_base = nullptr;
+    const uint8_t* b_base = nullptr;
+    auto set_tile = [&](int tr, int tc) {
+        int r0 = tr * Cfg::BM, c0 = tc * Cfg::BN;
+        a_base = g.A + (int64_t)r0 * g.lda;
+        b_base = g.B + (int64_t)c0 * g.ldb;
+        lo.init(g, wave, lane, r0, c0);
+    };
+    auto issue_loads = [&](int slot, int kt) {
+        uint8_t* sp = smem + slot * Cfg::STAGE_BYTES;
+        const uint8_t* ab = a_base + kt * Cfg::BK;
+        const uint8_t* bb = b_base + kt * Cfg::BK;
+#pragma unroll
+        for (int i = 0; i < Cfg::A_LOADS; ++i)
+            global_to_lds16(ab + lo.a_off[i], sp + (wave + i * Cfg::NWAVES) * 1024);
+#pragma unroll
+        for (int i = 0; i < Cfg::B_LOADS; ++i)
+            global_to_lds16(bb + lo.b_off[i], sp + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
+    };
+
+    // prologue: k-steps 0 and 1 in flight, wait for step 0, read its first fragments
+    StepCursor<Iter> pre(cur, nk);
+    set_tile(pre.it.tr(), pre.it.tc());
+    issue_loads(0, 0);
+    pre.advance();
+    bool pre_new_tile = (pre.kt == 0);
+    if (pre.valid()) {
+        if (pre_new_tile) set_tile(pre.it.tr(), pre.it.tc());
+        issue_loads(1, pre.kt);
+        pre.advance();
+        pre_new_tile = (pre.kt == 0);
+        wait_vmem_le<Cfg::LOADS>();
+    } else {
+        wait_vmem_le<0>();
+    }
+    epi.begin(bid, G, smem_all);
+    wg_barrier();
+
+    v8i a[TM], b[TN], an[TM];
+#pragma unroll
+    for (int t = 0; t < TM; ++t) a[t] = read_frag(0, 0, frag_a[t]);
+#pragma unroll
+    for (int t = 0; t < TN; ++t) b[t] = read_frag(0, 0, frag_b[t]);
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    int slot = 0;
+    while (cur.valid()) {
+        const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
+        if (cur.job_begin()) epi.template job_begin<Cfg>(c0);
+        for (int kt = 0; kt < nk; ++kt) {
+            const bool last = (kt + 1 == nk);
+            // ---- sub-step 0: MFMAs on the fragments in registers, rolling prefetch of sub-step 1
+#pragma unroll
+            for (int t = 0; t < TM; ++t) an[t] = read_frag(slot, 1, frag_a[t]);
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+                    acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
+                b[tn] = read_frag(slot, 1, frag_b[tn]);
+            }
+#pragma unroll
+            for (int t = 0; t < TM; ++t) a[t] = an[t];
+            // ---- every wave is past its reads of this stage; the next k-step has landed
+            wait_vmem_le<0>();
+            wg_barrier();                            // includes lgkmcnt(0): this wave's LDS reads are done
+            const bool refill_late = last && (Epi::NEEDS_SCRATCH || (Epi::JOB_END_NEEDS_SCRATCH && cur.job_end()));
+            if (!refill_late && pre.valid()) {
+                if (pre_new_tile) set_tile(pre.it.tr(), pre.it.tc());
+                if (!(g.ablate & 1)) issue_loads(slot, pre.kt);
+                pre.advance();
+                pre_new_tile = (pre.kt == 0);
+            }
+            // ---- sub-step 1, prefetching the first fragments of the next k-step from the other stage
+            if (!last) {
+#pragma unroll
+                for (int t = 0; t < TM; ++t) an[t] = read_frag(slot ^ 1, 0, frag_a[t]);
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+                    for (int tm = 0; tm < TM; ++tm)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
+                    b[tn] = read_frag(slot ^ 1, 0, frag_b[tn]);
+                }
+#pragma unroll
+                for (int t = 0; t < TM; ++t) a[t] = an[t];
+            } else {
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                    for (int tm = 0; tm < TM; ++tm)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
+                // tile finished: epilogue, then pick up the next tile's first fragments
+                uint8_t* scratch_stage = smem + slot * Cfg::STAGE_BYTES;   // free only if the refill was postponed
+                epi.template tile<Cfg>(acc, r0, c0, coords, scratch_stage + wave * Cfg::WAVE_SCRATCH, lane);
+                if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, scratch_stage);
+                if (refill_late) {
+                    wg_barrier();          // every wave is done with the scratch
+                    if (pre.valid()) {
+                        if (pre_new_tile) set_tile(pre.it.tr(), pre.it.tc());
+                        issue_loads(slot, pre.kt);
+                        pre.advance();
+                        pre_new_tile = (pre.kt == 0);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+#pragma unroll
+                for (int t = 0; t < TM; ++t) a[t] = read_frag(slot ^ 1, 0, frag_a[t]);
+#pragma unroll
+                for (int t = 0; t < TN; ++t) b[t] = read_frag(slot ^ 1, 0, frag_b[t]);
+            }
+            slot ^= 1;
+        }
+        cur.advance();
+    }
+    wg_barrier();
     epi.end(smem, bid, G);
 }
 
