@@ -64,6 +64,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device-to-device copy, the known-size kernel that scales "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU (the kernel on one GPU's share of the "
@@ -91,6 +94,12 @@ def main() -> int:
             sc["A"], sc["B"], sc["C"], False)
         return losses, dx, dw
 
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

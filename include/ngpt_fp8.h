@@ -56,8 +56,11 @@ int ngpt_num_cus(void);
 int ngpt_profile_enable(int on);
 int ngpt_profile_read(int slot, double* total_ms, int* launches);
 
-/* Tuning aid, no counterpart in the reference: key 0 selects the GEMM tile configuration
- * (0 = default), key 1 the number of persistent workgroups per compute unit. */
+/* Tuning / timing aid, no counterpart in the reference.  key 0: GEMM tile configuration (0 = default
+ * 256x256 two-stage, 1 = 256x256 four-stage, 5 = 256x128 two workgroups per CU); key 2: ablation bits
+ * for timing runs (1 = no operand loads, 2 = no MFMAs, 4 = no k-loop barrier; results are then
+ * meaningless); key 4: split-K factor used by ngpt_gemm_fp8_tn with out_kind 2; key 5: tile
+ * configuration of the fused CE kernels; key 6: split-K in the fused CE backward GEMMs. */
 int ngpt_tuning_set(int key, int value);
 
 /* ---- quantisers ---------------------------------------------------------------------------
@@ -117,6 +120,25 @@ int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f8, int M, i
 int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, int M, int N, int K,
                       void* post_bf16, void* post_f8, const float* act_scale,
                       float* partial_amax, int n_partials, void* stream);
+
+/* ---- delayed-scaling bookkeeping of the FP8 down projection, tied-embedding gradient add -----
+ * scales[l] = max(max_i partial_amax[l * partial_stride + i], 1e-12) * headroom / 448:
+ * reduce_mlp_activation_scales(_kernel), triton_kernels.py:502-519, 732-745. */
+int ngpt_reduce_scales(const float* partial_amax, int64_t partial_stride, int num_layers, int partial_count,
+                       float headroom, float* scales, void* stream);
+
+/* The tile kernel of quantize_transpose_mlp_down_weights, triton_kernels.py:522-565, 748-778:
+ * weights [L, hidden, model_dim] bf16 (layer stride in elements) -> out_f8 [L, model_dim, hidden] =
+ * e4m3(clamp(w / scales[l], +-448)); used_scales[l] = scales[l]; partial_amax[l, tile] = max |w| over
+ * each 64 x 64 tile (tiles = ceil(hidden/64) * ceil(model_dim/64)).  The caller then reduces the
+ * partials into the next scales with ngpt_reduce_scales.  hidden % 16 == 0, model_dim % 16 == 0. */
+int ngpt_quant_transpose_down(const void* weights_bf16, int num_layers, int hidden, int model_dim,
+                              int64_t layer_stride, const float* scales, void* out_f8, float* used_scales,
+                              float* partial_amax, void* stream);
+
+/* dst [cols, rows] += src [rows, cols]^T for bf16 (elem_bytes 2) or fp32 (4):
+ * transpose_add, triton_kernels.py:844-903. */
+int ngpt_transpose_add(const void* src, int rows, int cols, void* dst, int elem_bytes, void* stream);
 
 /* ---- nanogpt::ce_fwd_bwd on materialised logits -------------------------------------------
  * ce_fwd_bwd_kernel, triton_kernels.py:956-1170, 1182-1206.  logits [n_rows, n_cols] bf16,

@@ -8,10 +8,12 @@ its absence is an error: there is no fallback implementation.
 """
 from . import _lib, ops                                   # noqa: F401  (registers torch.ops.nanogpt.*)
 from .fused import (FusedLinearReLUSquareFunction, FusedSoftcappedCrossEntropy, ReLUSqrdMLP,  # noqa: F401
-                    linear_relu_square, transpose_copy)
+                    linear_relu_square, quantize_transpose_mlp_down_weights, reduce_mlp_activation_scales,
+                    transpose_add, transpose_copy)
 from .ops import gemm_fp8_tn, quant_fp8, quant_fp8_2d     # noqa: F401
 
 __all__ = [
     "FusedLinearReLUSquareFunction", "FusedSoftcappedCrossEntropy", "ReLUSqrdMLP",
-    "linear_relu_square", "transpose_copy", "gemm_fp8_tn", "quant_fp8", "quant_fp8_2d",
+    "linear_relu_square", "transpose_copy", "transpose_add", "quantize_transpose_mlp_down_weights",
+    "reduce_mlp_activation_scales", "gemm_fp8_tn", "quant_fp8", "quant_fp8_2d",
 ]

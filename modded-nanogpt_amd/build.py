@@ -17,7 +17,7 @@ PKG = pathlib.Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libngpt_fp8.so"
-SOURCES = ["gemm_api.hip", "quant.hip", "ce.hip"]
+SOURCES = ["gemm_api.hip", "quant.hip", "ce.hip", "mlp_aux.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

@@ -211,35 +211,45 @@ __global__ __launch_bounds__(ROW_THREADS) void ce_rows_kernel(
 // =====================================================================================================
 // Fused forward.  GEMM orientation: rows = vocabulary (A = w_f8 [V, K]), columns = tokens
 // (B = x_f8 [M, K]), so one lane owns one token per MFMA tile column and sums exponentials in
-// registers.  A job = (token tile, vocabulary split); XCD x (workgroups with bid % 8 == x) only
-// handles split x, so each XCD streams one eighth of the weight matrix and keeps it in its L2.
-constexpr int CE_SPLITS = 8;
+// registers.  A job = (token tile, vocabulary split); the workgroup walks the split's vocabulary
+// tiles with the token tile fixed and flushes its row sums at the end of the job.
+//
+// L2-aware placement (workgroup b runs on XCD b % 8, each XCD has its own 4 MB L2): XCD x owns a
+// contiguous block of token tiles.  Its workgroups form an MG x CE_SPLITS grid: MG token tiles are
+// processed at the same time, each by CE_SPLITS workgroups that take one vocabulary split each.
+// The MG token tiles (MG * 196 KB at K = 768) stay L2-resident for the whole round, and every
+// weight tile streamed from memory is used by the MG workgroups of its split at about the same time.
+constexpr int CE_SPLITS = 4;
+constexpr int CE_XCDS = 8;
 
 struct CEJobIter {
-    int tiles_v, tiles_m, slot, nslots, split, it, tr_, tr_end;
+    int tiles_v, tile_m_end, tile_m, mg, split, tr_, tr_begin, tr_end;
     __device__ CEJobIter(const GemmOperands& g, int BM, int BN, int bid, int G) {
         tiles_v = (g.R + BM - 1) / BM;
-        tiles_m = (g.C + BN - 1) / BN;
-        split = bid % CE_SPLITS;
-        slot = bid / CE_SPLITS;
-        nslots = G / CE_SPLITS;
-        it = 0;
-        tr_ = tiles_v * split / CE_SPLITS;
+        const int tiles_m = (g.C + BN - 1) / BN;
+        const int xcd = bid % CE_XCDS, slot = bid / CE_XCDS;
+        mg = G / (CE_XCDS * CE_SPLITS);                       // token tiles in flight per XCD
+        const int per_xcd = (tiles_m + CE_XCDS - 1) / CE_XCDS;
+        split = slot / mg;
+        tile_m = xcd * per_xcd + slot % mg;
+        tile_m_end = min(tiles_m, (xcd + 1) * per_xcd);
+        tr_begin = tiles_v * split / CE_SPLITS;
         tr_end = tiles_v * (split + 1) / CE_SPLITS;
-        if (tr_ >= tr_end) it = tiles_m;     // empty vocabulary range: nothing to do
+        tr_ = tr_begin;
+        if (tr_begin >= tr_end) tile_m = tile_m_end;          // empty vocabulary range: nothing to do
     }
-    __device__ bool valid() const { return slot + it * nslots < tiles_m; }
+    __device__ bool valid() const { return tile_m < tile_m_end; }
     __device__ int tr() const { return tr_; }
-    __device__ int tc() const { return slot + it * nslots; }
+    __device__ int tc() const { return tile_m; }
     __device__ int kt_begin(int) const { return 0; }
     __device__ int kt_end(int nk) const { return nk; }
-    __device__ bool job_begin() const { return tr_ == tiles_v * split / CE_SPLITS; }
+    __device__ bool job_begin() const { return tr_ == tr_begin; }
     __device__ bool job_end() const { return tr_ + 1 == tr_end; }
     __device__ int job_id() const { return split; }
     __device__ void advance() {
         if (++tr_ == tr_end) {
-            tr_ = tiles_v * split / CE_SPLITS;
-            ++it;
+            tr_ = tr_begin;
+            tile_m += mg;
         }
     }
 };
@@ -538,13 +548,15 @@ static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwd& epi, hipStream_t
         configured = true;
     }
     int cus = num_cus();
-    if (cus < CE_SPLITS) return fail(NGPT_EINVAL, "no HIP device");
+    if (cus < CE_XCDS * CE_SPLITS) return fail(NGPT_EINVAL, "no HIP device (or fewer than %d compute units)", CE_XCDS * CE_SPLITS);
     int tiles_m = (g.C + Cfg::BN - 1) / Cfg::BN;
-    int slots_max = cus * Cfg::WGS_PER_CU / CE_SPLITS;
-    int slots = slots_max < tiles_m ? slots_max : tiles_m;
+    int per_xcd = (tiles_m + CE_XCDS - 1) / CE_XCDS;
+    int mg = cus * Cfg::WGS_PER_CU / (CE_XCDS * CE_SPLITS);      // token tiles in flight per XCD
+    if (mg > per_xcd) mg = per_xcd;
+    if (mg < 1) mg = 1;
     {
         ProfileScope prof(PROF_CE_FWD, st);
-        kernel<<<slots * CE_SPLITS, Cfg::THREADS, LDS, st>>>(g, epi);
+        kernel<<<CE_XCDS * CE_SPLITS * mg, Cfg::THREADS, LDS, st>>>(g, epi);
     }
     return check_launch("lm_head CE forward");
 }
@@ -655,7 +667,9 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
     epi.sc = sc;
     epi.scale = x_s * w_s;
     epi.ncand = prefix_targets ? n_predict + 1 : n_predict;
-    if (int e = g_tuning[5] ? launch_ce_fwd<Cfg256x128k64s2>(g, epi, st) : launch_ce_fwd<MainCfg>(g, epi, st)) return e;
+    if (int e = g_tuning[5] == 1 ? launch_ce_fwd<Cfg256x128k64s2>(g, epi, st)
+              : g_tuning[5] == 2 ? launch_ce_fwd<Cfg256x256k64s4>(g, epi, st)
+                                 : launch_ce_fwd<MainCfg>(g, epi, st)) return e;
     ce_finalize_kernel<<<(M + 255) / 256, 256, 0, st>>>(part, saved_sigma, epi.ca, sc, losses, lse);
     return check_launch("ce_finalize_kernel");
 }
@@ -728,8 +742,9 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         epi.Mc = Mc;
         epi.V = V;
         epi.scale = x_s * w_s;
-        if (int e = g_tuning[5] ? launch_grid_kernel<Cfg256x128k64s2>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")
-                                : launch_grid_kernel<MainCfg>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
+        if (int e = g_tuning[5] == 1 ? launch_grid_kernel<Cfg256x128k64s2>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")
+                  : g_tuning[5] == 2 ? launch_grid_kernel<Cfg256x256k64s4>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")
+                                     : launch_grid_kernel<MainCfg>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
         ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, dl, dl_t);
         if (int e = check_launch("ce_dl_fix_kernel")) return e;

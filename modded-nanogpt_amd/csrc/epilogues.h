@@ -15,7 +15,9 @@ template <class Cfg>
 __device__ __forceinline__ void store_strip_rowmajor_u8(
     const uint32_t (&codes)[Cfg::TN][16], uint8_t* scratch, int lane,
     uint8_t* out, int64_t ld, int grow0 /* global row of strip row 0 */, int gcol0, int R, int C) {
-    constexpr int STRIDE = Cfg::WTN + 16;
+    // padded rows where the wave's scratch allows it (fewer bank conflicts on the 16-byte reads)
+    constexpr int STRIDE = (32 * (Cfg::WTN + 16) <= Cfg::WAVE_SCRATCH) ? Cfg::WTN + 16 : Cfg::WTN;
+    static_assert(32 * STRIDE <= Cfg::WAVE_SCRATCH, "strip does not fit the wave's LDS scratch");
     const int h = lane >> 5, j = lane & 31;
 #pragma unroll
     for (int tn = 0; tn < Cfg::TN; ++tn)
@@ -44,6 +46,7 @@ __device__ __forceinline__ void store_strip_transposed_u8(
     const uint32_t (&packed)[Cfg::TM][4], uint8_t* scratch, int lane,
     uint8_t* out, int64_t ld, int grow0, int gcol0 /* global col of strip col 0 */, int R, int C) {
     constexpr int STRIDE = Cfg::WTM + 16;
+    static_assert(32 * STRIDE <= Cfg::WAVE_SCRATCH, "strip does not fit the wave's LDS scratch");
     const int h = lane >> 5, j = lane & 31;
 #pragma unroll
     for (int tm = 0; tm < Cfg::TM; ++tm)

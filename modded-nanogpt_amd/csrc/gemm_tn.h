@@ -357,195 +357,4 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     epi.end(smem, bid, G);
 }
 
-// ---------------------------------------------------------------------------------------------
-// Software-pipelined variant (two LDS stages, BK = 128), meant for 4 waves per workgroup so that
-// each wave owns a whole SIMD: 128 x 128 per wave, 256 accumulator registers (AGPRs) and room for
-// double-buffered operand fragments.
-//
-// In gemm_tn_kernel every wave leaves the per-k-step barrier at the same moment, reads its operand
-// fragments from LDS, waits, and only then issues MFMAs, so LDS reads and MFMAs do not overlap.
-// Here each wave keeps its MFMA pipe fed:
-//   * fragments are prefetched on a rolling basis: as soon as the MFMAs that consume b[tn] of the
-//     current 64-byte contraction sub-step are issued, the same registers are reloaded with b[tn]
-//     of the next sub-step (A fragments use one spare set);
-//   * the workgroup barrier sits between the two contraction sub-steps of a k-step.  By then all LDS
-//     reads of the current stage are done, so the stage is refilled right after the barrier and the
-//     first fragments of the next k-step are read under the second sub-step's MFMAs.
-// Epilogues that stage data through LDS (Epi::NEEDS_SCRATCH for every tile, Epi::JOB_END_NEEDS_SCRATCH
-// for job ends only) get the current stage as scratch; for them the refill of that stage is issued
-// after the epilogue instead of before it.
-//
-template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
-__global__ __launch_bounds__(Cfg::THREADS) void gemm_tn_kernel_v2(GemmOperands g, Epi epi) {
-    static_assert(Cfg::NSTAGES == 2 && Cfg::KSUB == 2, "pipelined kernel: two stages of 128 contraction bytes");
-    extern __shared__ __attribute__((aligned(1024))) uint8_t smem_all[];
-    static_assert(Epi::EXTRA_LDS % 1024 == 0, "epilogue LDS must keep the stages 1 KiB aligned");
-    uint8_t* const smem = smem_all + Epi::EXTRA_LDS;
-    constexpr int TM = Cfg::TM, TN = Cfg::TN;
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wr = wave / Cfg::WAVES_N, wc = wave % Cfg::WAVES_N;
-    const int bid = blockIdx.x, G = gridDim.x;
-    const int nk = g.K / Cfg::BK;
-    AccCoords<Cfg> coords(wr, wc, lane);
-    Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
-    if (!cur.valid()) return;
-
-    // LDS byte offsets of this lane's first fragment chunk (stage 0, sub-step 0)
-    int frag_a[TM], frag_b[TN];
-    {
-        int h = lane >> 5;
-#pragma unroll
-        for (int t = 0; t < TM; ++t) {
-            int row = wr * Cfg::WTM + t * 32 + (lane & 31);
-            frag_a[t] = row * Cfg::BK + (((h * 2) ^ Cfg::swz(row)) << 4);
-        }
-#pragma unroll
-        for (int t = 0; t < TN; ++t) {
-            int row = wc * Cfg::WTN + t * 32 + (lane & 31);
-            frag_b[t] = Cfg::A_BYTES + row * Cfg::BK + (((h * 2) ^ Cfg::swz(row)) << 4);
-        }
-    }
-    auto read_frag = [&](int slot, int ks, int frag_off) -> v8i {
-        const uint8_t* sp = smem + slot * Cfg::STAGE_BYTES;
-        int o = frag_off ^ (ks * 64);
-        v4i lo = *(const v4i*)(sp + o);
-        v4i hi = *(const v4i*)(sp + (o ^ 16));
-        return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    };
-
-    // operand load state: uniform tile bases + per-lane 32-bit offsets
-    LaneOffsets<Cfg> lo;
-    const uint8_t* a_base = nullptr;
-    const uint8_t* b_base = nullptr;
-    auto set_tile = [&](int tr, int tc) {
-        int r0 = tr * Cfg::BM, c0 = tc * Cfg::BN;
-        a_base = g.A + (int64_t)r0 * g.lda;
-        b_base = g.B + (int64_t)c0 * g.ldb;
-        lo.init(g, wave, lane, r0, c0);
-    };
-    auto issue_loads = [&](int slot, int kt) {
-        uint8_t* sp = smem + slot * Cfg::STAGE_BYTES;
-        const uint8_t* ab = a_base + kt * Cfg::BK;
-        const uint8_t* bb = b_base + kt * Cfg::BK;
-#pragma unroll
-        for (int i = 0; i < Cfg::A_LOADS; ++i)
-            global_to_lds16(ab + lo.a_off[i], sp + (wave + i * Cfg::NWAVES) * 1024);
-#pragma unroll
-        for (int i = 0; i < Cfg::B_LOADS; ++i)
-            global_to_lds16(bb + lo.b_off[i], sp + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
-    };
-
-    // prologue: k-steps 0 and 1 in flight, wait for step 0, read its first fragments
-    StepCursor<Iter> pre(cur, nk);
-    set_tile(pre.it.tr(), pre.it.tc());
-    issue_loads(0, 0);
-    pre.advance();
-    bool pre_new_tile = (pre.kt == 0);
-    if (pre.valid()) {
-        if (pre_new_tile) set_tile(pre.it.tr(), pre.it.tc());
-        issue_loads(1, pre.kt);
-        pre.advance();
-        pre_new_tile = (pre.kt == 0);
-        wait_vmem_le<Cfg::LOADS>();
-    } else {
-        wait_vmem_le<0>();
-    }
-    epi.begin(bid, G, smem_all);
-    wg_barrier();
-
-    v8i a[TM], b[TN], an[TM];
-#pragma unroll
-    for (int t = 0; t < TM; ++t) a[t] = read_frag(0, 0, frag_a[t]);
-#pragma unroll
-    for (int t = 0; t < TN; ++t) b[t] = read_frag(0, 0, frag_b[t]);
-
-    v16f acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-    int slot = 0;
-    while (cur.valid()) {
-        const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
-        if (cur.job_begin()) epi.template job_begin<Cfg>(c0);
-        for (int kt = 0; kt < nk; ++kt) {
-            const bool last = (kt + 1 == nk);
-            // ---- sub-step 0: MFMAs on the fragments in registers, rolling prefetch of sub-step 1
-#pragma unroll
-            for (int t = 0; t < TM; ++t) an[t] = read_frag(slot, 1, frag_a[t]);
-#pragma unroll
-            for (int tn = 0; tn < TN; ++tn) {
-#pragma unroll
-                for (int tm = 0; tm < TM; ++tm)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
-                b[tn] = read_frag(slot, 1, frag_b[tn]);
-            }
-#pragma unroll
-            for (int t = 0; t < TM; ++t) a[t] = an[t];
-            // ---- every wave is past its reads of this stage; the next k-step has landed
-            wait_vmem_le<0>();
-            wg_barrier();                            // includes lgkmcnt(0): this wave's LDS reads are done
-            const bool refill_late = last && (Epi::NEEDS_SCRATCH || (Epi::JOB_END_NEEDS_SCRATCH && cur.job_end()));
-            if (!refill_late && pre.valid()) {
-                if (pre_new_tile) set_tile(pre.it.tr(), pre.it.tc());
-                if (!(g.ablate & 1)) issue_loads(slot, pre.kt);
-                pre.advance();
-                pre_new_tile = (pre.kt == 0);
-            }
-            // ---- sub-step 1, prefetching the first fragments of the next k-step from the other stage
-            if (!last) {
-#pragma unroll
-                for (int t = 0; t < TM; ++t) an[t] = read_frag(slot ^ 1, 0, frag_a[t]);
-#pragma unroll
-                for (int tn = 0; tn < TN; ++tn) {
-#pragma unroll
-                    for (int tm = 0; tm < TM; ++tm)
-                        acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
-                    b[tn] = read_frag(slot ^ 1, 0, frag_b[tn]);
-                }
-#pragma unroll
-                for (int t = 0; t < TM; ++t) a[t] = an[t];
-            } else {
-#pragma unroll
-                for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-                    for (int tm = 0; tm < TM; ++tm)
-                        acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
-                // tile finished: epilogue, then pick up the next tile's first fragments
-                uint8_t* scratch_stage = smem + slot * Cfg::STAGE_BYTES;   // free only if the refill was postponed
-                epi.template tile<Cfg>(acc, r0, c0, coords, scratch_stage + wave * Cfg::WAVE_SCRATCH, lane);
-                if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, scratch_stage);
-                if (refill_late) {
-                    wg_barrier();          // every wave is done with the scratch
-                    if (pre.valid()) {
-                        if (pre_new_tile) set_tile(pre.it.tr(), pre.it.tc());
-                        issue_loads(slot, pre.kt);
-                        pre.advance();
-                        pre_new_tile = (pre.kt == 0);
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-#pragma unroll
-                for (int t = 0; t < TM; ++t) a[t] = read_frag(slot ^ 1, 0, frag_a[t]);
-#pragma unroll
-                for (int t = 0; t < TN; ++t) b[t] = read_frag(slot ^ 1, 0, frag_b[t]);
-            }
-            slot ^= 1;
-        }
-        cur.advance();
-    }
-    wg_barrier();
-    epi.end(smem, bid, G);
-}
-
 }  // namespace ngpt

@@ -7,44 +7,29 @@ namespace ngpt {
 
 // 256 x 256 tile, 8 waves as 4 (rows) x 2 (cols): each wave owns 64 x 128 = 2 x 4 MFMA tiles.
 using MainCfg = TileCfg<256, 256, 4, 2, 128, 2>;
-// Alternatives selectable at run time through ngpt_tuning_set(0, id) (tuning aid).
+// Alternatives selectable at run time through ngpt_tuning_set(0, id) (tuning aid; slower on MI355X
+// for the shapes of this path).
 using Cfg256x256k64s4 = TileCfg<256, 256, 4, 2, 64, 4>;     // id 1: four 32 KiB stages
-using Cfg256x128k64s3 = TileCfg<256, 128, 2, 2, 64, 3, 2>;  // id 2: 4 waves, 72 KiB: two workgroups per CU
-using Cfg256x128k128s2 = TileCfg<256, 128, 2, 2, 128, 2>;   // id 3: 4 waves, 96 KiB
-using Cfg128x128k128s2 = TileCfg<128, 128, 2, 2, 128, 2, 2>;   // id 4: 4 waves, 64 KiB: two workgroups per CU
 using Cfg256x128k64s2 = TileCfg<256, 128, 2, 2, 64, 2, 2>;  // id 5: 4 waves, 48 KiB: two workgroups per CU
-using Cfg128x256k64s3 = TileCfg<128, 256, 2, 2, 64, 3, 2>;  // id 7: as id 2 with the tile turned
-using Cfg256x256w4 = TileCfg<256, 256, 2, 2, 128, 2>;       // id 6: 4 waves of 128 x 128, software-pipelined
 
-// [0] GEMM tile config id, [1] workgroups per CU for the persistent grid, [2] ablation bits (timing
-// aid), [3] 2 = use the software-pipelined kernel where one exists, [4] split-K factor of ngpt_gemm_fp8_tn,
-// [5] 1 = fused CE kernels use the 256x128 two-workgroups-per-CU tile, [6] 1 = split-K in the CE backward GEMMs
+// Tuning keys: [0] GEMM tile config id, [2] ablation bits (timing aid),
+// [4] split-K factor of ngpt_gemm_fp8_tn, [5] fused CE kernels: 1 = id 5 tile, 2 = id 1 tile,
+// [6] 1 = split-K in the CE backward GEMMs
 extern int g_tuning[8];
 
 template <class Cfg, int FA, int FB, class Epi>
-auto pick_kernel() {
-    if constexpr (Cfg::NSTAGES == 2 && Cfg::KSUB == 2 && Cfg::NWAVES == 4) {
-        return g_tuning[3] == 2 ? gemm_tn_kernel_v2<Cfg, FA, FB, Epi, GridIter> : gemm_tn_kernel<Cfg, FA, FB, Epi, GridIter>;
-    } else {
-        return gemm_tn_kernel<Cfg, FA, FB, Epi, GridIter>;
-    }
-}
-
-template <class Cfg, int FA, int FB, class Epi>
 int launch_gemm_fmt(const GemmOperands& g, const Epi& epi, hipStream_t st, int max_grid) {
-    auto kernel = pick_kernel<Cfg, FA, FB, Epi>();
+    auto kernel = gemm_tn_kernel<Cfg, FA, FB, Epi, GridIter>;
     constexpr int LDS = Cfg::SMEM_BYTES + Epi::EXTRA_LDS;
-    static bool configured[2] = {false, false};
-    if (!configured[g_tuning[3] == 2 ? 1 : 0]) {
+    static bool configured = false;
+    if (!configured) {
         if (int e = allow_lds(kernel, LDS)) return e;
-        configured[g_tuning[3] == 2 ? 1 : 0] = true;
+        configured = true;
     }
     int tiles = ((g.R + Cfg::BM - 1) / Cfg::BM) * ((g.C + Cfg::BN - 1) / Cfg::BN) * (g.splits < 1 ? 1 : g.splits);
     int cus = num_cus();
     if (cus <= 0) return fail(NGPT_EINVAL, "no HIP device");
-    int per_cu = g_tuning[1] > 0 ? g_tuning[1] : 2;
-    if ((int64_t)per_cu * (Cfg::SMEM_BYTES + Epi::EXTRA_LDS) > 160 * 1024) per_cu = 1;
-    int slots = cus * per_cu;
+    int slots = cus * Cfg::WGS_PER_CU;      // as many workgroups as can be resident at once
     int grid = tiles < slots ? tiles : slots;
     if (max_grid > 0 && grid > max_grid) grid = max_grid;
     kernel<<<grid, Cfg::THREADS, LDS, st>>>(g, epi);
@@ -64,12 +49,7 @@ template <class Cfg /* default */, class Epi>
 int launch_gemm(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {
     switch (g_tuning[0]) {
         case 1: return launch_gemm_cfg<Cfg256x256k64s4>(g, fa, fb, epi, st, max_grid);
-        case 2: return launch_gemm_cfg<Cfg256x128k64s3>(g, fa, fb, epi, st, max_grid);
-        case 3: return launch_gemm_cfg<Cfg256x128k128s2>(g, fa, fb, epi, st, max_grid);
-        case 4: return launch_gemm_cfg<Cfg128x128k128s2>(g, fa, fb, epi, st, max_grid);
         case 5: return launch_gemm_cfg<Cfg256x128k64s2>(g, fa, fb, epi, st, max_grid);
-        case 6: return launch_gemm_cfg<Cfg256x256w4>(g, fa, fb, epi, st, max_grid);
-        case 7: return launch_gemm_cfg<Cfg128x256k64s3>(g, fa, fb, epi, st, max_grid);
         default: return launch_gemm_cfg<Cfg>(g, fa, fb, epi, st, max_grid);
     }
 }

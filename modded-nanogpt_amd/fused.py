@@ -28,6 +28,49 @@ def transpose_copy(src: Tensor, dst: Tensor) -> None:
                "ngpt_transpose_u8")
 
 
+def transpose_add(src: Tensor, dst: Tensor) -> None:
+    """dst (N, M) += src (M, N).T -- reference triton_kernels.py:882-903 (tied embedding / lm_head gradients)."""
+    assert src.ndim == 2 and dst.ndim == 2
+    M, N = src.shape
+    assert dst.shape == (N, M), f"Expected dst shape ({N}, {M}), got {dst.shape}"
+    assert src.is_contiguous() and dst.is_contiguous() and src.dtype == dst.dtype
+    assert src.dtype in (torch.bfloat16, torch.float32)
+    ops._gpu(src, dst)
+    _lib.check(_lib.load().ngpt_transpose_add(src.data_ptr(), M, N, dst.data_ptr(), src.element_size(),
+                                              ops._stream(src)), "ngpt_transpose_add")
+
+
+def reduce_mlp_activation_scales(partial_amax: Tensor, scales: Tensor, headroom: float = 1.25) -> None:
+    """scales[l] = max(partial_amax[l].max(), 1e-12) * headroom / 448 -- reference triton_kernels.py:732-745."""
+    num_layers, partial_count = partial_amax.shape
+    assert scales.numel() >= num_layers
+    assert partial_amax.dtype == torch.float32 and scales.dtype == torch.float32 and partial_amax.stride(1) == 1
+    ops._gpu(partial_amax, scales)
+    _lib.check(_lib.load().ngpt_reduce_scales(partial_amax.data_ptr(), partial_amax.stride(0), num_layers,
+                                              partial_count, headroom, scales.data_ptr(), ops._stream(scales)),
+               "ngpt_reduce_scales")
+
+
+def quantize_transpose_mlp_down_weights(weights: Tensor, output_storage: Tensor, next_scales: Tensor,
+                                        used_scales: Tensor, partial_amax: Tensor, headroom: float = 1.12) -> None:
+    """Delayed-scale e4m3 copy of the MLP down projections, stored transposed, plus the next step's
+    scales -- reference triton_kernels.py:748-779.  weights [L, H, D] bf16 (a strided view of the MLP
+    bank is fine), output_storage [L, D, H] e4m3, next_scales / used_scales [L], partial_amax [L, tiles]."""
+    num_layers, hidden_dim, model_dim = weights.shape
+    assert output_storage.shape == (num_layers, model_dim, hidden_dim)
+    num_tiles = -(-hidden_dim // 64) * -(-model_dim // 64)
+    assert partial_amax.shape == (num_layers, num_tiles)
+    assert weights.dtype == torch.bfloat16 and weights.stride(2) == 1 and weights.stride(1) == model_dim
+    assert output_storage.is_contiguous() and partial_amax.is_contiguous()
+    ops._gpu(weights, output_storage, next_scales, used_scales, partial_amax)
+    _lib.check(_lib.load().ngpt_quant_transpose_down(weights.data_ptr(), num_layers, hidden_dim, model_dim,
+                                                     weights.stride(0), next_scales.data_ptr(),
+                                                     output_storage.data_ptr(), used_scales.data_ptr(),
+                                                     partial_amax.data_ptr(), ops._stream(weights)),
+               "ngpt_quant_transpose_down")
+    reduce_mlp_activation_scales(partial_amax, next_scales, headroom=headroom)
+
+
 def linear_relu_square(a, b, aux=None, a_f8=None, b_f8=None, dequant_scale_ptr=None,
                        activation_scale=None, partial_amax=None):
     """Reference launcher triton_kernels.py:576-665.

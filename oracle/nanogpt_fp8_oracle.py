@@ -148,6 +148,24 @@ def quantize_up_weights(w_fc: Tensor):
     return w_f8, scales.float()
 
 
+def reduce_mlp_activation_scales(partial_amax: Tensor, headroom: float = 1.25) -> Tensor:
+    """reduce_mlp_activation_scales_kernel -- triton_kernels.py:502-519.  partial_amax [L, P] -> scales [L]."""
+    return partial_amax.float().amax(dim=1).clamp(min=1.0e-12) * (headroom / E4M3_MAX)
+
+
+def quantize_transpose_mlp_down_weights(weights: Tensor, next_scales: Tensor, headroom: float = 1.12):
+    """quantize_transpose_mlp_down_weights(_kernel) -- triton_kernels.py:522-565, 748-779.
+    weights [L, H, D] bf16, next_scales [L] (the scales this call quantises with).
+    Returns (w_f8_t [L, D, H] e4m3, used_scales [L], new_next_scales [L], partial_amax [L, tiles])."""
+    L, H, D = weights.shape
+    w = weights.float()
+    q = (w / next_scales.float().view(L, 1, 1)).clamp(-E4M3_MAX, E4M3_MAX).to(E4M3)
+    th, td = -(-H // 64), -(-D // 64)
+    pad = F.pad(w.abs(), (0, td * 64 - D, 0, th * 64 - H))
+    partial = pad.view(L, th, 64, td, 64).amax(dim=(2, 4)).reshape(L, th * td)
+    return q.transpose(1, 2).contiguous(), next_scales.float().clone(), reduce_mlp_activation_scales(partial, headroom), partial
+
+
 # ----------------------------------------------------------------------------
 # a7, a8: fused linear + ReLU^2 and the MLP autograd function
 

@@ -123,3 +123,25 @@ def test_package_never_imports_the_oracle():
     for p in (ROOT / "modded-nanogpt_amd").rglob("*"):
         if p.suffix in (".py", ".hip", ".h") and p.is_file():
             assert "oracle" not in p.read_text(), p
+
+
+def test_shipped_gemm_kernels_do_not_spill(amd, tmp_path):
+    """The 8-wave GEMM kernels must fit 256 VGPRs without spilling: one scratch reload inside the
+    k-loop makes the compiler wait for all outstanding operand loads and serialises them."""
+    import re
+    import subprocess
+    from modded_nanogpt_amd import build as b
+    src = b.CSRC / "ce.hip"
+    cmd = [b.hipcc_path(), *[f for f in b.HIPCC_FLAGS if f != "-shared"], "-I", str(ROOT / "include"),
+           "-S", "--cuda-device-only", "-o", str(tmp_path / "ce.s"), str(src)]
+    subprocess.run(cmd, check=True, capture_output=True)
+    text = (tmp_path / "ce.s").read_text()
+    seen = 0
+    for block in text.split("- .agpr_count:")[1:]:
+        name = re.search(r"\.name:\s+(\S+)", block).group(1)
+        if "gemm_tn_kernel" in name and "Li256ELi256ELi4ELi2ELi128ELi2ELi1" in name:
+            spills = int(re.search(r"\.vgpr_spill_count:\s+(\d+)", block).group(1))
+            vgprs = int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1))
+            assert spills == 0 and vgprs <= 256, (name, vgprs, spills)
+            seen += 1
+    assert seen >= 2          # fused CE forward + dlogits kernels

@@ -326,3 +326,58 @@ def test_fused_lmhead_ce_reduces_to_cross_entropy(amd, oracle):
     ref = oracle.softcap_ce_closed_form((xq @ wq.T).float(), t)
     assert abs(float(losses.mean().cpu() - ref.mean())) < 5e-3
     assert (losses.cpu() - ref).abs().max() < 0.15
+
+
+# ------------------------------------------------------------------------------------------ delayed-scaling helpers
+def test_reduce_scales_and_down_weight_requantiser(amd, oracle):
+    g = torch.Generator().manual_seed(31)
+    L, H, D = 3, 3072, 768
+    bank = (torch.randn(L, 2, H, D, generator=g) * 0.02).bfloat16()
+    w = bank[:, 1]                                                  # strided view, as the reference passes it
+    scales = w.float().abs().amax(dim=(1, 2)) / 448 * torch.tensor([1.0, 0.9, 1.3])
+    q_ref, used_ref, next_ref, partial_ref = oracle.quantize_transpose_mlp_down_weights(w, scales, headroom=1.12)
+    bank_d = dev(bank)
+    out = torch.empty((L, D, H), dtype=E4M3, device="cuda")
+    nxt, used = dev(scales.clone()), torch.zeros(L, device="cuda")
+    partial = torch.empty((L, (H // 64) * (D // 64)), device="cuda")
+    amd.quantize_transpose_mlp_down_weights(bank_d[:, 1], out, nxt, used, partial, headroom=1.12)
+    assert torch.equal(u8(out), u8(q_ref))                          # bit-exact, clamped at +-448
+    assert torch.equal(used.cpu(), used_ref) and torch.equal(partial.cpu(), partial_ref)
+    assert torch.allclose(nxt.cpu(), next_ref, rtol=1e-6)
+    p = torch.rand(11, 256, generator=g)
+    p[3] = 0
+    s = torch.zeros(12, device="cuda")
+    amd.reduce_mlp_activation_scales(dev(p), s, headroom=1.80)
+    assert torch.allclose(s[:11].cpu(), oracle.reduce_mlp_activation_scales(p, 1.80), rtol=1e-6) and s[11] == 0
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+def test_transpose_add(amd, dt):
+    g = torch.Generator().manual_seed(32)
+    for (M, N) in [(64, 64), (100, 36), (768, 1000)]:
+        src = torch.randn(M, N, generator=g).to(dt)
+        dst = torch.randn(N, M, generator=g).to(dt)
+        want = (dst.float() + src.float().T).to(dt)
+        d = dev(dst)
+        amd.transpose_add(dev(src), d)
+        assert torch.equal(d.cpu(), want)
+
+
+def test_mlp_forward_with_fp8_down_projection(amd, oracle):
+    """FusedLinearReLUSquareFunction with W2_f8: EMIT_FP8 epilogue + FP8 down projection (record #89 path)."""
+    M, D, H = 1024, 256, 1024
+    x, w_fc, w_proj_t = oracle.make_cfg2(seed=33, M=M, D=D, H=H)
+    w_f8, scales = oracle.quantize_up_weights(w_fc[None])
+    x_f8, dequant = oracle.mlp_input_quant(x, scales[0:1])
+    post_ref = oracle.fc_relu2_fwd(x_f8, w_f8[0], dequant)
+    act = torch.tensor([float(post_ref.float().max()) * 1.8 / 448])
+    w2_scale = w_proj_t.float().abs().max().reshape(1) / 448
+    w2q_t, _, _, _ = oracle.quantize_transpose_mlp_down_weights(w_proj_t[None], w2_scale)     # [1, D, H]
+    w2_f8 = w2q_t[0].T                                                                        # (H, D) view, H contiguous
+    out_ref, _, _ = oracle.mlp_fwd(x[None], w_fc, w_proj_t, w_f8[0], dequant, x_f8[None], w2_f8, w2_scale, act)
+    partial = torch.zeros(256, device="cuda")
+    out = amd.ReLUSqrdMLP(dev(x[None]), dev(w_fc), dev(w_proj_t), dev(w_f8[0]), dev(dequant), dev(x_f8[None]),
+                          dev(w2q_t)[0].T, dev(w2_scale), dev(act), partial)
+    assert out.shape == (1, M, D) and out.dtype == torch.bfloat16
+    assert_close_gemm(out, out_ref)
+    assert float(partial.max()) > 0

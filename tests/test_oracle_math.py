@@ -233,3 +233,23 @@ def test_lm_head_ce_backward_matches_autograd(oracle):
     dx, dw = oracle.lm_head_ce_bwd(ctx)
     assert n == 96 and torch.allclose(l_c, losses, atol=1e-6) and torch.equal(dx_c, dx)
     assert rel_err(dw_c, dw) < 1e-6
+
+
+def test_down_projection_requantiser_oracle(oracle):
+    """quantize_transpose_mlp_down_weights / reduce_mlp_activation_scales against element-wise statements."""
+    g = torch.Generator().manual_seed(13)
+    L, H, D = 3, 192, 128
+    w = (torch.randn(L, H, D, generator=g) * 0.02).bfloat16()
+    scales = w.float().abs().amax(dim=(1, 2)) / 448 * 0.9          # a stale (too small) scale: some values clamp
+    q_t, used, nxt, partial = oracle.quantize_transpose_mlp_down_weights(w, scales, headroom=1.12)
+    assert q_t.shape == (L, D, H) and partial.shape == (L, 3 * 2) and torch.equal(used, scales)
+    for l, h, d in [(0, 0, 0), (1, 100, 77), (2, 191, 127)]:
+        want = max(-448.0, min(448.0, float(w[l, h, d]) / float(scales[l])))
+        assert float(q_t[l, d, h]) == float(torch.tensor(want).to(torch.float8_e4m3fn))
+    assert float(q_t.float().abs().max()) == 448.0                 # clamped, not NaN
+    assert torch.isfinite(q_t.float()).all()
+    assert torch.allclose(partial.amax(dim=1), w.float().abs().amax(dim=(1, 2)))
+    assert torch.allclose(nxt, w.float().abs().amax(dim=(1, 2)) * 1.12 / 448)
+    p = torch.tensor([[0.0, 3.0, 1.0], [0.0, 0.0, 0.0]])
+    s = oracle.reduce_mlp_activation_scales(p, headroom=1.8)
+    assert torch.allclose(s, torch.tensor([3.0 * 1.8 / 448, 1e-12 * 1.8 / 448]))
