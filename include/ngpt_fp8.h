@@ -121,6 +121,14 @@ int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, 
                       void* post_bf16, void* post_f8, const float* act_scale,
                       float* partial_amax, int n_partials, void* stream);
 
+/* ---- MLP backward through ReLU^2 ----------------------------------------------------------
+ * linear_relu_square_kernel with FORWARD = False, triton_kernels.py:472-476, 493-496, called at :726.
+ * dy [M, D] bf16, w2 [H, D] bf16, post [M, H] bf16 ->
+ * dpre [M, H] = bf16(2 * bf16(dy . w2^T) * sqrt(post)), a bf16 MFMA GEMM (fp32 accumulate) with the
+ * product fused into the epilogue.  D % 64 == 0. */
+int ngpt_fc_relu2_bwd_dpre(const void* dy_bf16, const void* w2_bf16, const void* post_bf16, int M, int H, int D,
+                           void* dpre_bf16, void* stream);
+
 /* ---- delayed-scaling bookkeeping of the FP8 down projection, tied-embedding gradient add -----
  * scales[l] = max(max_i partial_amax[l * partial_stride + i], 1e-12) * headroom / 448:
  * reduce_mlp_activation_scales(_kernel), triton_kernels.py:502-519, 732-745. */

@@ -31,6 +31,7 @@ SIGNATURES = {
     "ngpt_mm_bwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
     "ngpt_mm_bwd": (_I, [_P, _P, _P, _I, _I, _I, _F, _F, _F, _P, _P, _I, _P, _L, _P]),
     "ngpt_fc_relu2_fwd": (_I, [_P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _P]),
+    "ngpt_fc_relu2_bwd_dpre": (_I, [_P, _P, _P, _I, _I, _I, _P, _P]),
     "ngpt_reduce_scales": (_I, [_P, _L, _I, _I, _F, _P, _P]),
     "ngpt_quant_transpose_down": (_I, [_P, _I, _I, _I, _L, _P, _P, _P, _P, _P]),
     "ngpt_transpose_add": (_I, [_P, _I, _I, _P, _I, _P]),

@@ -11,7 +11,8 @@ typedef int   v8i  __attribute__((ext_vector_type(8)));
 typedef float v4f  __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-enum : int { FMT_E4M3 = 0, FMT_E5M2 = 1 };
+enum : int { FMT_E4M3 = 0, FMT_E5M2 = 1, FMT_BF16 = 2 };   // FMT_BF16: both operands bf16, contraction counted in bytes
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 constexpr int kWave = 64;
 

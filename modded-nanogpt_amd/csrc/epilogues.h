@@ -111,6 +111,54 @@ struct EpiStoreBf16 {
     }
 };
 
+// dpre[r, c] = bf16(2 * bf16(acc) * sqrt(post[r, c])): the backward of relu(pre)^2 through the down
+// projection, with relu(pre) recovered as sqrt(post) (linear_relu_square_kernel, FORWARD = False).
+struct EpiDpre {
+    uint16_t* out;
+    const uint16_t* post;
+    int64_t ld;
+    int R, C;
+    static constexpr int EXTRA_LDS = 0;
+    static constexpr bool NEEDS_SCRATCH = false;
+    static constexpr bool JOB_END_NEEDS_SCRATCH = false;
+    __device__ void begin(int, int, uint8_t*) {}
+    __device__ void end(uint8_t*, int, int) {}
+    template <class Cfg>
+    __device__ void job_begin(int) {}
+    template <class Cfg>
+    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
+                         uint8_t*, int) {
+        const int64_t tile_off = (int64_t)r0 * ld + c0;
+        uint16_t* origin = out + tile_off;
+        const uint16_t* porigin = post + tile_off;
+        const uint32_t lane_off = (uint32_t)co.row_base * (uint32_t)ld + (uint32_t)co.col_base;
+        const int rlim = R - r0 - co.row_base, clim = C - c0 - co.col_base;
+        const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
+#pragma unroll
+        for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < Cfg::TN; ++tn) {
+#pragma unroll
+                for (int v = 0; v < 16; v += 2) {
+                    const int dr = tm * 32 + 8 * (v >> 2) + (v & 3), dc = tn * 32;
+                    const int64_t uo = (int64_t)dr * ld + dc;
+                    const bool ok0 = full || (dr < rlim && dc < clim), ok1 = full || (dr + 1 < rlim && dc < clim);
+                    float p0 = ok0 ? bf16_bits_to_f32(porigin[uo + lane_off]) : 0.0f;
+                    float p1 = ok1 ? bf16_bits_to_f32(porigin[uo + lane_off + (uint32_t)ld]) : 0.0f;
+                    uint32_t c01 = cvt_pk_bf16(acc[tm][tn][v], acc[tm][tn][v + 1]);        // c = bf16(acc)
+                    float d0 = 2.0f * bf16_bits_to_f32(c01 & 0xffffu) * __fsqrt_rn(p0);
+                    float d1 = 2.0f * bf16_bits_to_f32(c01 >> 16) * __fsqrt_rn(p1);
+                    uint32_t pk = cvt_pk_bf16(d0, d1);
+                    if (ok0) origin[uo + lane_off] = (uint16_t)pk;
+                    if (ok1) origin[uo + lane_off + (uint32_t)ld] = (uint16_t)(pk >> 16);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    }
+};
+
 // Mainloop-only timing aid: keeps the accumulators alive but writes (practically) nothing.
 struct EpiDiscard {
     float* out;   // >= 4 floats; workgroup 0 leaves its shader-clock and 100 MHz wall-clock tick counts in out[2], out[3]

@@ -244,6 +244,18 @@ extern "C" int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f
     return gemm_store(x_f8_t, FMT_E4M3, M, g_f8_t, FMT_E5M2, M, K, N, M, x_s * grad_s, dw_kn_f32, N, 1, st, 1);
 }
 
+// ------------------------------------------------------------------------------------------ dpre (bf16)
+extern "C" int ngpt_fc_relu2_bwd_dpre(const void* dy_bf16, const void* w2_bf16, const void* post_bf16, int M, int H, int D,
+                                      void* dpre_bf16, void* stream) {
+    if (!dy_bf16 || !w2_bf16 || !post_bf16 || !dpre_bf16) return fail(NGPT_EINVAL, "ngpt_fc_relu2_bwd_dpre: null pointer");
+    if (M <= 0 || H <= 0 || D <= 0) return fail(NGPT_EINVAL, "ngpt_fc_relu2_bwd_dpre: empty problem M=%d H=%d D=%d", M, H, D);
+    if (D % 64) return fail(NGPT_EALIGN, "ngpt_fc_relu2_bwd_dpre: D=%d must be a multiple of 64", D);
+    // bf16 operands: the loader works in bytes, so the contraction length and row strides are 2 * D
+    GemmOperands g{(const uint8_t*)dy_bf16, (const uint8_t*)w2_bf16, 2 * (int64_t)D, 2 * (int64_t)D, M, H, 2 * D, 1, 0};
+    EpiDpre epi{(uint16_t*)dpre_bf16, (const uint16_t*)post_bf16, H, M, H};
+    return launch_gemm_fmt<MainCfg, FMT_BF16, FMT_BF16>(g, epi, (hipStream_t)stream, 0);
+}
+
 // ------------------------------------------------------------------------------------------ fc + relu^2
 extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, int M, int N, int K,
                                  void* post_bf16, void* post_f8, const float* act_scale,

@@ -135,16 +135,18 @@ struct TileMainloop {
         wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         wr = wave / Cfg::WAVES_N;
         wc = wave % Cfg::WAVES_N;
-        int h = lane >> 5;
+        // first 16-byte chunk of this lane's operand fragment: fp8 MFMAs (32x32x64) take 32 bytes per
+        // lane (chunks 2h, 2h+1), the bf16 MFMA (32x32x16) takes 16 bytes (chunk h)
+        int q0 = (AFMT == FMT_BF16) ? (lane >> 5) : (lane >> 5) * 2;
 #pragma unroll
         for (int t = 0; t < Cfg::TM; ++t) {
             int row = wr * Cfg::WTM + t * 32 + (lane & 31);
-            frag_a[t] = row * Cfg::BK + (((h * 2) ^ Cfg::swz(row)) << 4);
+            frag_a[t] = row * Cfg::BK + ((q0 ^ Cfg::swz(row)) << 4);
         }
 #pragma unroll
         for (int t = 0; t < Cfg::TN; ++t) {
             int row = wc * Cfg::WTN + t * 32 + (lane & 31);
-            frag_b[t] = Cfg::A_BYTES + row * Cfg::BK + (((h * 2) ^ Cfg::swz(row)) << 4);
+            frag_b[t] = Cfg::A_BYTES + row * Cfg::BK + ((q0 ^ Cfg::swz(row)) << 4);
         }
     }
 
@@ -173,6 +175,23 @@ struct TileMainloop {
     template <bool FIRST>
     __device__ void compute(const uint8_t* smem, int stage, v16f (&acc)[Cfg::TM][Cfg::TN]) {
         const uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
+        if constexpr (AFMT == FMT_BF16) {
+            // bf16 operands: 32 contraction bytes (16 elements) per MFMA, one 16-byte chunk per lane
+#pragma unroll
+            for (int ks = 0; ks < Cfg::BK / 32; ++ks) {
+                v8bf a[Cfg::TM], b[Cfg::TN];
+#pragma unroll
+                for (int t = 0; t < Cfg::TM; ++t) a[t] = *(const v8bf*)(s + (frag_a[t] ^ (ks * 32)));
+#pragma unroll
+                for (int t = 0; t < Cfg::TN; ++t) b[t] = *(const v8bf*)(s + (frag_b[t] ^ (ks * 32)));
+#pragma unroll
+                for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < Cfg::TN; ++tn)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[tm], b[tn], acc[tm][tn], 0, 0, 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int ks = 0; ks < Cfg::KSUB; ++ks) {
             v8i a[Cfg::TM], b[Cfg::TN];
@@ -197,10 +216,10 @@ struct TileMainloop {
                     if (FIRST && ks == 0) {
                         const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                         acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            a[tm], b[tn], zero, AFMT, BFMT, 0, 0, 0, 0);
+                            a[tm], b[tn], zero, AFMT & 1, BFMT & 1, 0, 0, 0, 0);
                     } else {
                         acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            a[tm], b[tn], acc[tm][tn], AFMT, BFMT, 0, 0, 0, 0);
+                            a[tm], b[tn], acc[tm][tn], AFMT & 1, BFMT & 1, 0, 0, 0, 0);
                     }
                 }
         }

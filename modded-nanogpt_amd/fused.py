@@ -94,8 +94,7 @@ def linear_relu_square(a, b, aux=None, a_f8=None, b_f8=None, dequant_scale_ptr=N
         c = a @ b.T                                     # bf16 GEMM (hipBLASLt), fp32 accumulate
         r = torch.clamp_min(c, 0)
         return r * r
-    c = a @ b.T
-    return (2 * c.float() * torch.sqrt(aux.float())).to(a.dtype)
+    return ops.fc_relu2_bwd_dpre(a.contiguous(), b.contiguous(), aux.contiguous())
 
 
 class FusedLinearReLUSquareFunction(torch.autograd.Function):

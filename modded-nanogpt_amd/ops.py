@@ -334,6 +334,26 @@ def _(x_f8, w_f8, dequant_scale, activation_scale, partial_amax):
             torch.empty((M, N), dtype=E4M3, device=x_f8.device))
 
 
+@torch.library.custom_op("nanogpt::fc_relu2_bwd_dpre", mutates_args=())
+def fc_relu2_bwd_dpre(dy: Tensor, w2: Tensor, post: Tensor) -> Tensor:
+    """dpre [M,H] = bf16(2 * bf16(dy @ w2.T) * sqrt(post)) for dy [M,D], w2 [H,D], post [M,H], all bf16."""
+    _gpu(dy, w2, post)
+    assert dy.dtype == w2.dtype == post.dtype == torch.bfloat16
+    assert dy.is_contiguous() and w2.is_contiguous() and post.is_contiguous()
+    M, D = dy.shape
+    H = w2.shape[0]
+    assert w2.shape[1] == D and post.shape == (M, H)
+    dpre = torch.empty((M, H), dtype=torch.bfloat16, device=dy.device)
+    _lib.check(_lib.load().ngpt_fc_relu2_bwd_dpre(_p(dy), _p(w2), _p(post), M, H, D, _p(dpre), _stream(dy)),
+               "ngpt_fc_relu2_bwd_dpre")
+    return dpre
+
+
+@fc_relu2_bwd_dpre.register_fake
+def _(dy, w2, post):
+    return torch.empty_like(post)
+
+
 # ------------------------------------------------------------------------------------------------
 # Building blocks exposed for callers and tests (plain functions, not registered ops)
 
