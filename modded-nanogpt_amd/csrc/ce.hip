@@ -667,9 +667,7 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
     epi.sc = sc;
     epi.scale = x_s * w_s;
     epi.ncand = prefix_targets ? n_predict + 1 : n_predict;
-    if (int e = g_tuning[5] == 1 ? launch_ce_fwd<Cfg256x128k64s2>(g, epi, st)
-              : g_tuning[5] == 2 ? launch_ce_fwd<Cfg256x256k64s4>(g, epi, st)
-                                 : launch_ce_fwd<MainCfg>(g, epi, st)) return e;
+    if (int e = launch_ce_fwd<MainCfg>(g, epi, st)) return e;
     ce_finalize_kernel<<<(M + 255) / 256, 256, 0, st>>>(part, saved_sigma, epi.ca, sc, losses, lse);
     return check_launch("ce_finalize_kernel");
 }
@@ -742,9 +740,7 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         epi.Mc = Mc;
         epi.V = V;
         epi.scale = x_s * w_s;
-        if (int e = g_tuning[5] == 1 ? launch_grid_kernel<Cfg256x128k64s2>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")
-                  : g_tuning[5] == 2 ? launch_grid_kernel<Cfg256x256k64s4>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")
-                                     : launch_grid_kernel<MainCfg>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
+        if (int e = launch_grid_kernel<MainCfg>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
         ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, dl, dl_t);
         if (int e = check_launch("ce_dl_fix_kernel")) return e;

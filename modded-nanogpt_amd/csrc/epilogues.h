@@ -161,6 +161,7 @@ struct EpiDpre {
 
 // Mainloop-only timing aid: keeps the accumulators alive but writes (practically) nothing.
 struct EpiDiscard {
+    static constexpr bool ABLATABLE = true;
     float* out;   // >= 4 floats; workgroup 0 leaves its shader-clock and 100 MHz wall-clock tick counts in out[2], out[3]
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;

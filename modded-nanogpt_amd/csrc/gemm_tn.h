@@ -22,6 +22,7 @@
 // Any permutation of the contraction bytes is harmless as long as A and B use the same one.
 #pragma once
 #include "common.h"
+#include <type_traits>
 
 namespace ngpt {
 
@@ -170,13 +171,28 @@ struct TileMainloop {
             global_to_lds16(bb + lo.b_off[i], s + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
     }
 
-    // One k-step of MFMAs.  FIRST: this is the first k-step of a tile, so its first sub-step starts the
-    // accumulators from the constant 0 (the C operand of the MFMA) instead of from zeroed registers.
-    template <bool FIRST>
-    __device__ void compute(const uint8_t* smem, int stage, v16f (&acc)[Cfg::TM][Cfg::TN]) {
+    // Operand fragment of one 32-row MFMA tile for contraction sub-step ks (two 16-byte chunks).
+    __device__ __forceinline__ v8i frag(const uint8_t* s, int off, int ks) const {
+        int o = off ^ (ks * 64);
+        v4i lo = *(const v4i*)(s + o);
+        v4i hi = *(const v4i*)(s + (o ^ 16));
+        return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+
+    // One k-step of MFMAs.  The LDS reads are software-pipelined against the MFMAs by hand: the A
+    // fragments and the first B fragment of a sub-step are read while the previous sub-step's last
+    // MFMAs run, every further B fragment while the MFMAs of the one before it run, and scheduling
+    // barriers keep the compiler from hoisting all reads to the top (which would leave the matrix
+    // pipe idle for a full LDS round trip per sub-step).  `after_first` runs once, behind the first
+    // group of MFMAs of the k-step: the kernel issues the next operand loads there, so that their
+    // address arithmetic is hidden too.
+    template <bool FIRST, class F>
+    __device__ __forceinline__ void compute(const uint8_t* smem, int stage, v16f (&acc)[Cfg::TM][Cfg::TN],
+                                            F&& after_first) {
         const uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
         if constexpr (AFMT == FMT_BF16) {
             // bf16 operands: 32 contraction bytes (16 elements) per MFMA, one 16-byte chunk per lane
+            after_first();
 #pragma unroll
             for (int ks = 0; ks < Cfg::BK / 32; ++ks) {
                 v8bf a[Cfg::TM], b[Cfg::TN];
@@ -187,41 +203,47 @@ struct TileMainloop {
 #pragma unroll
                 for (int tm = 0; tm < Cfg::TM; ++tm)
 #pragma unroll
-                    for (int tn = 0; tn < Cfg::TN; ++tn)
-                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[tm], b[tn], acc[tm][tn], 0, 0, 0);
+                    for (int tn = 0; tn < Cfg::TN; ++tn) {
+                        const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            a[tm], b[tn], (FIRST && ks == 0) ? zero : acc[tm][tn], 0, 0, 0);
+                    }
             }
             return;
-        }
+        } else {
+            v8i a[Cfg::TM], bcur;
 #pragma unroll
-        for (int ks = 0; ks < Cfg::KSUB; ++ks) {
-            v8i a[Cfg::TM], b[Cfg::TN];
+            for (int t = 0; t < Cfg::TM; ++t) a[t] = frag(s, frag_a[t], 0);
+            bcur = frag(s, frag_b[0], 0);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int t = 0; t < Cfg::TM; ++t) {
-                int o = frag_a[t] ^ (ks * 64);
-                v4i lo = *(const v4i*)(s + o);
-                v4i hi = *(const v4i*)(s + (o ^ 16));
-                a[t] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            }
-#pragma unroll
-            for (int t = 0; t < Cfg::TN; ++t) {
-                int o = frag_b[t] ^ (ks * 64);
-                v4i lo = *(const v4i*)(s + o);
-                v4i hi = *(const v4i*)(s + (o ^ 16));
-                b[t] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            }
-#pragma unroll
-            for (int tm = 0; tm < Cfg::TM; ++tm)
+            for (int ks = 0; ks < Cfg::KSUB; ++ks) {
+                v8i an[Cfg::TM];
 #pragma unroll
                 for (int tn = 0; tn < Cfg::TN; ++tn) {
-                    if (FIRST && ks == 0) {
+                    v8i bnext;
+                    if (tn + 1 < Cfg::TN) {
+                        bnext = frag(s, frag_b[tn + 1], ks);
+                    } else if (ks + 1 < Cfg::KSUB) {
+#pragma unroll
+                        for (int t = 0; t < Cfg::TM; ++t) an[t] = frag(s, frag_a[t], ks + 1);
+                        bnext = frag(s, frag_b[0], ks + 1);
+                    }
+#pragma unroll
+                    for (int tm = 0; tm < Cfg::TM; ++tm) {
                         const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                         acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            a[tm], b[tn], zero, AFMT & 1, BFMT & 1, 0, 0, 0, 0);
-                    } else {
-                        acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            a[tm], b[tn], acc[tm][tn], AFMT & 1, BFMT & 1, 0, 0, 0, 0);
+                            a[tm], bcur, (FIRST && ks == 0) ? zero : acc[tm][tn], AFMT & 1, BFMT & 1, 0, 0, 0, 0);
                     }
+                    if (ks == 0 && tn == 0) after_first();
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (tn + 1 < Cfg::TN || ks + 1 < Cfg::KSUB) bcur = bnext;
                 }
+                if (ks + 1 < Cfg::KSUB) {
+#pragma unroll
+                    for (int t = 0; t < Cfg::TM; ++t) a[t] = an[t];
+                }
+            }
         }
     }
 };
@@ -243,10 +265,10 @@ struct AccCoords {
 // together work on neighbouring tiles of the same split.
 struct GridIter {
     TileOrder order;
-    int it, bid, G, seq, tr_, tc_, split_, splits, jobs;
+    int it, bid, G, seq, tr_, tc_, split_, splits, jobs, nk_, kt_lo_, kt_hi_;
     __device__ GridIter(const GemmOperands& g, int BM, int BN, int bid_, int G_)
         : order(g.R, g.C, BM, BN), it(0), bid(bid_), G(G_), tr_(0), tc_(0), split_(0),
-          splits(g.splits < 1 ? 1 : g.splits) {
+          splits(g.splits < 1 ? 1 : g.splits), nk_(g.K / 128), kt_lo_(0), kt_hi_(0) {
         jobs = order.total * splits;
         seq = TileOrder::seq_of(0, bid, G);
         locate();
@@ -255,13 +277,21 @@ struct GridIter {
         if (seq < jobs) {
             split_ = seq / order.total;
             order.coords(seq - split_ * order.total, tr_, tc_);
+            // the walk depends on the workgroup id only: tell the compiler these are scalars
+            split_ = __builtin_amdgcn_readfirstlane(split_);
+            tr_ = __builtin_amdgcn_readfirstlane(tr_);
+            tc_ = __builtin_amdgcn_readfirstlane(tc_);
+            // contraction range of the job in units of 128 bytes (scaled to k-steps by kt_begin/kt_end)
+            kt_lo_ = (splits == 1) ? 0 : __builtin_amdgcn_readfirstlane(nk_ * split_ / splits);
+            kt_hi_ = (splits == 1) ? nk_ : __builtin_amdgcn_readfirstlane(nk_ * (split_ + 1) / splits);
         }
     }
     __device__ bool valid() const { return seq < jobs; }
     __device__ int tr() const { return tr_; }
     __device__ int tc() const { return tc_; }
-    __device__ int kt_begin(int nk) const { return (int)((int64_t)nk * split_ / splits); }
-    __device__ int kt_end(int nk) const { return (int)((int64_t)nk * (split_ + 1) / splits); }
+    // nk k-steps of BK bytes cover the same contraction as nk_ units of 128 bytes
+    __device__ int kt_begin(int nk) const { return nk == nk_ ? kt_lo_ : 2 * kt_lo_; }
+    __device__ int kt_end(int nk) const { return nk == nk_ ? kt_hi_ : 2 * kt_hi_; }
     __device__ bool job_begin() const { return false; }
     __device__ bool job_end() const { return false; }
     __device__ int job_id() const { return 0; }
@@ -287,19 +317,30 @@ struct GridIter {
 template <class Iter>
 struct StepCursor {
     Iter it;
-    int kt, nk;
-    __device__ StepCursor(const Iter& i, int nk_) : it(i), kt(0), nk(nk_) {
-        if (it.valid()) kt = it.kt_begin(nk);
+    int kt, kt_lo, kt_hi, nk;
+    __device__ StepCursor(const Iter& i, int nk_) : it(i), kt(0), kt_lo(0), kt_hi(0), nk(nk_) { enter(); }
+    __device__ void enter() {
+        if (it.valid()) {
+            kt_lo = it.kt_begin(nk);
+            kt_hi = it.kt_end(nk);
+        }
+        kt = kt_lo;
     }
     __device__ bool valid() const { return it.valid(); }
-    __device__ bool at_job_start() const { return kt == it.kt_begin(nk); }
+    __device__ bool at_job_start() const { return kt == kt_lo; }
     __device__ void advance() {
-        if (++kt == it.kt_end(nk)) {
+        if (++kt == kt_hi) {
             it.advance();
-            kt = it.valid() ? it.kt_begin(nk) : 0;
+            enter();
         }
     }
 };
+
+// Epilogues that declare `static constexpr bool ABLATABLE = true` honour GemmOperands::ablate (timing aid).
+template <class E, class = void>
+struct EpiAblatable : std::false_type {};
+template <class E>
+struct EpiAblatable<E, std::void_t<decltype(E::ABLATABLE)>> : std::bool_constant<E::ABLATABLE> {};
 
 template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(GemmOperands g, Epi epi) {
@@ -307,6 +348,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     static_assert(Epi::EXTRA_LDS % 1024 == 0, "epilogue LDS must keep the stages 1 KiB aligned");
     uint8_t* const smem = smem_all + Epi::EXTRA_LDS;      // operand stages
     constexpr int NS = Cfg::NSTAGES;
+    const int ablate = EpiAblatable<Epi>::value ? g.ablate : 0;
     TileMainloop<Cfg, AFMT, BFMT> ml;
     ml.init();
     const int bid = blockIdx.x, G = gridDim.x;
@@ -329,47 +371,48 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     epi.begin(bid, G, smem_all);
 
     v16f acc[Cfg::TM][Cfg::TN];
-#pragma unroll
-    for (int i = 0; i < Cfg::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < Cfg::TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-    int slot = 0;
-    while (cur.valid()) {
-        const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
-        if (cur.job_begin()) epi.template job_begin<Cfg>(c0);   // made visible by the k-loop's barriers
-        const int kt0 = cur.kt_begin(nk), kt1 = cur.kt_end(nk);
-        for (int kt = kt0; kt < kt1; ++kt) {
-            // The loads of this k-step are the oldest loads in flight and loads retire in order, so it
-            // is enough that at most the NS-2 newer load groups remain outstanding.  Stores issued by
-            // an epilogue share the counter and may retire in any order relative to loads; they only
-            // make this wait stricter, never too weak.  Near the end of the walk fewer groups were
-            // issued, so wait for everything.
-            if (pre.valid()) wait_vmem_le<(NS - 2) * Cfg::LOADS>();
-            else wait_vmem_le<0>();
-            if (!(g.ablate & 4)) wg_barrier();
-            // refill the slot consumed in the previous step with the k-step NS-1 ahead
-            if (pre.valid()) {
-                if (pre.at_job_start()) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
-                if (!(g.ablate & 1)) ml.issue_loads(smem, pre_slot, pre.kt);
-                pre.advance();
-                pre_slot = (pre_slot + 1 == NS) ? 0 : pre_slot + 1;
-            }
-            if (!(g.ablate & 2)) ml.template compute<false>(smem, slot, acc);
-            slot = (slot + 1 == NS) ? 0 : slot + 1;
-        }
-        wg_barrier();   // every wave is done reading the last slot: reuse it as scratch
-        uint8_t* free_stage = smem + (slot == 0 ? NS - 1 : slot - 1) * Cfg::STAGE_BYTES;
-        epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
-        if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
+    if (ablate) {   // the first k-step of a job overwrites the accumulators, unless the MFMAs are ablated
 #pragma unroll
         for (int i = 0; i < Cfg::TM; ++i)
 #pragma unroll
             for (int j = 0; j < Cfg::TN; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    }
+    int slot = 0;
+    // One k-step: wait for its operands, make them visible to the workgroup, refill the slot that the
+    // previous k-step consumed with the k-step NS-1 ahead (behind the first MFMAs), run the MFMAs.
+    // The loads of this k-step are the oldest loads in flight and loads retire in order, so it is
+    // enough that at most the NS-2 newer load groups remain outstanding.  Stores issued by an
+    // epilogue share the counter and may retire in any order relative to loads; they only make this
+    // wait stricter, never too weak.  Near the end of the walk fewer groups were issued, so wait for
+    // everything.
+    auto kstep = [&](auto first) {
+        if (pre.valid()) wait_vmem_le<(NS - 2) * Cfg::LOADS>();
+        else wait_vmem_le<0>();
+        if (!(ablate & 4)) wg_barrier();
+        auto refill = [&]() {
+            if (pre.valid()) {
+                if (pre.at_job_start()) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
+                if (!(ablate & 1)) ml.issue_loads(smem, pre_slot, pre.kt);
+                pre.advance();
+                pre_slot = (pre_slot + 1 == NS) ? 0 : pre_slot + 1;
+            }
+        };
+        if (!(ablate & 2)) ml.template compute<decltype(first)::value>(smem, slot, acc, refill);
+        else refill();
+        slot = (slot + 1 == NS) ? 0 : slot + 1;
+    };
+    while (cur.valid()) {
+        const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
+        if (cur.job_begin()) epi.template job_begin<Cfg>(c0);   // made visible by the k-loop's barriers
+        const int kt0 = cur.kt_begin(nk), kt1 = cur.kt_end(nk);
+        kstep(std::true_type{});                                 // starts the accumulators from zero
+        for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{});
+        wg_barrier();   // every wave is done reading the last slot: reuse it as scratch
+        uint8_t* free_stage = smem + (slot == 0 ? NS - 1 : slot - 1) * Cfg::STAGE_BYTES;
+        epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
+        if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
         cur.advance();
     }
     wg_barrier();

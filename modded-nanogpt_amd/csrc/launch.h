@@ -7,14 +7,12 @@ namespace ngpt {
 
 // 256 x 256 tile, 8 waves as 4 (rows) x 2 (cols): each wave owns 64 x 128 = 2 x 4 MFMA tiles.
 using MainCfg = TileCfg<256, 256, 4, 2, 128, 2>;
-// Alternatives selectable at run time through ngpt_tuning_set(0, id) (tuning aid; slower on MI355X
-// for the shapes of this path).
-using Cfg256x256k64s4 = TileCfg<256, 256, 4, 2, 64, 4>;     // id 1: four 32 KiB stages
-using Cfg256x128k64s2 = TileCfg<256, 128, 2, 2, 64, 2, 2>;  // id 5: 4 waves, 48 KiB: two workgroups per CU
+// (Measured slower on MI355X for the shapes of this path: four 32 KiB stages of 64-byte k-steps, and a
+// 256 x 128 tile with two 4-wave workgroups per CU.  The kernel stays generic over TileCfg.)
 
-// Tuning keys: [0] GEMM tile config id, [2] ablation bits (timing aid),
-// [4] split-K factor of ngpt_gemm_fp8_tn, [5] fused CE kernels: 1 = id 5 tile, 2 = id 1 tile,
-// [6] 1 = split-K in the CE backward GEMMs
+// Tuning keys: [2] ablation bits (timing aid, honoured by the discarding epilogue only),
+// [4] split-K factor of ngpt_gemm_fp8_tn, [6] 1 = split-K in the CE backward GEMMs,
+// [7] 1 = accept operand row strides below K (timing aid: overlapping rows keep the operands cache resident)
 extern int g_tuning[8];
 
 template <class Cfg, int FA, int FB, class Epi>
@@ -44,14 +42,9 @@ int launch_gemm_cfg(const GemmOperands& g, int fa, int fb, const Epi& epi, hipSt
     return launch_gemm_fmt<Cfg, FMT_E5M2, FMT_E5M2>(g, epi, st, max_grid);
 }
 
-// Dispatch on the run-time tile configuration (default MainCfg).
-template <class Cfg /* default */, class Epi>
+template <class Cfg, class Epi>
 int launch_gemm(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {
-    switch (g_tuning[0]) {
-        case 1: return launch_gemm_cfg<Cfg256x256k64s4>(g, fa, fb, epi, st, max_grid);
-        case 5: return launch_gemm_cfg<Cfg256x128k64s2>(g, fa, fb, epi, st, max_grid);
-        default: return launch_gemm_cfg<Cfg>(g, fa, fb, epi, st, max_grid);
-    }
+    return launch_gemm_cfg<Cfg>(g, fa, fb, epi, st, max_grid);
 }
 
 }  // namespace ngpt
