@@ -243,6 +243,7 @@ struct CEJobIter {
     __device__ int tc() const { return tile_m; }
     __device__ int kt_begin(int) const { return 0; }
     __device__ int kt_end(int nk) const { return nk; }
+    __device__ bool partial() const { return false; }
     __device__ bool job_begin() const { return tr_ == tr_begin; }
     __device__ bool job_end() const { return tr_ + 1 == tr_end; }
     __device__ int job_id() const { return split; }
@@ -272,6 +273,7 @@ struct EpiCEFwd {
     int* cand;            // LDS: [MAX_CAND][CE_MAX_BN] valid target column of the job's tokens, else -1
     float sum[8];
 
+    __device__ void partial(bool) {}
     __device__ void begin(int, int, uint8_t* extra) {
         cand = (int*)extra;
         load_table(lds_table(), gtabE);
@@ -409,108 +411,207 @@ __global__ void ce_rowf_kernel(const float* __restrict__ lse, CandArgs ca, Softc
     rowf[m] = coef * (row_weight_sum(ca, m) * expf(sc.A - lse[m]));
 }
 
-// GEMM orientation: rows = tokens of the current chunk (A = x_f8), columns = vocabulary (B = w_f8).
-// Writes the e5m2 dlogits of the chunk row-major (dl [Mc, V]) and transposed (dl_t [V, Mc]).
+// ------------------------------------------------------------------------------------------------
+// dlogits panels.  The e5m2 gradient of a chunk of tokens is consumed twice: as the A operand of
+// dx = dl . W (rows = tokens, contraction = vocabulary) and as an operand of dW = dl^T . x (rows =
+// vocabulary, contraction = tokens).  It is written once in each orientation, panel-blocked (see
+// GemmOperands), and with the contraction bytes of every 128-byte k-step row permuted into the order
+// in which the recompute kernel's accumulator registers already hold them, so that both copies leave
+// the registers as full 16-byte stores without a trip through LDS.  A GEMM is indifferent to the
+// order of its contraction as long as both operands agree, so the other operand of each product
+// (W^T, x^T) is produced with the same permutation by panel_transpose_kernel.
+//
+// token-major panel ("dx panel"):  vocabulary column vv of a k-step (0..127) sits at byte dx_pos(vv)
+// vocab-major panel ("dw panel"):  token tt of a k-step (0..127) sits at byte dw_pos(tt)
+__host__ __device__ inline int dx_pos(int vv) { return 16 * ((vv & 31) >> 2) + 4 * (vv >> 5) + (vv & 3); }
+__host__ __device__ inline int dx_pos_inv(int p) { return 32 * ((p >> 2) & 3) + 4 * (p >> 4) + (p & 3); }
+__host__ __device__ inline int dw_pos(int tt) { return (tt & ~31) | (((tt >> 2) & 1) << 4) | (((tt >> 3) & 3) << 2) | (tt & 3); }
+__host__ __device__ inline int dw_pos_inv(int p) { return (p & ~31) | (((p >> 2) & 3) << 3) | (((p >> 4) & 1) << 2) | (p & 3); }
+
+__host__ __device__ inline int64_t panel_offset(int row, int kbyte, int nk /* k-steps per row */) {
+    return ((int64_t)(row >> 8) * nk + (kbyte >> 7)) * kPanelBytes + (row & 255) * 128;
+}
+
+// 4 x 4 byte transpose across the four lanes of a quad: lane m ends up with byte m of lanes 0..3.
+__device__ __forceinline__ uint32_t quad_transpose_u8(uint32_t x, uint32_t sel1, uint32_t sel2) {
+    uint32_t y = (uint32_t)__builtin_amdgcn_mov_dpp((int)x, 0xB1, 0xf, 0xf, true);   // quad_perm [1,0,3,2]
+    uint32_t r = __builtin_amdgcn_perm(x, y, sel1);
+    uint32_t z = (uint32_t)__builtin_amdgcn_mov_dpp((int)r, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+    return __builtin_amdgcn_perm(r, z, sel2);
+}
+
+// Epilogue of the backward's logits recompute (A = x chunk, rows = tokens; B = W, rows = vocabulary):
+// dl = e5m2_sat(rowf[token] * D(logit)) written to both panels.  Rows past Mc get rowf = 0, i.e. zero codes,
+// so the token padding of the dw panel contracts to nothing.
 struct EpiDlStore {
-    static constexpr int EXTRA_LDS = 0;
-    static constexpr bool NEEDS_SCRATCH = true;
+    static constexpr int TILE_STORES = 16;   // 8 dw-panel + 8 dx-panel 16-byte stores per wave and tile, always
+    static constexpr bool HAS_TILE_BEGIN = true;
+    static constexpr int EXTRA_LDS = 2048;   // row factors of the current and the next tile (2 x 256 floats)
+    static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     template <class Cfg>
     __device__ void job_begin(int) {}
     const float* gtabD;
     const float* rowf;     // already offset to the chunk's first row
-    uint8_t* dl;           // [Mc, V]
-    uint8_t* dl_t;         // [V, Mc]
-    int Mc, V;
+    uint8_t* dx_panel;     // [Mt / 256][V / 128] blocks, Mt = Mc rounded up to 256, plus one more block: the sink
+                           // for the stores of the columns past V in the last vocabulary tile
+    uint8_t* dw_panel;     // [Vp / 256][Mt / 128] blocks, Vp = V rounded up to 256
+    int Mc, V, nkv, nkt;   // k-steps per panel row: V / 128, Mt / 128
     float scale;
+    float* rowf_lds;       // LDS [2][256]
+    int rslot;
 
-    __device__ void begin(int, int, uint8_t*) { load_table(lds_table(), gtabD); }
+    __device__ void partial(bool) {}
+    __device__ void begin(int, int, uint8_t* extra) {
+        rowf_lds = (float*)extra;
+        rslot = 0;
+        load_table(lds_table(), gtabD);
+    }
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
     __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
 
+    // The tile's 256 row factors go straight to LDS with one wave-level load, issued before the k-loop, so
+    // that tile() contains no global load: a load there would make the wave wait for its own earlier
+    // panel stores (the memory counter retires in order).  Two slots: the other one may still be read
+    // by waves that are finishing the previous tile.
+    template <class Cfg>
+    __device__ void tile_begin(int r0, int) {
+        rslot ^= 1;
+        if ((threadIdx.x >> 6) == 0) {
+            int row = min(r0 + 4 * (int)(threadIdx.x & 63), Mc - 4);   // rows past Mc are masked in tile()
+            global_to_lds16(rowf + row, rowf_lds + rslot * 256);
+        }
+    }
+
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
-                         uint8_t* scratch, int lane) {
-        const int h = lane >> 5;
+                         uint8_t*, int lane) {
+        static_assert(Cfg::BM == kPanelRows && Cfg::BN == kPanelRows && Cfg::WTM == 64 && Cfg::WTN == 128,
+                      "the panel stores assume a 256 x 256 tile of 64 x 128 wave tiles");
+        const int h = lane >> 5, j = lane & 31;
         const float* tab = lds_table();
-        uint32_t pk[Cfg::TM][Cfg::TN][4];
+        const int wr = co.wave_row0 >> 6, wc = co.wave_col0 >> 7;
+        // dw panel: row = vocabulary column of this lane, 16 bytes = 16 tokens of one (tm, h) group
+        uint8_t* dw_base = dw_panel + ((int64_t)(c0 >> 8) * nkt + (r0 >> 7) + (wr >> 1)) * kPanelBytes;
+        const uint32_t dw_lane = (uint32_t)((128 * wc + j) * 128 + 64 * (wr & 1) + 16 * h);
+        // dx panel: row = token, 16 bytes = vocabulary columns 4q..4q+3 of the four tn blocks
+        const int ktv = (c0 >> 7) + wc;
+        // the last vocabulary tile may be half empty: its stores go to the sink block behind the panel
+        const int64_t dx_block = ktv < nkv ? (int64_t)(r0 >> 8) * nkv + ktv : (int64_t)((Mc + 255) >> 8) * nkv;
+        uint8_t* dx_base = dx_panel + dx_block * kPanelBytes;
+        const uint32_t dx_lane = (uint32_t)((64 * wr + 4 * h + (j & 3)) * 128 + 16 * (j >> 2));
+        const uint32_t sel1 = (j & 1) ? 0x07030501u : 0x02060004u;
+        const uint32_t sel2 = (j & 2) ? 0x07060302u : 0x01000504u;
 #pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm)
+        for (int tm = 0; tm < Cfg::TM; ++tm) {
+            uint32_t pk[Cfg::TN][4];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                int row = r0 + co.wave_row0 + tm * 32 + 8 * g + 4 * h;
-                v4f rf = (row + 4 <= Mc) ? *(const v4f*)(rowf + row) : (v4f){0.f, 0.f, 0.f, 0.f};
+                const int lrow = co.wave_row0 + tm * 32 + 8 * g + 4 * h;
+                v4f rf = *(const v4f*)(rowf_lds + rslot * 256 + lrow);
+                if (r0 + lrow + 4 > Mc) rf = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int tn = 0; tn < Cfg::TN; ++tn) {
                     const v16f& a = acc[tm][tn];
                     uint32_t o01 = tab_offsets2(pack_logits(a[4 * g] * scale, a[4 * g + 1] * scale));
                     uint32_t o23 = tab_offsets2(pack_logits(a[4 * g + 2] * scale, a[4 * g + 3] * scale));
-                    pk[tm][tn][g] = f32x4_to_e5m2_sat(rf[0] * tab_at(tab, o01 & 0xffffu), rf[1] * tab_at(tab, o01 >> 16),
-                                                      rf[2] * tab_at(tab, o23 & 0xffffu), rf[3] * tab_at(tab, o23 >> 16));
+                    pk[tn][g] = f32x4_to_e5m2_sat(rf[0] * tab_at(tab, o01 & 0xffffu), rf[1] * tab_at(tab, o01 >> 16),
+                                                  rf[2] * tab_at(tab, o23 & 0xffffu), rf[3] * tab_at(tab, o23 >> 16));
                 }
             }
-        // row-major copy: one 32-row strip per tm
-#pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm) {
-            uint32_t codes[Cfg::TN][16];
 #pragma unroll
             for (int tn = 0; tn < Cfg::TN; ++tn)
+                *(v4i*)(dw_base + (dw_lane + tn * 4096 + tm * 32)) =
+                    (v4i){(int)pk[tn][0], (int)pk[tn][1], (int)pk[tn][2], (int)pk[tn][3]};
 #pragma unroll
-                for (int v = 0; v < 16; ++v) codes[tn][v] = (pk[tm][tn][v >> 2] >> (8 * (v & 3))) & 0xffu;
-            store_strip_rowmajor_u8<Cfg>(codes, scratch, lane, dl, V, r0 + co.wave_row0 + tm * 32,
-                                         c0 + co.wave_col0, Mc, V);
-        }
-        // transposed copy: one 32-column strip per tn
+            for (int g = 0; g < 4; ++g) {
+                uint32_t t[Cfg::TN];
 #pragma unroll
-        for (int tn = 0; tn < Cfg::TN; ++tn) {
-            uint32_t packed[Cfg::TM][4];
-#pragma unroll
-            for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) packed[tm][g] = pk[tm][tn][g];
-            store_strip_transposed_u8<Cfg>(packed, scratch, lane, dl_t, Mc, r0 + co.wave_row0,
-                                           c0 + co.wave_col0 + tn * 32, Mc, V);
+                for (int tn = 0; tn < Cfg::TN; ++tn) t[tn] = quad_transpose_u8(pk[tn][g], sel1, sel2);
+                *(v4i*)(dx_base + (dx_lane + (32 * tm + 8 * g) * 128)) = (v4i){(int)t[0], (int)t[1], (int)t[2], (int)t[3]};
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 };
 
 // Rewrites the (at most MAX_CAND) target columns of every row of the chunk with the exact gradient.
 __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __restrict__ saved_sigma,
-                                 CandArgs ca, Softcap sc, float coef, int m_begin, int Mc,
-                                 uint8_t* __restrict__ dl, uint8_t* __restrict__ dl_t) {
+                                 CandArgs ca, Softcap sc, float coef, int m_begin, int Mc, int nkv, int nkt,
+                                 uint8_t* __restrict__ dx_panel, uint8_t* __restrict__ dw_panel) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= Mc) return;
     int m = m_begin + i;
     float s_w = row_weight_sum(ca, m);
     float p_scale = expf(sc.A - lse[m]);
     for (int c = 0; c <= ca.n_predict; ++c) {
-        int64_t t = cand_target(ca, m, c);
-        if (t < 0 || t >= ca.V) continue;
+        int64_t t64 = cand_target(ca, m, c);
+        if (t64 < 0 || t64 >= ca.V) continue;
+        int t = (int)t64;
         float term2 = 0.0f;
         for (int k = 0; k <= ca.n_predict; ++k)
-            if (cand_target(ca, m, k) == t) term2 += cand_weight(ca, k);
+            if (cand_target(ca, m, k) == t64) term2 += cand_weight(ca, k);
         float sg = saved_sigma[(int64_t)c * ca.M + m];
         float gz = s_w * (softcap_E(sg, sc) * p_scale) - term2;
         float gx = coef * gz * sg * (1.0f - sg);
         uint8_t code = (uint8_t)(f32x2_to_e5m2_sat(gx, gx) & 0xffu);
-        dl[(int64_t)i * ca.V + t] = code;
-        dl_t[(int64_t)t * Mc + i] = code;
+        dx_panel[panel_offset(i, t, nkv) + dx_pos(t & 127)] = code;
+        dw_panel[panel_offset(t, i, nkt) + dw_pos(i & 127)] = code;
     }
+}
+
+// Panel-blocked transpose of a row-major fp8 matrix: out row = input column c (c < cols), contraction =
+// input rows [row0, row0 + nrows) padded with zeros to nk * 128, contraction bytes of each k-step
+// permuted by PERM (0 none, 1 dx_pos, 2 dw_pos).  One workgroup moves a 128 (rows) x 64 (columns) tile.
+template <int PERM>
+__global__ __launch_bounds__(256) void panel_transpose_kernel(const uint8_t* __restrict__ in, int64_t ld, int row0, int nrows, int cols,
+                                                              int nk, uint8_t* __restrict__ out) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[128][80];
+    const int kt = blockIdx.x, cg = blockIdx.y, tid = threadIdx.x;
+    for (int i = tid; i < 512; i += 256) {
+        int r = i >> 2, ch = i & 3;
+        int gr = kt * 128 + r;
+        v4i v = {0, 0, 0, 0};
+        if (gr < nrows && cg * 64 + ch * 16 < cols) v = *(const v4i*)(in + (int64_t)(row0 + gr) * ld + cg * 64 + ch * 16);
+        *(v4i*)&tile[r][ch * 16] = v;
+    }
+    __syncthreads();
+    const int o = tid >> 2, part = tid & 3;
+    const int c = cg * 64 + o;
+    if (c >= cols) return;
+    uint32_t w[8];
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            int p = part * 32 + d * 4 + b;
+            int t = PERM == 1 ? dx_pos_inv(p) : PERM == 2 ? dw_pos_inv(p) : p;
+            word |= (uint32_t)tile[t][o] << (8 * b);
+        }
+        w[d] = word;
+    }
+    uint8_t* dst = out + panel_offset(c, kt * 128, nk) + part * 32;
+    *(v4i*)dst = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    *(v4i*)(dst + 16) = (v4i){(int)w[4], (int)w[5], (int)w[6], (int)w[7]};
+}
+
+template <int PERM>
+static int panel_transpose(const uint8_t* in, int64_t ld, int row0, int nrows, int cols, int nk, uint8_t* out, hipStream_t st) {
+    if (cols % 16 || ld % 16) return fail(NGPT_EALIGN, "panel_transpose: cols=%d ld=%lld", cols, (long long)ld);
+    dim3 grid(nk, (cols + 63) / 64);
+    panel_transpose_kernel<PERM><<<grid, 256, 0, st>>>(in, ld, row0, nrows, cols, nk, out);
+    return check_launch("panel_transpose_kernel");
 }
 
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
                float scale, void* out, int64_t ldc, int out_kind, hipStream_t st, int splits);
-int pick_splits(int tiles, int ksteps);
+int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
+                       float scale, void* out_bf16, int64_t ldc, float* part32, hipStream_t st);
+int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
+                      float scale, float* out, int64_t ldc, bool accumulate, hipStream_t st);
 
-// out[i] = bf16(in[i]), eight elements per thread
-__global__ void f32_to_bf16_kernel(const float* __restrict__ in, uint16_t* __restrict__ out, int64_t n8) {
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n8) return;
-    v4f a = *(const v4f*)(in + i * 8), b = *(const v4f*)(in + i * 8 + 4);
-    v4i o = {(int)cvt_pk_bf16(a[0], a[1]), (int)cvt_pk_bf16(a[2], a[3]), (int)cvt_pk_bf16(b[0], b[1]), (int)cvt_pk_bf16(b[2], b[3])};
-    *(v4i*)(out + i * 8) = o;
-}
 extern int g_gemm_slot;
 struct GemmSlot {   // books the plain GEMM launches inside a scope under a CE profile slot
     int saved;
@@ -582,8 +683,10 @@ static int launch_grid_kernel(const GemmOperands& g, const Epi& epi, hipStream_t
     return check_launch(what);
 }
 
-constexpr int BWD_CHUNK_ROWS = 16384;
+// Tokens per pass of the backward: the dlogits panels of one pass take 2 * rows * V bytes of workspace.
+constexpr int BWD_CHUNK_ROWS = 65536;
 static int bwd_chunk_rows(int M) { return M < BWD_CHUNK_ROWS ? M : BWD_CHUNK_ROWS; }
+static int64_t round256(int64_t n) { return (n + 255) / 256 * 256; }
 
 }  // namespace ngpt
 
@@ -673,12 +776,13 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
 }
 
 // ------------------------------------------------------------------------------------------------
-// backward workspace: tabE | tabD | rowf [M] | x_f8^T [K, M] | w_f8^T [K, V] | dl [Mc, V] | dl^T [V, Mc] | dx fp32 [Mc, K]
+// backward workspace: tabE | tabD | rowf [M] | x^T panel [Kp, Mt] | W^T panel [Kp, V] | dx panel [Mt, V] + 32 KiB |
+// dw panel [Vp, Mt] | dx fp32 [Mc, K]   (Mc = tokens per pass, Mt / Kp / Vp = Mc / K / V rounded up to 256)
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
-    int64_t Mc = bwd_chunk_rows(M);
-    return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)M * 4, 256) + align_up((int64_t)K * M, 256) +
-           align_up((int64_t)K * V, 256) + 2 * align_up(Mc * V, 256) + align_up(Mc * K * 4, 256);
+    int64_t Mc = bwd_chunk_rows(M), Mt = round256(Mc), Kp = round256(K), Vp = round256(V);
+    return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)M * 4, 256) + Kp * Mt + Kp * (int64_t)V + Mt * (int64_t)V + kPanelBytes + Vp * Mt +
+           align_up(Mc * K * 4, 256);
 }
 
 extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const int64_t* targets,
@@ -700,20 +804,21 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         return fail(NGPT_EWORKSPACE, "ngpt_lmhead_ce_bwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
     hipStream_t st = (hipStream_t)stream;
     const int Mc_max = bwd_chunk_rows(M);
+    const int64_t Mt_max = round256(Mc_max), Kp = round256(K), Vp = round256(V);
     uint8_t* ws = (uint8_t*)workspace;
     float* tabE = (float*)ws;
     float* tabD = tabE + TAB_ENTRIES;
     ws += align_up(2 * TAB_BYTES, 256);
     float* rowf = (float*)ws;
     ws += align_up((int64_t)M * 4, 256);
-    uint8_t* x_t = ws;
-    ws += align_up((int64_t)K * M, 256);
-    uint8_t* w_t = ws;
-    ws += align_up((int64_t)K * V, 256);
-    uint8_t* dl = ws;
-    ws += align_up((int64_t)Mc_max * V, 256);
-    uint8_t* dl_t = ws;
-    ws += align_up((int64_t)Mc_max * V, 256);
+    uint8_t* x_t = ws;       // x^T panel of the pass: rows = K features, contraction = tokens (dw_pos order)
+    ws += Kp * Mt_max;
+    uint8_t* w_t = ws;       // W^T panel: rows = K features, contraction = vocabulary (dx_pos order)
+    ws += Kp * (int64_t)V;
+    uint8_t* dx_panel = ws;
+    ws += Mt_max * (int64_t)V + kPanelBytes;     // + the sink block
+    uint8_t* dw_panel = ws;
+    ws += Vp * Mt_max;
     float* dx32 = (float*)ws;
 
     Softcap sc = make_softcap(A, B, C);
@@ -722,57 +827,45 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
     ce_rowf_kernel<<<(M + 255) / 256, 256, 0, st>>>(lse, ca, sc, coef, rowf);
     if (int e = check_launch("ce_rowf_kernel")) return e;
-    if (int e = ngpt_transpose_u8(x_f8, M, K, x_t, stream)) return e;
-    if (int e = ngpt_transpose_u8(w_f8_vk, V, K, w_t, stream)) return e;
-    const bool split_k = g_tuning[6] != 0;
-    if (split_k) fill_f32_kernel<<<(int)(((int64_t)V * K + 255) / 256), 256, 0, st>>>((float*)dw_f32, (int64_t)V * K, 0.0f);
+    const int nkv = V / 128;
+    if (int e = panel_transpose<1>((const uint8_t*)w_f8_vk, K, 0, V, K, nkv, w_t, st)) return e;
+    const bool several = M > Mc_max;       // dw then accumulates over the passes
+    if (several) fill_f32_kernel<<<(int)(((int64_t)V * K + 255) / 256), 256, 0, st>>>((float*)dw_f32, (int64_t)V * K, 0.0f);
 
-    using Cfg = MainCfg;
     for (int m0 = 0; m0 < M; m0 += Mc_max) {
         const int Mc = (M - m0 < Mc_max) ? (M - m0) : Mc_max;
-        // 1. recompute the chunk's logits and turn them into e5m2 dlogits (both layouts)
+        const int Mt = (int)round256(Mc), nkt = Mt / 128;
+        if (int e = panel_transpose<2>((const uint8_t*)x_f8, K, m0, Mc, K, nkt, x_t, st)) return e;
+        // 1. recompute the pass's logits and turn them into e5m2 dlogits (both panels)
         GemmOperands g{(const uint8_t*)x_f8 + (int64_t)m0 * K, (const uint8_t*)w_f8_vk, K, K, Mc, V, K, 1, 0};
         EpiDlStore epi{};
         epi.gtabD = tabD;
         epi.rowf = rowf + m0;
-        epi.dl = dl;
-        epi.dl_t = dl_t;
+        epi.dx_panel = dx_panel;
+        epi.dw_panel = dw_panel;
         epi.Mc = Mc;
         epi.V = V;
+        epi.nkv = nkv;
+        epi.nkt = nkt;
         epi.scale = x_s * w_s;
         if (int e = launch_grid_kernel<MainCfg>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
-        ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, dl, dl_t);
+        ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, nkv, nkt, dx_panel, dw_panel);
         if (int e = check_launch("ce_dl_fix_kernel")) return e;
-        // 3. dx[chunk] = dl [Mc, V] . (w^T [K, V])^T.  The output has only K/256 tile columns, so the
-        //    contraction over V is split across jobs that add into an fp32 staging buffer.
+        // 3. dx[pass] = dl [Mc, V] . (W^T [K, V])^T
         {
             GemmSlot slot(PROF_CE_DX);
-            const int tiles = ((Mc + Cfg::BM - 1) / Cfg::BM) * ((K + Cfg::BN - 1) / Cfg::BN);
-            const int splits = pick_splits(tiles, V / Cfg::BK);
-            if (splits > 1) {
-                fill_f32_kernel<<<(int)(((int64_t)Mc * K + 255) / 256), 256, 0, st>>>(dx32, (int64_t)Mc * K, 0.0f);
-                if (int e = gemm_store(dl, FMT_E5M2, V, w_t, FMT_E4M3, V, Mc, K, V, grad_s * w_s, dx32, K, 2, st, splits)) return e;
-                int64_t n8 = (int64_t)Mc * K / 8;
-                f32_to_bf16_kernel<<<(int)((n8 + 255) / 256), 256, 0, st>>>(dx32, (uint16_t*)dx_bf16 + (int64_t)m0 * K, n8);
-                if (int e = check_launch("f32_to_bf16_kernel")) return e;
-            } else {
-                if (int e = gemm_store(dl, FMT_E5M2, V, w_t, FMT_E4M3, V, Mc, K, V, grad_s * w_s,
-                                       (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, 0, st, 1)) return e;
-            }
+            if (int e = gemm_balanced_bf16(dx_panel, FMT_E5M2, 0, w_t, FMT_E4M3, 0, kBlockedA | kBlockedB, Mc, K, V, grad_s * w_s,
+                                           (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, dx32, st)) return e;
         }
-        // 4. dw: the first chunk stores, later chunks add (fp32 atomics); with split-K every chunk adds
-        //    into the zeroed output
+        // 4. dw (+)= dl^T . x over the tokens of the pass (zero padded to Mt)
         GemmSlot slot(PROF_CE_DW);
-        const int kind = (split_k || m0 > 0) ? 2 : 1;
-        if (w_layout == NGPT_W_OUT_IN) {   // dw [V, K] = dl^T [V, Mc] . (x^T [K, Mc])^T
-            const int tiles = ((V + Cfg::BM - 1) / Cfg::BM) * ((K + Cfg::BN - 1) / Cfg::BN);
-            if (int e = gemm_store(dl_t, FMT_E5M2, Mc, x_t + m0, FMT_E4M3, M, V, K, Mc, x_s * grad_s,
-                                   dw_f32, K, kind, st, pick_splits(tiles, Mc / Cfg::BK))) return e;
-        } else {                           // dw [K, V] = x^T [K, Mc] . (dl^T [V, Mc])^T
-            const int tiles = ((K + Cfg::BM - 1) / Cfg::BM) * ((V + Cfg::BN - 1) / Cfg::BN);
-            if (int e = gemm_store(x_t + m0, FMT_E4M3, M, dl_t, FMT_E5M2, Mc, K, V, Mc, x_s * grad_s,
-                                   dw_f32, V, kind, st, pick_splits(tiles, Mc / Cfg::BK))) return e;
+        if (w_layout == NGPT_W_OUT_IN) {   // dw [V, K] = dl^T [V, Mt] . (x^T [K, Mt])^T
+            if (int e = gemm_balanced_f32(dw_panel, FMT_E5M2, 0, x_t, FMT_E4M3, 0, kBlockedA | kBlockedB, V, K, Mt, x_s * grad_s,
+                                          (float*)dw_f32, K, several, st)) return e;
+        } else {                           // dw [K, V] = x^T [K, Mt] . (dl^T [V, Mt])^T
+            if (int e = gemm_balanced_f32(x_t, FMT_E4M3, 0, dw_panel, FMT_E5M2, 0, kBlockedA | kBlockedB, K, V, Mt, x_s * grad_s,
+                                          (float*)dw_f32, V, several, st)) return e;
         }
     }
     return NGPT_OK;

@@ -69,16 +69,53 @@ __device__ __forceinline__ void store_strip_transposed_u8(
     __builtin_amdgcn_s_waitcnt(0xc07f);
 }
 
+// acc * scale into an fp32 matrix: plain stores, or fire-and-forget L2 atomics (no read-modify-write
+// through registers) when `atomic`.  Shared by the fp32 output and by partial tiles of a split contraction.
+template <class Cfg>
+__device__ __forceinline__ void store_tile_f32(v16f (&acc)[Cfg::TM][Cfg::TN], float* out, int64_t ld, float scale, int R, int C,
+                                               int r0, int c0, const AccCoords<Cfg>& co, bool atomic) {
+    float* origin = out + ((int64_t)r0 * ld + c0);
+    const uint32_t lane_off = (uint32_t)co.row_base * (uint32_t)ld + (uint32_t)co.col_base;
+    const int rlim = R - r0 - co.row_base, clim = C - c0 - co.col_base;
+    const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
+#pragma unroll
+    for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < Cfg::TN; ++tn) {
+#pragma unroll
+            for (int v = 0; v < 16; v += 2) {
+                const int dr = tm * 32 + 8 * (v >> 2) + (v & 3), dc = tn * 32;
+                float* pu = origin + ((int64_t)dr * ld + dc);
+                float v0 = acc[tm][tn][v] * scale, v1 = acc[tm][tn][v + 1] * scale;
+                if (full || (dr < rlim && dc < clim)) {
+                    if (atomic) (void)__hip_atomic_fetch_add(&pu[lane_off], v0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    else pu[lane_off] = v0;
+                }
+                if (full || (dr + 1 < rlim && dc < clim)) {
+                    if (atomic) (void)__hip_atomic_fetch_add(&pu[lane_off + (uint32_t)ld], v1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    else pu[lane_off + (uint32_t)ld] = v1;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+}
+
 // ---------------------------------------------------------------------------------------------
 // out[r, c] = bf16(acc * scale)
+// A job that holds only part of its tile's contraction adds acc * scale into the fp32 matrix `part32`
+// (same shape, zeroed by the caller, converted to bf16 by a later pass) instead.
 struct EpiStoreBf16 {
     uint16_t* out;
     int64_t ld;
     float scale;
     int R, C;
+    float* part32;       // required when the walk splits tiles
+    int64_t ld32;
+    bool is_partial;
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
+    __device__ void partial(bool p) { is_partial = p; }
     __device__ void begin(int, int, uint8_t*) {}
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
@@ -88,6 +125,10 @@ struct EpiStoreBf16 {
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t*, int) {
+        if (is_partial) {
+            store_tile_f32<Cfg>(acc, part32, ld32, scale, R, C, r0, c0, co, true);
+            return;
+        }
         // address = wave-uniform pointer (tile origin + the element's fixed position inside the wave
         // tile, all scalar) + ONE per-lane 32-bit offset, so no per-element address registers exist
         uint16_t* origin = out + ((int64_t)r0 * ld + c0);
@@ -121,6 +162,7 @@ struct EpiDpre {
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
+    __device__ void partial(bool) {}
     __device__ void begin(int, int, uint8_t*) {}
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
@@ -167,6 +209,7 @@ struct EpiDiscard {
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     long long t_clk, t_wall;
+    __device__ void partial(bool) {}
     __device__ void begin(int, int, uint8_t*) {
         t_clk = clock64();
         t_wall = wall_clock64();
@@ -194,16 +237,19 @@ struct EpiDiscard {
     }
 };
 
-// out[r, c] (+)= acc * scale in fp32 (the += form uses floating-point atomics)
+// out[r, c] (+)= acc * scale in fp32.  The += form (ACCUMULATE, or a job that holds only part of its
+// tile's contraction) uses floating-point atomics on an output the caller has initialised.
 template <bool ACCUMULATE>
 struct EpiStoreF32 {
     float* out;
     int64_t ld;
     float scale;
     int R, C;
+    bool is_partial;
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
+    __device__ void partial(bool p) { is_partial = p; }
     __device__ void begin(int, int, uint8_t*) {}
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
@@ -213,31 +259,8 @@ struct EpiStoreF32 {
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t*, int) {
-        float* origin = out + ((int64_t)r0 * ld + c0);
-        const uint32_t lane_off = (uint32_t)co.row_base * (uint32_t)ld + (uint32_t)co.col_base;
-        const int rlim = R - r0 - co.row_base, clim = C - c0 - co.col_base;
-        const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
-#pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < Cfg::TN; ++tn) {
-#pragma unroll
-                for (int v = 0; v < 16; v += 2) {
-                    const int dr = tm * 32 + 8 * (v >> 2) + (v & 3), dc = tn * 32;
-                    float* pu = origin + ((int64_t)dr * ld + dc);
-                    float v0 = acc[tm][tn][v] * scale, v1 = acc[tm][tn][v + 1] * scale;
-                    // accumulation is a fire-and-forget L2 atomic: no read-modify-write through registers
-                    if (full || (dr < rlim && dc < clim)) {
-                        if constexpr (ACCUMULATE) (void)__hip_atomic_fetch_add(&pu[lane_off], v0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        else pu[lane_off] = v0;
-                    }
-                    if (full || (dr + 1 < rlim && dc < clim)) {
-                        if constexpr (ACCUMULATE) (void)__hip_atomic_fetch_add(&pu[lane_off + (uint32_t)ld], v1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        else pu[lane_off + (uint32_t)ld] = v1;
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
+        if (ACCUMULATE || is_partial) store_tile_f32<Cfg>(acc, out, ld, scale, R, C, r0, c0, co, true);
+        else store_tile_f32<Cfg>(acc, out, ld, scale, R, C, r0, c0, co, false);
     }
 };
 
@@ -261,6 +284,7 @@ struct EpiRelu2 {
     __device__ void job_begin(int) {}
     template <class Cfg>
     __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+    __device__ void partial(bool) {}
     __device__ void begin(int, int, uint8_t*) {
         scale = *dequant;
         inv_act = post_f8 ? 1.0f / *act_scale : 0.0f;

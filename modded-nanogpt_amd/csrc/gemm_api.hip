@@ -77,24 +77,89 @@ static int check_gemm_dims(const char* who, int R, int C, int K, int64_t lda, in
 // Which profile slot the next gemm_store launches are booked under (set by the fused CE backward).
 int g_gemm_slot = PROF_GEMM;
 
-// Smallest split-K factor (<= 8) whose job count fills the persistent grid to >= 94 %, or else the
-// best one found.  One job must keep at least 8 k-steps.
-int pick_splits(int tiles, int ksteps) {
-    // Measured on MI355X: the skinny backward GEMMs are bound by their strided operand loads, not by
-    // grid occupancy, so splitting the contraction buys nothing; it stays opt-in (tuning key 6).
-    if (!g_tuning[6]) return 1;
-    int cus = num_cus();
-    if (cus <= 0 || tiles <= 0) return 1;
-    int best = 1;
-    double best_eff = 0.0;
-    for (int s = 1; s <= 8 && ksteps / s >= 8; ++s) {
-        int jobs = tiles * s;
-        int rounds = (jobs + cus - 1) / cus;
-        double eff = (double)jobs / ((double)rounds * cus);
-        if (eff > best_eff + 1e-9) { best_eff = eff; best = s; }
-        if (eff >= 0.94) break;
+// ---------------------------------------------------------------------------------------------
+// Balanced walk.  A persistent grid of G workgroups finishes `tiles` tiles in ceil(tiles / G) rounds,
+// and in the last round tiles % G workgroups work while the others idle (dx of the lm_head backward:
+// 576 tiles on 256 CUs = 2.25 rounds, paid as 3).  Instead the first floor(tiles / G) * G tiles run as
+// whole tiles and each of the remaining ones is cut along the contraction into as many jobs as fill
+// one more round; those partial results meet in fp32 through atomics.
+struct BalancePlan {
+    int tiles, full, rem, splits;
+};
+static BalancePlan plan_balance(int R, int C, int K) {
+    BalancePlan p{};
+    p.tiles = ((R + MainCfg::BM - 1) / MainCfg::BM) * ((C + MainCfg::BN - 1) / MainCfg::BN);
+    int G = num_cus() * MainCfg::WGS_PER_CU;
+    if (G <= 0) G = 1;
+    p.full = p.tiles / G * G;
+    p.rem = p.tiles - p.full;
+    p.splits = 1;
+    if (p.rem > 0) {
+        int s = G / p.rem;                       // jobs of the last round: rem * s <= G
+        int max_s = K / MainCfg::BK / 8;          // a job keeps at least 8 k-steps
+        if (s > max_s) s = max_s;
+        if (s > 1) p.splits = s;
     }
-    return best;
+    if (p.splits == 1) { p.full = p.tiles; p.rem = 0; }
+    return p;
+}
+
+// Zero (MODE 0) or convert to bf16 (MODE 1) the 256 x 256 tiles number [first, first + gridDim.x) of the
+// walk order, i.e. exactly the tiles that the balanced walk splits.
+template <int MODE>
+__global__ void rem_tiles_kernel(float* part32, int64_t ld32, uint16_t* out, int64_t ldo, int R, int C, int first) {
+    TileOrder order(R, C, MainCfg::BM, MainCfg::BN);
+    int tr, tc;
+    order.coords(first + blockIdx.x, tr, tc);
+    const int r0 = tr * MainCfg::BM, c0 = tc * MainCfg::BN;
+    const int cols4 = MainCfg::BN / 4;
+    for (int i = threadIdx.x; i < MainCfg::BM * cols4; i += blockDim.x) {
+        int r = r0 + i / cols4, c = c0 + (i % cols4) * 4;
+        if (r >= R || c >= C) continue;          // C % 4 == 0 is checked by the caller
+        float* p = part32 + (int64_t)r * ld32 + c;
+        if (MODE == 0) {
+            *(v4f*)p = (v4f){0.f, 0.f, 0.f, 0.f};
+        } else {
+            v4f v = *(const v4f*)p;
+            v2i o = {(int)cvt_pk_bf16(v[0], v[1]), (int)cvt_pk_bf16(v[2], v[3])};
+            *(v2i*)(out + (int64_t)r * ldo + c) = o;
+        }
+    }
+}
+
+// C[R, C] = scale * A . B^T with the balanced walk.  `layout`: kBlockedA | kBlockedB.
+// bf16 output: part32 is an fp32 [R, C] scratch matrix (row stride C) that only the split tiles touch.
+int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
+                       float scale, void* out_bf16, int64_t ldc, float* part32, hipStream_t st) {
+    if (R <= 0 || C <= 0 || K <= 0 || K % 128 || C % 4 || ldc % 4)
+        return fail(NGPT_EALIGN, "gemm_balanced_bf16: R=%d C=%d K=%d ldc=%lld", R, C, K, (long long)ldc);
+    BalancePlan p = plan_balance(R, C, K);
+    if (p.splits > 1 && !part32) return fail(NGPT_EINVAL, "gemm_balanced_bf16: split tiles need the fp32 scratch matrix");
+    ProfileScope prof(g_gemm_slot, st);
+    if (p.splits > 1) rem_tiles_kernel<0><<<p.rem, 256, 0, st>>>(part32, C, nullptr, 0, R, C, p.full);
+    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full};
+    EpiStoreBf16 epi{(uint16_t*)out_bf16, ldc, scale, R, C, part32, C, false};
+    if (int e = launch_gemm<MainCfg>(g, fa, fb, epi, st)) return e;
+    if (p.splits > 1) rem_tiles_kernel<1><<<p.rem, 256, 0, st>>>(part32, C, (uint16_t*)out_bf16, ldc, R, C, p.full);
+    return check_launch("gemm_balanced_bf16");
+}
+
+// fp32 output.  accumulate: every tile adds into `out` (which the caller initialised); otherwise whole
+// tiles are stored and the split tiles are zeroed here and then added to.
+int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
+                      float scale, float* out, int64_t ldc, bool accumulate, hipStream_t st) {
+    if (R <= 0 || C <= 0 || K <= 0 || K % 128 || C % 4 || ldc % 4)
+        return fail(NGPT_EALIGN, "gemm_balanced_f32: R=%d C=%d K=%d ldc=%lld", R, C, K, (long long)ldc);
+    BalancePlan p = plan_balance(R, C, K);
+    ProfileScope prof(g_gemm_slot, st);
+    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full};
+    if (accumulate) {
+        EpiStoreF32<true> epi{out, ldc, scale, R, C, false};
+        return launch_gemm<MainCfg>(g, fa, fb, epi, st);
+    }
+    if (p.splits > 1) rem_tiles_kernel<0><<<p.rem, 256, 0, st>>>(out, ldc, nullptr, 0, R, C, p.full);
+    EpiStoreF32<false> epi{out, ldc, scale, R, C, false};
+    return launch_gemm<MainCfg>(g, fa, fb, epi, st);
 }
 
 // out_kind: 0 bf16, 1 fp32, 2 fp32 accumulate (atomic), 3 discard.  splits > 1 cuts each tile's
@@ -108,7 +173,7 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
     GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, splits, g_tuning[2]};
     ProfileScope prof(g_gemm_slot, st);
     if (out_kind == 0) {
-        EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C};
+        EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C, nullptr, 0, false};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
     if (out_kind == 3) {
@@ -116,10 +181,10 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
     if (out_kind == 2) {
-        EpiStoreF32<true> epi{(float*)out, ldc, scale, R, C};
+        EpiStoreF32<true> epi{(float*)out, ldc, scale, R, C, false};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
-    EpiStoreF32<false> epi{(float*)out, ldc, scale, R, C};
+    EpiStoreF32<false> epi{(float*)out, ldc, scale, R, C, false};
     return launch_gemm<MainCfg>(g, fa, fb, epi, st);
 }
 

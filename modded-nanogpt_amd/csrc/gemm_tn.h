@@ -26,13 +26,24 @@
 
 namespace ngpt {
 
+// Operand layouts.  Row-major: row r, contraction byte c at r * ld + c.  Panel-blocked (256-row tiles,
+// 128-byte k-steps only): the 256 x 128 slab that one k-step of one tile consumes is one contiguous
+// 32 KiB block, blocks ordered [row tile][k-step]:  ((r / 256) * (K / 128) + c / 128) * 32768 +
+// (r % 256) * 128 + c % 128.  A blocked operand is allocated for whole tiles (rows padded to 256).
+// One k-step then reads 2 x 32 KiB of consecutive addresses instead of 512 rows that lie a full
+// matrix row apart, which for long rows costs a TLB entry and a DRAM page per 128 bytes.
+constexpr int kBlockedA = 1, kBlockedB = 2;
+constexpr int kPanelRows = 256, kPanelBytes = kPanelRows * 128;
+
 struct GemmOperands {
     const uint8_t* A;   // [R, K] fp8, row stride lda bytes
     const uint8_t* B;   // [C, K] fp8, row stride ldb bytes
-    int64_t lda, ldb;
+    int64_t lda, ldb;   // ignored for a blocked operand
     int R, C, K;        // K % 128 == 0
-    int splits;         // split-K: each tile's contraction is cut into this many jobs (>= 1); needs an accumulating epilogue if > 1
+    int splits;         // split-K: the contraction of a split tile is cut into this many jobs (>= 1); needs an accumulating epilogue if > 1
     int ablate;         // timing aid: bit 0 = issue no operand loads after the first, bit 1 = no MFMA work, bit 2 = no k-loop barrier
+    int layout;         // kBlockedA | kBlockedB
+    int full_tiles;     // the first full_tiles tiles (in walk order) are never split; 0 = `splits` applies to every tile
 };
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1>
@@ -108,6 +119,7 @@ struct LaneOffsets {
         for (int i = 0; i < Cfg::A_LOADS; ++i) {
             int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
             int q = lchunk ^ Cfg::swz(R);
+            if (g.layout & kBlockedA) { a_off[i] = (uint32_t)(R * 128 + q * 16); continue; }   // padded: no clamp
             int rr = min(R, g.R - 1 - r0);                       // clamp rows past the end
             a_off[i] = (uint32_t)((int64_t)rr * g.lda + q * 16);
         }
@@ -115,6 +127,7 @@ struct LaneOffsets {
         for (int i = 0; i < Cfg::B_LOADS; ++i) {
             int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
             int q = lchunk ^ Cfg::swz(R);
+            if (g.layout & kBlockedB) { b_off[i] = (uint32_t)(R * 128 + q * 16); continue; }
             int rr = min(R, g.C - 1 - c0);
             b_off[i] = (uint32_t)((int64_t)rr * g.ldb + q * 16);
         }
@@ -128,6 +141,7 @@ struct TileMainloop {
     const uint8_t* b_base;
     int frag_a[Cfg::TM];     // LDS byte offset of this lane's first 16-byte chunk, stage 0, ksub 0
     int frag_b[Cfg::TN];
+    int a_step, b_step;      // bytes from one k-step's slab to the next
     int wave, lane, wr, wc;
 
     __device__ void init() {
@@ -154,15 +168,18 @@ struct TileMainloop {
     // Point the loads at tile (r0, c0).  Rows past the end are clamped to the last row: they are
     // loaded (valid memory) and their results discarded by the epilogue.
     __device__ void set_tile(const GemmOperands& g, int r0, int c0) {
-        a_base = g.A + (int64_t)r0 * g.lda;
-        b_base = g.B + (int64_t)c0 * g.ldb;
+        // a blocked operand's tile starts r0 / 256 * (K / 128) blocks in, which is r0 * K bytes
+        a_base = g.A + (int64_t)r0 * ((g.layout & kBlockedA) ? (int64_t)g.K : g.lda);
+        b_base = g.B + (int64_t)c0 * ((g.layout & kBlockedB) ? (int64_t)g.K : g.ldb);
+        a_step = (g.layout & kBlockedA) ? kPanelBytes : Cfg::BK;
+        b_step = (g.layout & kBlockedB) ? kPanelBytes : Cfg::BK;
         lo.init(g, wave, lane, r0, c0);
     }
 
     __device__ void issue_loads(uint8_t* smem, int stage, int kt) {
         uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
-        const uint8_t* ab = a_base + kt * Cfg::BK;
-        const uint8_t* bb = b_base + kt * Cfg::BK;
+        const uint8_t* ab = a_base + (int64_t)kt * a_step;
+        const uint8_t* bb = b_base + (int64_t)kt * b_step;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i)
             global_to_lds16(ab + lo.a_off[i], s + (wave + i * Cfg::NWAVES) * 1024);
@@ -260,30 +277,41 @@ struct AccCoords {
     __device__ int col(int tn) const { return col_base + tn * 32; }
 };
 
-// Default job walk: every (tile, contraction split) of the R x C grid once.  Jobs are numbered
-// split-major (all tiles of split 0 in TileOrder, then split 1, ...), so the workgroups that run
-// together work on neighbouring tiles of the same split.
+// Default job walk: the tiles of the R x C grid in TileOrder.  The first `full` tiles are one job
+// each; every later tile is cut into `splits` jobs along the contraction (partial results, for an
+// accumulating epilogue).  Split jobs are numbered split-major, so the workgroups that run together
+// work on neighbouring tiles.  With full = tiles rounded down to a multiple of the grid and the
+// remainder split to fill one more round, no workgroup idles while the last tiles finish.
 struct GridIter {
     TileOrder order;
-    int it, bid, G, seq, tr_, tc_, split_, splits, jobs, nk_, kt_lo_, kt_hi_;
+    int it, bid, G, seq, tr_, tc_, split_, splits, full, jobs, nk_, kt_lo_, kt_hi_;
     __device__ GridIter(const GemmOperands& g, int BM, int BN, int bid_, int G_)
         : order(g.R, g.C, BM, BN), it(0), bid(bid_), G(G_), tr_(0), tc_(0), split_(0),
           splits(g.splits < 1 ? 1 : g.splits), nk_(g.K / 128), kt_lo_(0), kt_hi_(0) {
-        jobs = order.total * splits;
+        full = (splits == 1) ? order.total : min(max(g.full_tiles, 0), order.total);
+        jobs = full + (order.total - full) * splits;
         seq = TileOrder::seq_of(0, bid, G);
         locate();
     }
     __device__ void locate() {
         if (seq < jobs) {
-            split_ = seq / order.total;
-            order.coords(seq - split_ * order.total, tr_, tc_);
+            int tile = seq;
+            split_ = 0;
+            kt_lo_ = 0;
+            kt_hi_ = nk_;
+            if (seq >= full) {
+                const int rem = order.total - full, idx = seq - full;
+                split_ = idx / rem;
+                tile = full + idx - split_ * rem;
+                split_ = __builtin_amdgcn_readfirstlane(split_);
+                // contraction range of the job in units of 128 bytes
+                kt_lo_ = __builtin_amdgcn_readfirstlane(nk_ * split_ / splits);
+                kt_hi_ = __builtin_amdgcn_readfirstlane(nk_ * (split_ + 1) / splits);
+            }
+            order.coords(tile, tr_, tc_);
             // the walk depends on the workgroup id only: tell the compiler these are scalars
-            split_ = __builtin_amdgcn_readfirstlane(split_);
             tr_ = __builtin_amdgcn_readfirstlane(tr_);
             tc_ = __builtin_amdgcn_readfirstlane(tc_);
-            // contraction range of the job in units of 128 bytes (scaled to k-steps by kt_begin/kt_end)
-            kt_lo_ = (splits == 1) ? 0 : __builtin_amdgcn_readfirstlane(nk_ * split_ / splits);
-            kt_hi_ = (splits == 1) ? nk_ : __builtin_amdgcn_readfirstlane(nk_ * (split_ + 1) / splits);
         }
     }
     __device__ bool valid() const { return seq < jobs; }
@@ -292,6 +320,7 @@ struct GridIter {
     // nk k-steps of BK bytes cover the same contraction as nk_ units of 128 bytes
     __device__ int kt_begin(int nk) const { return nk == nk_ ? kt_lo_ : 2 * kt_lo_; }
     __device__ int kt_end(int nk) const { return nk == nk_ ? kt_hi_ : 2 * kt_hi_; }
+    __device__ bool partial() const { return seq >= full; }     // the job holds part of its tile's contraction
     __device__ bool job_begin() const { return false; }
     __device__ bool job_end() const { return false; }
     __device__ int job_id() const { return 0; }
@@ -304,6 +333,7 @@ struct GridIter {
 
 // The generic persistent kernel.  `Iter` walks the tiles of this workgroup (see GridIter).  `Epi` supplies
 //   void begin(int bid, int nblocks)
+//   void partial(bool)   -- before each tile(): the job holds only part of the tile's contraction
 //   void tile(acc, r0, c0, coords, scratch /* wave-private LDS */, lane)
 //   void job_begin(c0) / job_end(c0, job_id, coords, stage_scratch /* whole free LDS stage */)
 //                                                              -- only if Iter reports job boundaries
@@ -341,6 +371,22 @@ template <class E, class = void>
 struct EpiAblatable : std::false_type {};
 template <class E>
 struct EpiAblatable<E, std::void_t<decltype(E::ABLATABLE)>> : std::bool_constant<E::ABLATABLE> {};
+
+// Epilogues that declare `static constexpr int TILE_STORES = n` promise that every wave issues exactly n
+// vector-memory instructions in each tile() call (and none in job_end).  The memory counter retires in
+// issue order and the operand loads of a tile's first k-step are issued before the previous tile's
+// epilogue, so that k-step may start while those n stores are still in flight.
+template <class E, class = void>
+struct EpiTileStores : std::integral_constant<int, 0> {};
+template <class E>
+struct EpiTileStores<E, std::void_t<decltype(E::TILE_STORES)>> : std::integral_constant<int, E::TILE_STORES> {};
+
+// Epilogues with `static constexpr bool HAS_TILE_BEGIN = true` get tile_begin<Cfg>(r0, c0) before the
+// k-loop of every job; LDS it fills (also through direct-to-LDS loads) is visible in tile().
+template <class E, class = void>
+struct EpiHasTileBegin : std::false_type {};
+template <class E>
+struct EpiHasTileBegin<E, std::void_t<decltype(E::HAS_TILE_BEGIN)>> : std::bool_constant<E::HAS_TILE_BEGIN> {};
 
 template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(GemmOperands g, Epi epi) {
@@ -387,9 +433,10 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     // epilogue share the counter and may retire in any order relative to loads; they only make this
     // wait stricter, never too weak.  Near the end of the walk fewer groups were issued, so wait for
     // everything.
-    auto kstep = [&](auto first) {
-        if (pre.valid()) wait_vmem_le<(NS - 2) * Cfg::LOADS>();
-        else wait_vmem_le<0>();
+    auto kstep = [&](auto first, auto after_epilogue) {
+        constexpr int STORES = decltype(after_epilogue)::value ? EpiTileStores<Epi>::value : 0;
+        if (pre.valid()) wait_vmem_le<(NS - 2) * Cfg::LOADS + STORES>();
+        else wait_vmem_le<STORES>();
         if (!(ablate & 4)) wg_barrier();
         auto refill = [&]() {
             if (pre.valid()) {
@@ -403,14 +450,21 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         else refill();
         slot = (slot + 1 == NS) ? 0 : slot + 1;
     };
+    bool first_job = true;
     while (cur.valid()) {
         const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
         if (cur.job_begin()) epi.template job_begin<Cfg>(c0);   // made visible by the k-loop's barriers
         const int kt0 = cur.kt_begin(nk), kt1 = cur.kt_end(nk);
-        kstep(std::true_type{});                                 // starts the accumulators from zero
-        for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{});
+        if constexpr (EpiHasTileBegin<Epi>::value) epi.template tile_begin<Cfg>(r0, c0);
+        // the first k-step starts the accumulators from zero
+        if (first_job || EpiTileStores<Epi>::value == 0) kstep(std::true_type{}, std::false_type{});
+        else kstep(std::true_type{}, std::true_type{});
+        first_job = false;
+        for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{}, std::false_type{});
+        if (EpiHasTileBegin<Epi>::value && kt1 - kt0 < 2) wait_vmem_le<0>();   // tile_begin's loads: no later k-step waited for them
         wg_barrier();   // every wave is done reading the last slot: reuse it as scratch
         uint8_t* free_stage = smem + (slot == 0 ? NS - 1 : slot - 1) * Cfg::STAGE_BYTES;
+        epi.partial(cur.partial());
         epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
         if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
         cur.advance();
