@@ -202,8 +202,9 @@ struct EpiDpre {
 };
 
 // Mainloop-only timing aid: keeps the accumulators alive but writes (practically) nothing.
-struct EpiDiscard {
-    static constexpr bool ABLATABLE = true;
+template <bool ABLATE>
+struct EpiDiscardT {
+    static constexpr bool ABLATABLE = ABLATE;
     float* out;   // >= 4 floats; workgroup 0 leaves its shader-clock and 100 MHz wall-clock tick counts in out[2], out[3]
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;
@@ -263,6 +264,9 @@ struct EpiStoreF32 {
         else store_tile_f32<Cfg>(acc, out, ld, scale, R, C, r0, c0, co, false);
     }
 };
+
+using EpiDiscard = EpiDiscardT<false>;
+using EpiDiscardAblate = EpiDiscardT<true>;    // honours GemmOperands::ablate, at the price of its branches
 
 // post = bf16(max(bf16(acc * *dequant), 0)^2); optionally post_f8 = e4m3(min(post / act_scale, 448))
 // and a per-workgroup running max of post written to partial_amax[bid].

@@ -177,6 +177,10 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
     if (out_kind == 3) {
+        if (g.ablate) {
+            EpiDiscardAblate epi{(float*)out, 0, 0};
+            return launch_gemm<MainCfg>(g, fa, fb, epi, st);
+        }
         EpiDiscard epi{(float*)out, 0, 0};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }

@@ -137,8 +137,8 @@ struct LaneOffsets {
 template <class Cfg, int AFMT, int BFMT>
 struct TileMainloop {
     LaneOffsets<Cfg> lo;
-    const uint8_t* a_base;   // wave-uniform: first row of the tile
-    const uint8_t* b_base;
+    const uint8_t* a_next;   // wave-uniform: slab of the next k-step to load (first row of the tile)
+    const uint8_t* b_next;
     int frag_a[Cfg::TM];     // LDS byte offset of this lane's first 16-byte chunk, stage 0, ksub 0
     int frag_b[Cfg::TN];
     int a_step, b_step;      // bytes from one k-step's slab to the next
@@ -167,19 +167,23 @@ struct TileMainloop {
 
     // Point the loads at tile (r0, c0).  Rows past the end are clamped to the last row: they are
     // loaded (valid memory) and their results discarded by the epilogue.
-    __device__ void set_tile(const GemmOperands& g, int r0, int c0) {
-        // a blocked operand's tile starts r0 / 256 * (K / 128) blocks in, which is r0 * K bytes
-        a_base = g.A + (int64_t)r0 * ((g.layout & kBlockedA) ? (int64_t)g.K : g.lda);
-        b_base = g.B + (int64_t)c0 * ((g.layout & kBlockedB) ? (int64_t)g.K : g.ldb);
+    // `kt`: first k-step that will be loaded from this tile.
+    __device__ void set_tile(const GemmOperands& g, int r0, int c0, int kt) {
         a_step = (g.layout & kBlockedA) ? kPanelBytes : Cfg::BK;
         b_step = (g.layout & kBlockedB) ? kPanelBytes : Cfg::BK;
+        // a blocked operand's tile starts r0 / 256 * (K / 128) blocks in, which is r0 * K bytes
+        a_next = g.A + (int64_t)r0 * ((g.layout & kBlockedA) ? (int64_t)g.K : g.lda) + (int64_t)kt * a_step;
+        b_next = g.B + (int64_t)c0 * ((g.layout & kBlockedB) ? (int64_t)g.K : g.ldb) + (int64_t)kt * b_step;
         lo.init(g, wave, lane, r0, c0);
     }
 
-    __device__ void issue_loads(uint8_t* smem, int stage, int kt) {
+    // Loads the next k-step of the current tile into LDS slot `stage` and moves on to the one after.
+    __device__ void issue_loads(uint8_t* smem, int stage) {
         uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
-        const uint8_t* ab = a_base + (int64_t)kt * a_step;
-        const uint8_t* bb = b_base + (int64_t)kt * b_step;
+        const uint8_t* ab = a_next;
+        const uint8_t* bb = b_next;
+        a_next += a_step;
+        b_next += b_step;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i)
             global_to_lds16(ab + lo.a_off[i], s + (wave + i * Cfg::NWAVES) * 1024);
@@ -196,42 +200,52 @@ struct TileMainloop {
         return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
 
-    // One k-step of MFMAs.  The LDS reads are software-pipelined against the MFMAs by hand: the A
-    // fragments and the first B fragment of a sub-step are read while the previous sub-step's last
-    // MFMAs run, every further B fragment while the MFMAs of the one before it run, and scheduling
-    // barriers keep the compiler from hoisting all reads to the top (which would leave the matrix
-    // pipe idle for a full LDS round trip per sub-step).  `after_first` runs once, behind the first
-    // group of MFMAs of the k-step: the kernel issues the next operand loads there, so that their
-    // address arithmetic is hidden too.
-    template <bool FIRST, class F>
-    __device__ __forceinline__ void compute(const uint8_t* smem, int stage, v16f (&acc)[Cfg::TM][Cfg::TN],
-                                            F&& after_first) {
+    // One k-step of MFMAs on the operands in LDS slot `stage`, software-pipelined by hand.
+    //  * Fragment reads run one MFMA group (TM MFMAs that share a B fragment) ahead of their use, and
+    //    scheduling barriers keep the compiler from hoisting all reads to the top, which would leave
+    //    the matrix pipe idle for an LDS round trip per sub-step.
+    //  * `sync` (operand wait + workgroup barrier + issue of the next loads, supplied by the kernel) runs
+    //    before the LAST group instead of between k-steps: at that point every LDS read of this slot
+    //    has been issued, so after the barrier the slot may be refilled, and the first fragments of the
+    //    next k-step (slot `next_stage`, if `want_next`) are read behind the last group's MFMAs.
+    //    They are handed to the next call in a / b0 (`have` = they are valid on entry).
+    //    `refill` (issue of the operand loads two k-steps ahead into the slot just freed) runs behind the
+    //    last group's MFMAs, so that its address arithmetic is hidden too.
+    template <bool FIRST, class Sync, class Refill>
+    __device__ __forceinline__ void compute(const uint8_t* smem, int stage, int next_stage, bool have, bool want_next,
+                                            v16f (&acc)[Cfg::TM][Cfg::TN], v8i (&a)[Cfg::TM], v8i& b0, Sync&& sync,
+                                            Refill&& refill) {
         const uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
+        const uint8_t* sn = smem + next_stage * Cfg::STAGE_BYTES;
         if constexpr (AFMT == FMT_BF16) {
-            // bf16 operands: 32 contraction bytes (16 elements) per MFMA, one 16-byte chunk per lane
-            after_first();
+            // bf16 operands: 32 contraction bytes (16 elements) per MFMA, one 16-byte chunk per lane;
+            // no fragment hand-over between k-steps
+            constexpr int KS = Cfg::BK / 32;
 #pragma unroll
-            for (int ks = 0; ks < Cfg::BK / 32; ++ks) {
-                v8bf a[Cfg::TM], b[Cfg::TN];
+            for (int ks = 0; ks < KS; ++ks) {
+                v8bf fa[Cfg::TM], fb[Cfg::TN];
 #pragma unroll
-                for (int t = 0; t < Cfg::TM; ++t) a[t] = *(const v8bf*)(s + (frag_a[t] ^ (ks * 32)));
+                for (int t = 0; t < Cfg::TM; ++t) fa[t] = *(const v8bf*)(s + (frag_a[t] ^ (ks * 32)));
 #pragma unroll
-                for (int t = 0; t < Cfg::TN; ++t) b[t] = *(const v8bf*)(s + (frag_b[t] ^ (ks * 32)));
+                for (int t = 0; t < Cfg::TN; ++t) fb[t] = *(const v8bf*)(s + (frag_b[t] ^ (ks * 32)));
+                if (ks == KS - 1) sync();
 #pragma unroll
                 for (int tm = 0; tm < Cfg::TM; ++tm)
 #pragma unroll
                     for (int tn = 0; tn < Cfg::TN; ++tn) {
                         const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                         acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            a[tm], b[tn], (FIRST && ks == 0) ? zero : acc[tm][tn], 0, 0, 0);
+                            fa[tm], fb[tn], (FIRST && ks == 0) ? zero : acc[tm][tn], 0, 0, 0);
                     }
             }
-            return;
+            refill();
         } else {
-            v8i a[Cfg::TM], bcur;
+            v8i bcur = b0;
+            if (!have) {
 #pragma unroll
-            for (int t = 0; t < Cfg::TM; ++t) a[t] = frag(s, frag_a[t], 0);
-            bcur = frag(s, frag_b[0], 0);
+                for (int t = 0; t < Cfg::TM; ++t) a[t] = frag(s, frag_a[t], 0);
+                bcur = frag(s, frag_b[0], 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int ks = 0; ks < Cfg::KSUB; ++ks) {
@@ -245,6 +259,17 @@ struct TileMainloop {
 #pragma unroll
                         for (int t = 0; t < Cfg::TM; ++t) an[t] = frag(s, frag_a[t], ks + 1);
                         bnext = frag(s, frag_b[0], ks + 1);
+                    } else {
+                        sync();
+                        if (want_next) {
+#pragma unroll
+                            for (int t = 0; t < Cfg::TM; ++t) an[t] = frag(sn, frag_a[t], 0);
+                            bnext = frag(sn, frag_b[0], 0);
+                        } else {
+#pragma unroll
+                            for (int t = 0; t < Cfg::TM; ++t) an[t] = a[t];
+                            bnext = bcur;
+                        }
                     }
 #pragma unroll
                     for (int tm = 0; tm < Cfg::TM; ++tm) {
@@ -252,15 +277,15 @@ struct TileMainloop {
                         acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                             a[tm], bcur, (FIRST && ks == 0) ? zero : acc[tm][tn], AFMT & 1, BFMT & 1, 0, 0, 0, 0);
                     }
-                    if (ks == 0 && tn == 0) after_first();
                     __builtin_amdgcn_sched_barrier(0);
-                    if (tn + 1 < Cfg::TN || ks + 1 < Cfg::KSUB) bcur = bnext;
+                    bcur = bnext;
                 }
-                if (ks + 1 < Cfg::KSUB) {
 #pragma unroll
-                    for (int t = 0; t < Cfg::TM; ++t) a[t] = an[t];
-                }
+                for (int t = 0; t < Cfg::TM; ++t) a[t] = an[t];
             }
+            b0 = bcur;
+            refill();
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 };
@@ -360,6 +385,7 @@ struct StepCursor {
     __device__ bool at_job_start() const { return kt == kt_lo; }
     __device__ void advance() {
         if (++kt == kt_hi) {
+            asm volatile("; next job" ::: "memory");   // rare: keep it a branch, out of the k-loop's straight path
             it.advance();
             enter();
         }
@@ -388,13 +414,21 @@ struct EpiHasTileBegin : std::false_type {};
 template <class E>
 struct EpiHasTileBegin<E, std::void_t<decltype(E::HAS_TILE_BEGIN)>> : std::bool_constant<E::HAS_TILE_BEGIN> {};
 
+// Epilogues with `static constexpr bool TIGHT_REGISTERS = true` need every register in tile(): the last
+// k-step of a job then does not read the next job's first fragments ahead (they would stay live across
+// the epilogue).
+template <class E, class = void>
+struct EpiTightRegisters : std::false_type {};
+template <class E>
+struct EpiTightRegisters<E, std::void_t<decltype(E::TIGHT_REGISTERS)>> : std::bool_constant<E::TIGHT_REGISTERS> {};
+
 template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(GemmOperands g, Epi epi) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_all[];
     static_assert(Epi::EXTRA_LDS % 1024 == 0, "epilogue LDS must keep the stages 1 KiB aligned");
-    uint8_t* const smem = smem_all + Epi::EXTRA_LDS;      // operand stages
-    constexpr int NS = Cfg::NSTAGES;
-    const int ablate = EpiAblatable<Epi>::value ? g.ablate : 0;
+    static_assert(Cfg::NSTAGES == 2, "the k-loop below alternates between two LDS slots");
+    uint8_t* const smem = smem_all + Epi::EXTRA_LDS;      // operand slots
+    const int ablate = EpiAblatable<Epi>::value ? __builtin_amdgcn_readfirstlane(g.ablate) : 0;
     TileMainloop<Cfg, AFMT, BFMT> ml;
     ml.init();
     const int bid = blockIdx.x, G = gridDim.x;
@@ -402,19 +436,28 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane);
     Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
 
-    // prologue: put NS-1 k-steps in flight
+    // `pre` walks the (job, k-step) sequence of this workgroup ahead of the MFMAs; `ahead` counts the
+    // k-steps whose operand loads have been issued and not yet consumed (at most one per slot).
     StepCursor<Iter> pre(cur, nk);
-    int pre_slot = 0;
-#pragma unroll
-    for (int i = 0; i < NS - 1; ++i) {
+    int ahead = 0;
+    auto refill = [&](int into_slot) {
         if (pre.valid()) {
-            if (pre.at_job_start()) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
-            ml.issue_loads(smem, pre_slot, pre.kt);
+            if (pre.at_job_start()) {
+                asm volatile("; new tile" ::: "memory");   // rare: keep it a branch, out of the k-loop's straight path
+                ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN, pre.kt);
+            }
+            if (!(ablate & 1) || ahead == 0) ml.issue_loads(smem, into_slot);
             pre.advance();
+            ++ahead;
         }
-        pre_slot = (pre_slot + 1 == NS) ? 0 : pre_slot + 1;
-    }
+    };
+    refill(0);
+    refill(1);
     epi.begin(bid, G, smem_all);
+    // operands of the first k-step
+    if (ahead == 2) wait_vmem_le<Cfg::LOADS>();
+    else wait_vmem_le<0>();
+    wg_barrier();
 
     v16f acc[Cfg::TM][Cfg::TN];
     if (ablate) {   // the first k-step of a job overwrites the accumulators, unless the MFMAs are ablated
@@ -425,48 +468,61 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
     }
+    v8i fa[Cfg::TM], fb = {};      // first fragments of the upcoming k-step, when `have`
+#pragma unroll
+    for (int t = 0; t < Cfg::TM; ++t) fa[t] = (v8i){};
+    bool have = false;
     int slot = 0;
-    // One k-step: wait for its operands, make them visible to the workgroup, refill the slot that the
-    // previous k-step consumed with the k-step NS-1 ahead (behind the first MFMAs), run the MFMAs.
-    // The loads of this k-step are the oldest loads in flight and loads retire in order, so it is
-    // enough that at most the NS-2 newer load groups remain outstanding.  Stores issued by an
-    // epilogue share the counter and may retire in any order relative to loads; they only make this
-    // wait stricter, never too weak.  Near the end of the walk fewer groups were issued, so wait for
-    // everything.
-    auto kstep = [&](auto first, auto after_epilogue) {
-        constexpr int STORES = decltype(after_epilogue)::value ? EpiTileStores<Epi>::value : 0;
-        if (pre.valid()) wait_vmem_le<(NS - 2) * Cfg::LOADS + STORES>();
-        else wait_vmem_le<STORES>();
-        if (!(ablate & 4)) wg_barrier();
-        auto refill = [&]() {
-            if (pre.valid()) {
-                if (pre.at_job_start()) ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN);
-                if (!(ablate & 1)) ml.issue_loads(smem, pre_slot, pre.kt);
-                pre.advance();
-                pre_slot = (pre_slot + 1 == NS) ? 0 : pre_slot + 1;
-            }
-        };
-        if (!(ablate & 2)) ml.template compute<decltype(first)::value>(smem, slot, acc, refill);
-        else refill();
-        slot = (slot + 1 == NS) ? 0 : slot + 1;
-    };
     bool first_job = true;
     while (cur.valid()) {
         const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
         if (cur.job_begin()) epi.template job_begin<Cfg>(c0);   // made visible by the k-loop's barriers
         const int kt0 = cur.kt_begin(nk), kt1 = cur.kt_end(nk);
         if constexpr (EpiHasTileBegin<Epi>::value) epi.template tile_begin<Cfg>(r0, c0);
-        // the first k-step starts the accumulators from zero
-        if (first_job || EpiTileStores<Epi>::value == 0) kstep(std::true_type{}, std::false_type{});
-        else kstep(std::true_type{}, std::true_type{});
+        // the epilogue of this job reuses the slot of its last k-step as scratch: keep loads out of it
+        const bool keep_slot = Epi::NEEDS_SCRATCH || (Epi::JOB_END_NEEDS_SCRATCH && cur.job_end());
+        // One k-step.  sync() runs before its last MFMA group: the next k-step's operands must have
+        // landed (its loads are the newest load group in flight; the memory counter retires in issue
+        // order, so anything issued after them -- the previous epilogue's stores -- may still be
+        // pending), the workgroup meets, and the slot just read is refilled two k-steps ahead.
+        auto kstep = [&](auto first, auto relaxed, bool last_kt) {
+            constexpr int PENDING_OK = decltype(relaxed)::value ? EpiTileStores<Epi>::value : 0;
+            // a k-step follows this one (and its first fragments may be read ahead)
+            const bool more = ahead >= 2;
+            auto sync = [&]() {
+                wait_vmem_le<PENDING_OK>();
+                if (!(ablate & 4)) wg_barrier();
+            };
+            auto refill_here = [&]() {
+                if (!(last_kt && keep_slot)) refill(slot);
+            };
+            if (!(ablate & 2)) {
+                ml.template compute<decltype(first)::value>(smem, slot, slot ^ 1, have, more, acc, fa, fb, sync, refill_here);
+            } else {
+                sync();
+                refill_here();
+            }
+            have = more && AFMT != FMT_BF16 && !(ablate & 2);
+            --ahead;
+            slot ^= 1;
+        };
+        // relaxed wait: only behind an epilogue that stored (not the first job), with a later k-step of
+        // the same job to wait for tile_begin's load, and only if that epilogue's refill was not deferred
+        constexpr bool kNeverDefers = !Epi::NEEDS_SCRATCH && !Epi::JOB_END_NEEDS_SCRATCH;
+        const bool relax = kNeverDefers && EpiTileStores<Epi>::value > 0 && !first_job && kt1 - kt0 >= 2;
+        if (relax) kstep(std::true_type{}, std::true_type{}, kt0 + 1 == kt1);
+        else kstep(std::true_type{}, std::false_type{}, kt0 + 1 == kt1);
         first_job = false;
-        for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{}, std::false_type{});
-        if (EpiHasTileBegin<Epi>::value && kt1 - kt0 < 2) wait_vmem_le<0>();   // tile_begin's loads: no later k-step waited for them
-        wg_barrier();   // every wave is done reading the last slot: reuse it as scratch
-        uint8_t* free_stage = smem + (slot == 0 ? NS - 1 : slot - 1) * Cfg::STAGE_BYTES;
+        for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{}, std::false_type{}, kt + 1 == kt1);
+        // every wave passed the last k-step's barrier after its final read of slot ^ 1
+        uint8_t* free_stage = smem + (slot ^ 1) * Cfg::STAGE_BYTES;
         epi.partial(cur.partial());
         epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
         if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
+        if (keep_slot) {
+            wg_barrier();          // all waves are done with the scratch
+            refill(slot ^ 1);
+        }
         cur.advance();
     }
     wg_barrier();
