@@ -144,6 +144,25 @@ int ngpt_quant_transpose_down(const void* weights_bf16, int num_layers, int hidd
                               int64_t layer_stride, const float* scales, void* out_f8, float* used_scales,
                               float* partial_amax, void* stream);
 
+/* MLP input producer, train_gpt.py:1643-1647 with norm() = F.rms_norm(x, (dim,)) (:952-953):
+ *   normed  = rms_norm(x)                         bf16 [rows, dim]
+ *   amax    = max(|normed|) clamped to 1e-12      (bf16 value)
+ *   x_f8    = e4m3(bf16(normed * bf16(448 / amax)))
+ *   dequant = up_scale[0] * amax / 448            1-element fp32 device buffer (no host sync)
+ * Two passes over the activations.  up_scale and dequant are device pointers.  dim % 8 == 0, dim <= 2048.
+ * workspace: ngpt_mlp_input_quant_workspace_bytes() bytes of device memory. */
+int64_t ngpt_mlp_input_quant_workspace_bytes(void);
+int ngpt_mlp_input_quant(const void* x_bf16, int rows, int dim, const float* up_scale, void* normed_bf16,
+                         void* x_f8, float* dequant, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Up-projection part of GPT.quantize_mlp_fp8, train_gpt.py:1419-1422: per layer l of w [layers, per_layer] bf16,
+ *   scales[l] = bf16(max(amax(|w_l|), 1e-12) / 448)   (written as fp32)
+ *   w_f8[l]   = e4m3(bf16(w_l / scales[l]))
+ * per_layer % 8 == 0.  workspace: ngpt_quant_up_weights_workspace_bytes(layers) bytes. */
+int64_t ngpt_quant_up_weights_workspace_bytes(int layers);
+int ngpt_quant_up_weights(const void* w_bf16, int layers, int64_t per_layer, void* w_f8, float* scales,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+
 /* dst [cols, rows] += src [rows, cols]^T for bf16 (elem_bytes 2) or fp32 (4):
  * transpose_add, triton_kernels.py:844-903. */
 int ngpt_transpose_add(const void* src, int rows, int cols, void* dst, int elem_bytes, void* stream);

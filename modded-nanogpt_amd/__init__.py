@@ -10,10 +10,10 @@ from . import _lib, ops                                   # noqa: F401  (registe
 from .fused import (FusedLinearReLUSquareFunction, FusedSoftcappedCrossEntropy, ReLUSqrdMLP,  # noqa: F401
                     linear_relu_square, quantize_transpose_mlp_down_weights, reduce_mlp_activation_scales,
                     transpose_add, transpose_copy)
-from .ops import gemm_fp8_tn, quant_fp8, quant_fp8_2d     # noqa: F401
+from .ops import gemm_fp8_tn, mlp_input_quant, quant_fp8, quant_fp8_2d, quant_up_weights     # noqa: F401
 
 __all__ = [
     "FusedLinearReLUSquareFunction", "FusedSoftcappedCrossEntropy", "ReLUSqrdMLP",
     "linear_relu_square", "transpose_copy", "transpose_add", "quantize_transpose_mlp_down_weights",
-    "reduce_mlp_activation_scales", "gemm_fp8_tn", "quant_fp8", "quant_fp8_2d",
+    "reduce_mlp_activation_scales", "gemm_fp8_tn", "quant_fp8", "quant_fp8_2d", "mlp_input_quant", "quant_up_weights",
 ]

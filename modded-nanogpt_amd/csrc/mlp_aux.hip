@@ -94,6 +94,135 @@ __global__ __launch_bounds__(256) void transpose_add_kernel(const T* __restrict_
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// MLP input producer: rms-norm, per-tensor amax and dynamic e4m3 quantisation (two passes over the
+// activations instead of the two reductions plus two element-wise passes of the eager formulation).
+constexpr int kNormPartials = 1024;      // per-workgroup running maxima of |normed|
+
+// Pass 1.  One wave per row: normed = bf16(x * rsqrt(mean(x^2) + eps)) in fp32 like F.rms_norm on
+// bf16 input with eps = None (machine epsilon of fp32); partial[bid] = max |normed| seen by the workgroup.
+__global__ __launch_bounds__(256) void rmsnorm_amax_kernel(const uint16_t* __restrict__ x, int rows, int dim,
+                                                           uint16_t* __restrict__ normed, float* __restrict__ partial) {
+    __shared__ float red[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int chunks = dim / 8;              // 16-byte chunks per row
+    float amax = 0.0f;
+    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+        const v4i* xr = (const v4i*)(x + (int64_t)row * dim);
+        v4i buf[4];                          // up to 4 chunks per lane: dim <= 2048
+        float ss = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            int ch = lane + 64 * c;
+            if (ch < chunks) {
+                buf[c] = xr[ch];
+                const uint32_t u[4] = {(uint32_t)buf[c].x, (uint32_t)buf[c].y, (uint32_t)buf[c].z, (uint32_t)buf[c].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float lo = bf16_bits_to_f32(u[i] & 0xffffu), hi = bf16_bits_to_f32(u[i] >> 16);
+                    ss += lo * lo + hi * hi;
+                }
+            }
+        }
+        ss = wave_sum(ss);
+        const float r = __fdiv_rn(1.0f, __fsqrt_rn(ss / (float)dim + 1.1920928955078125e-07f));
+        v4i* nr = (v4i*)(normed + (int64_t)row * dim);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            int ch = lane + 64 * c;
+            if (ch < chunks) {
+                const uint32_t u[4] = {(uint32_t)buf[c].x, (uint32_t)buf[c].y, (uint32_t)buf[c].z, (uint32_t)buf[c].w};
+                uint32_t o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float lo = round_to_bf16(bf16_bits_to_f32(u[i] & 0xffffu) * r);
+                    float hi = round_to_bf16(bf16_bits_to_f32(u[i] >> 16) * r);
+                    amax = fmaxf(amax, fmaxf(fabsf(lo), fabsf(hi)));
+                    o[i] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
+                }
+                nr[ch] = (v4i){(int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+            }
+        }
+    }
+    amax = wave_max(amax);
+    if (lane == 0) red[wave] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) partial[blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+__device__ __forceinline__ float block_max_of(const float* __restrict__ v, int n, float* red) {
+    float m = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) m = fmaxf(m, v[i]);
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// Pass 2.  amax = max(partials) clamped to bf16(1e-12); x_f8 = e4m3(bf16(normed * bf16(448 / amax)))
+// (every bf16 operation of the eager expression rounds); dequant[0] = up_scale * amax / 448 in fp32.
+__global__ __launch_bounds__(256) void amax_quant_kernel(const v4i* __restrict__ normed, int64_t n8, const float* __restrict__ partial,
+                                                         int npartial, const float* __restrict__ up_scale,
+                                                         v2i* __restrict__ x_f8, float* __restrict__ dequant) {
+    __shared__ float red[4];
+    float amax = fmaxf(block_max_of(partial, npartial, red), round_to_bf16(1.0e-12f));
+    if (blockIdx.x == 0 && threadIdx.x == 0) dequant[0] = __fdiv_rn(up_scale[0] * amax, 448.0f);
+    const float q = round_to_bf16(__fdiv_rn(448.0f, amax));
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+        v4i v = normed[i];
+        const uint32_t u[4] = {(uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w};
+        uint32_t c[8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            c[2 * k] = f32_to_e4m3_torch(round_to_bf16(bf16_bits_to_f32(u[k] & 0xffffu) * q));
+            c[2 * k + 1] = f32_to_e4m3_torch(round_to_bf16(bf16_bits_to_f32(u[k] >> 16) * q));
+        }
+        x_f8[i] = (v2i){(int)(c[0] | c[1] << 8 | c[2] << 16 | c[3] << 24), (int)(c[4] | c[5] << 8 | c[6] << 16 | c[7] << 24)};
+    }
+}
+
+// Up-projection weights, per layer: partial[l, b] = max |w| over a slice of layer l ...
+__global__ __launch_bounds__(256) void layer_amax_kernel(const v4i* __restrict__ w, int64_t n8_per_layer, float* __restrict__ partial) {
+    __shared__ float red[4];
+    const int layer = blockIdx.y;
+    const v4i* wl = w + layer * n8_per_layer;
+    float m = 0.0f;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8_per_layer; i += (int64_t)gridDim.x * 256) {
+        v4i v = wl[i];
+        const uint32_t u[4] = {(uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            m = fmaxf(m, fmaxf(fabsf(bf16_bits_to_f32(u[k] & 0xffffu)), fabsf(bf16_bits_to_f32(u[k] >> 16))));
+    }
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) partial[layer * gridDim.x + blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// ... then scale[l] = bf16(max(amax_l, bf16(1e-12)) / 448) and w_f8 = e4m3(bf16(w / scale[l])).
+__global__ __launch_bounds__(256) void layer_quant_kernel(const v4i* __restrict__ w, int64_t n8_per_layer, const float* __restrict__ partial,
+                                                          int npartial, v2i* __restrict__ w_f8, float* __restrict__ scales) {
+    __shared__ float red[4];
+    const int layer = blockIdx.y;
+    const float amax = fmaxf(block_max_of(partial + layer * npartial, npartial, red), round_to_bf16(1.0e-12f));
+    const float scale = round_to_bf16(__fdiv_rn(amax, 448.0f));
+    if (blockIdx.x == 0 && threadIdx.x == 0) scales[layer] = scale;
+    const v4i* wl = w + layer * n8_per_layer;
+    v2i* ol = w_f8 + layer * n8_per_layer;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8_per_layer; i += (int64_t)gridDim.x * 256) {
+        v4i v = wl[i];
+        const uint32_t u[4] = {(uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w};
+        uint32_t c[8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            c[2 * k] = f32_to_e4m3_torch(round_to_bf16(__fdiv_rn(bf16_bits_to_f32(u[k] & 0xffffu), scale)));
+            c[2 * k + 1] = f32_to_e4m3_torch(round_to_bf16(__fdiv_rn(bf16_bits_to_f32(u[k] >> 16), scale)));
+        }
+        ol[i] = (v2i){(int)(c[0] | c[1] << 8 | c[2] << 16 | c[3] << 24), (int)(c[4] | c[5] << 8 | c[6] << 16 | c[7] << 24)};
+    }
+}
+
 }  // namespace ngpt
 
 using namespace ngpt;
@@ -132,4 +261,47 @@ extern "C" int ngpt_transpose_add(const void* src, int rows, int cols, void* dst
     else
         return fail(NGPT_EINVAL, "ngpt_transpose_add: elem_bytes=%d (2 = bf16, 4 = fp32)", elem_bytes);
     return check_launch("transpose_add_kernel");
+}
+
+extern "C" int64_t ngpt_mlp_input_quant_workspace_bytes(void) { return kNormPartials * (int64_t)sizeof(float); }
+
+extern "C" int ngpt_mlp_input_quant(const void* x_bf16, int rows, int dim, const float* up_scale, void* normed_bf16,
+                                    void* x_f8, float* dequant, void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!x_bf16 || !up_scale || !normed_bf16 || !x_f8 || !dequant || !workspace)
+        return fail(NGPT_EINVAL, "ngpt_mlp_input_quant: null pointer");
+    if (rows <= 0 || dim <= 0) return fail(NGPT_EINVAL, "ngpt_mlp_input_quant: empty problem rows=%d dim=%d", rows, dim);
+    if (dim % 8 || dim > 2048) return fail(NGPT_EALIGN, "ngpt_mlp_input_quant: dim=%d must be a multiple of 8 and at most 2048", dim);
+    if (workspace_bytes < ngpt_mlp_input_quant_workspace_bytes())
+        return fail(NGPT_EWORKSPACE, "ngpt_mlp_input_quant: workspace %lld < %lld bytes", (long long)workspace_bytes,
+                    (long long)ngpt_mlp_input_quant_workspace_bytes());
+    hipStream_t st = (hipStream_t)stream;
+    float* partial = (float*)workspace;
+    int blocks = (rows + 3) / 4;
+    if (blocks > kNormPartials) blocks = kNormPartials;
+    rmsnorm_amax_kernel<<<blocks, 256, 0, st>>>((const uint16_t*)x_bf16, rows, dim, (uint16_t*)normed_bf16, partial);
+    if (int e = check_launch("rmsnorm_amax_kernel")) return e;
+    const int64_t n8 = (int64_t)rows * dim / 8;
+    int grid = (int)((n8 + 255) / 256 < (int64_t)num_cus() * 8 ? (n8 + 255) / 256 : (int64_t)num_cus() * 8);
+    amax_quant_kernel<<<grid, 256, 0, st>>>((const v4i*)normed_bf16, n8, partial, blocks, up_scale, (v2i*)x_f8, dequant);
+    return check_launch("amax_quant_kernel");
+}
+
+constexpr int kLayerPartials = 64;
+extern "C" int64_t ngpt_quant_up_weights_workspace_bytes(int layers) { return (int64_t)layers * kLayerPartials * sizeof(float); }
+
+extern "C" int ngpt_quant_up_weights(const void* w_bf16, int layers, int64_t per_layer, void* w_f8, float* scales,
+                                     void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!w_bf16 || !w_f8 || !scales || !workspace) return fail(NGPT_EINVAL, "ngpt_quant_up_weights: null pointer");
+    if (layers <= 0 || per_layer <= 0) return fail(NGPT_EINVAL, "ngpt_quant_up_weights: empty problem");
+    if (per_layer % 8) return fail(NGPT_EALIGN, "ngpt_quant_up_weights: elements per layer (%lld) must be a multiple of 8", (long long)per_layer);
+    if (workspace_bytes < ngpt_quant_up_weights_workspace_bytes(layers))
+        return fail(NGPT_EWORKSPACE, "ngpt_quant_up_weights: workspace %lld < %lld bytes", (long long)workspace_bytes,
+                    (long long)ngpt_quant_up_weights_workspace_bytes(layers));
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t n8 = per_layer / 8;
+    layer_amax_kernel<<<dim3(kLayerPartials, layers), 256, 0, st>>>((const v4i*)w_bf16, n8, (float*)workspace);
+    if (int e = check_launch("layer_amax_kernel")) return e;
+    layer_quant_kernel<<<dim3(kLayerPartials, layers), 256, 0, st>>>((const v4i*)w_bf16, n8, (const float*)workspace, kLayerPartials,
+                                                                    (v2i*)w_f8, scales);
+    return check_launch("layer_quant_kernel");
 }

@@ -355,6 +355,77 @@ def _(dy, w2, post):
 
 
 # ------------------------------------------------------------------------------------------------
+# MLP input producer (reference train_gpt.py:1643-1647) and the up-projection weight quantiser (:1419-1422)
+
+@torch.library.custom_op("nanogpt::mlp_input_quant", mutates_args=())
+def mlp_input_quant(x: Tensor, up_scale: Tensor) -> tuple[Tensor, Tensor, Tensor]:
+    """(normed, x_f8, dequant) = (rms_norm(x), e4m3(normed * (448 / amax(|normed|))), up_scale * amax / 448) for
+    bf16 x [..., D]; dequant is a 1-element fp32 device tensor (what the reference keeps in
+    `_mlp_dequant_scale_buf`).  Nothing synchronises with the host."""
+    _gpu(x, up_scale)
+    assert x.dtype == torch.bfloat16 and x.is_contiguous()
+    assert up_scale.dtype == torch.float32 and up_scale.numel() >= 1
+    dequant = torch.empty(1, dtype=torch.float32, device=x.device)
+    dim = x.shape[-1]
+    rows = x.numel() // dim
+    lib = _lib.load()
+    normed = torch.empty_like(x)
+    x_f8 = torch.empty(x.shape, dtype=E4M3, device=x.device)
+    nbytes = lib.ngpt_mlp_input_quant_workspace_bytes()
+    ws = _workspace(nbytes, x.device)
+    _lib.check(lib.ngpt_mlp_input_quant(_p(x), rows, dim, _p(up_scale), _p(normed), _p(x_f8), _p(dequant), _p(ws), nbytes,
+                                        _stream(x)), "ngpt_mlp_input_quant")
+    return normed, x_f8, dequant
+
+
+@mlp_input_quant.register_fake
+def _(x, up_scale):
+    return (torch.empty_like(x), torch.empty(x.shape, dtype=E4M3, device=x.device),
+            torch.empty(1, dtype=torch.float32, device=x.device))
+
+
+def _mlp_input_quant_setup(ctx, inputs, output):
+    ctx.save_for_backward(inputs[0])
+
+
+def _mlp_input_quant_backward(ctx, d_normed, d_x_f8, d_dequant):
+    # x_f8 and dequant come from detached values in the reference; the gradient flows through the norm only
+    (x,) = ctx.saved_tensors
+    if d_normed is None:
+        return None, None
+    with torch.enable_grad():
+        xr = x.detach().requires_grad_(True)
+        y = torch.nn.functional.rms_norm(xr, (xr.size(-1),))
+    (dx,) = torch.autograd.grad(y, xr, d_normed)
+    return dx, None
+
+
+mlp_input_quant.register_autograd(_mlp_input_quant_backward, setup_context=_mlp_input_quant_setup)
+
+
+@torch.library.custom_op("nanogpt::quant_up_weights", mutates_args=())
+def quant_up_weights(w: Tensor) -> tuple[Tensor, Tensor]:
+    """Per-layer e4m3 copy of w [L, ...] bf16 with scales[l] = amax(|w[l]|).clamp(1e-12) / 448 (fp32 [L])."""
+    _gpu(w)
+    assert w.dtype == torch.bfloat16 and w.is_contiguous() and w.ndim >= 2
+    layers = w.shape[0]
+    per_layer = w.numel() // layers
+    lib = _lib.load()
+    w_f8 = torch.empty(w.shape, dtype=E4M3, device=w.device)
+    scales = torch.empty(layers, dtype=torch.float32, device=w.device)
+    nbytes = lib.ngpt_quant_up_weights_workspace_bytes(layers)
+    ws = _workspace(nbytes, w.device)
+    _lib.check(lib.ngpt_quant_up_weights(_p(w), layers, per_layer, _p(w_f8), _p(scales), _p(ws), nbytes, _stream(w)),
+               "ngpt_quant_up_weights")
+    return w_f8, scales
+
+
+@quant_up_weights.register_fake
+def _(w):
+    return torch.empty(w.shape, dtype=E4M3, device=w.device), torch.empty(w.shape[0], dtype=torch.float32, device=w.device)
+
+
+# ------------------------------------------------------------------------------------------------
 # Building blocks exposed for callers and tests (plain functions, not registered ops)
 
 def quant_fp8(x: Tensor, scale: float, dtype: torch.dtype = E4M3) -> Tensor:

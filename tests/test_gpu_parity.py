@@ -396,3 +396,42 @@ def test_dpre_bf16_kernel(amd, oracle, M, D, H):
     assert_close_gemm(got, ref)
     assert torch.equal(got.cpu() == 0, ref == 0) or ((got.cpu() == 0) != (ref == 0)).float().mean() < 1e-4
     assert (got.cpu() == ref).float().mean() > 0.97            # fp32 accumulation order only moves bf16 ties
+
+
+@pytest.mark.parametrize("rows,dim", [(64, 768), (1000, 768), (4096, 1024), (16, 2048)])
+def test_mlp_input_quant(amd, oracle, rows, dim):
+    """rms-norm + amax + dynamic e4m3 quantisation of the MLP input against the eager formulation."""
+    g = torch.Generator().manual_seed(rows + dim)
+    x = (torch.randn(rows, dim, generator=g) * torch.rand(rows, 1, generator=g) * 3).bfloat16()
+    up_scale = torch.tensor([0.0123], dtype=torch.float32)
+    normed, x_f8, dequant = torch.ops.nanogpt.mlp_input_quant(dev(x), dev(up_scale))
+    ref_n = oracle.rms_norm(x)
+    # the row sum of squares is accumulated in a different order: a few results may land on the other side of a bf16 tie
+    n_cpu = normed.cpu()
+    assert (n_cpu == ref_n).float().mean() > 0.999
+    torch.testing.assert_close(n_cpu.float(), ref_n.float(), rtol=2 ** -7, atol=0)
+    # given the kernel's own normed values the quantisation is bit-exact
+    ref_f8, ref_dq = oracle.mlp_input_quant(n_cpu, up_scale)
+    assert torch.equal(x_f8.cpu().view(torch.uint8), ref_f8.view(torch.uint8))
+    assert torch.equal(dequant.cpu(), ref_dq)
+
+
+def test_mlp_input_quant_grad(amd):
+    x = torch.randn(256, 768).bfloat16()
+    xd = dev(x).requires_grad_(True)
+    normed, _, _ = torch.ops.nanogpt.mlp_input_quant(xd, torch.ones(1, device="cuda"))
+    gy = torch.randn(256, 768).bfloat16()
+    normed.backward(dev(gy))
+    xr = x.clone().requires_grad_(True)
+    torch.nn.functional.rms_norm(xr, (768,)).backward(gy)
+    torch.testing.assert_close(xd.grad.cpu().float(), xr.grad.float(), rtol=2e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("L,H,D", [(3, 256, 128), (12, 3072, 768)])
+def test_quant_up_weights(amd, oracle, L, H, D):
+    g = torch.Generator().manual_seed(L)
+    w = (torch.randn(L, H, D, generator=g) * torch.logspace(-2, 0, L).view(L, 1, 1)).bfloat16()
+    w_f8, scales = torch.ops.nanogpt.quant_up_weights(dev(w))
+    ref_f8, ref_s = oracle.quantize_up_weights(w)
+    assert torch.equal(scales.cpu(), ref_s)
+    assert torch.equal(w_f8.cpu().view(torch.uint8), ref_f8.view(torch.uint8))
