@@ -79,13 +79,20 @@ struct TileCfg {
 // numbers form a 4 x 8 block of tiles that shares 4 A panels and 8 B panels.  Workgroups are
 // dealt to the 8 XCDs round-robin by the dispatcher (workgroup b runs on XCD b % 8); giving
 // XCD x the sequence numbers [32x, 32x+32) of every batch of 256 keeps such a block inside one
-// XCD's L2.
+// XCD's L2.  An output with few tile columns (the skinny backward GEMMs: 3) is walked row-major
+// instead: the tiles of one row, which share the long A panel, are consecutive, so only the rows that
+// straddle a multiple of 32 are fetched by two XCDs.
 struct TileOrder {
     int tiles_r, tiles_c, total;
     __device__ TileOrder(int R, int C, int BM, int BN)
         : tiles_r((R + BM - 1) / BM), tiles_c((C + BN - 1) / BN), total(tiles_r * tiles_c) {}
     __device__ void coords(int seq, int& tr, int& tc) const {
         constexpr int GROUP = 4;
+        if (tiles_c <= 8 && tiles_r > GROUP) {
+            tr = seq / tiles_c;
+            tc = seq - tr * tiles_c;
+            return;
+        }
         int per_group = GROUP * tiles_c;
         int grp = seq / per_group;
         int first = grp * GROUP;
