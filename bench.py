@@ -26,6 +26,16 @@ import torch
 PEAK_FP8_TFLOPS = 5033.0      # MI355X dense FP8 MFMA (published)
 M, K, V = 49152, 768, 50304
 SLOT_NAMES = ["lm_head_ce_fwd", "dlogits_recompute", "dx_gemm", "dw_gemm", "other_gemm"]
+# HBM bytes (read + write) per launch at this workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script scaled by a 1 GiB copy in the same run (FETCH_SIZE x 2 KiB, WRITE_SIZE x 1 KiB); the runs and
+# their commands are in profiles/lmhead_ce_cfg3_hbm_traffic.txt.  Counters cannot be read from inside the
+# process, so these are recorded values, not live ones.
+MEASURED_HBM_BYTES = {
+    "lm_head_ce_fwd": 975.8e6 + 3.8e6,
+    "dlogits_recompute": 3637.7e6 + 5639.5e6,
+    "dx_gemm": 3835.8e6 + 134.3e6 + 16.8e6 + 25.2e6,
+    "dw_gemm": 3867.9e6 + 195.2e6 + 20.3e6,
+}
 
 
 def profile_read(lib):
@@ -137,7 +147,8 @@ def main() -> int:
     achieved = flops_per_launch[dominant] / (dom["avg_ms"] * 1e-3) / 1e12
     roofline = {
         "bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-        "frac": achieved / PEAK_FP8_TFLOPS, "traffic": None,
+        "frac": achieved / PEAK_FP8_TFLOPS, "traffic": MEASURED_HBM_BYTES.get(dominant),
+        "traffic_unit": "bytes per launch (recorded rocprofv3 FETCH_SIZE + WRITE_SIZE measurement, see profiles/)",
         "avg_launch_ms": dom["avg_ms"], "flop_per_launch": flops_per_launch[dominant],
         "note": "executed 2*rows*K*V FLOP per launch of each GEMM-shaped kernel / its HIP-event duration",
     }

@@ -56,11 +56,11 @@ int ngpt_num_cus(void);
 int ngpt_profile_enable(int on);
 int ngpt_profile_read(int slot, double* total_ms, int* launches);
 
-/* Tuning / timing aid, no counterpart in the reference.  key 0: GEMM tile configuration (0 = default
- * 256x256 two-stage, 1 = 256x256 four-stage, 5 = 256x128 two workgroups per CU); key 2: ablation bits
- * for timing runs (1 = no operand loads, 2 = no MFMAs, 4 = no k-loop barrier; results are then
- * meaningless); key 4: split-K factor used by ngpt_gemm_fp8_tn with out_kind 2; key 5: tile
- * configuration of the fused CE kernels; key 6: split-K in the fused CE backward GEMMs. */
+/* Timing aid, no counterpart in the reference.  key 2: ablation bits for timing runs of
+ * ngpt_gemm_fp8_tn with out_kind 3 (1 = no operand loads, 2 = no MFMAs, 4 = no k-loop barrier; results
+ * are then meaningless); key 4: split-K factor used by ngpt_gemm_fp8_tn with out_kind 2; key 7: 1 =
+ * accept operand row strides below K (overlapping rows keep the operands cache resident in timing runs).
+ * Other keys are reserved. */
 int ngpt_tuning_set(int key, int value);
 
 /* ---- quantisers ---------------------------------------------------------------------------

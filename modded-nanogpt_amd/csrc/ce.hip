@@ -446,7 +446,6 @@ __device__ __forceinline__ uint32_t quad_transpose_u8(uint32_t x, uint32_t sel1,
 struct EpiDlStore {
     static constexpr int TILE_STORES = 16;   // 8 dw-panel + 8 dx-panel 16-byte stores per wave and tile, always
     static constexpr bool HAS_TILE_BEGIN = true;
-    static constexpr bool TIGHT_REGISTERS = true;
     static constexpr int EXTRA_LDS = 2048;   // row factors of the current and the next tile (2 x 256 floats)
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;

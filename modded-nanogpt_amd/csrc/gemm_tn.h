@@ -421,14 +421,6 @@ struct EpiHasTileBegin : std::false_type {};
 template <class E>
 struct EpiHasTileBegin<E, std::void_t<decltype(E::HAS_TILE_BEGIN)>> : std::bool_constant<E::HAS_TILE_BEGIN> {};
 
-// Epilogues with `static constexpr bool TIGHT_REGISTERS = true` need every register in tile(): the last
-// k-step of a job then does not read the next job's first fragments ahead (they would stay live across
-// the epilogue).
-template <class E, class = void>
-struct EpiTightRegisters : std::false_type {};
-template <class E>
-struct EpiTightRegisters<E, std::void_t<decltype(E::TIGHT_REGISTERS)>> : std::bool_constant<E::TIGHT_REGISTERS> {};
-
 template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(GemmOperands g, Epi epi) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_all[];

@@ -11,7 +11,7 @@ using MainCfg = TileCfg<256, 256, 4, 2, 128, 2>;
 // 256 x 128 tile with two 4-wave workgroups per CU.  The kernel stays generic over TileCfg.)
 
 // Tuning keys: [2] ablation bits (timing aid, honoured by the discarding epilogue only),
-// [4] split-K factor of ngpt_gemm_fp8_tn, [6] 1 = split-K in the CE backward GEMMs,
+// [4] split-K factor of ngpt_gemm_fp8_tn,
 // [7] 1 = accept operand row strides below K (timing aid: overlapping rows keep the operands cache resident)
 extern int g_tuning[8];
 
