@@ -285,6 +285,23 @@ def ce_fwd_bwd(logits: Tensor, targets: Tensor, mtp_weights: Tensor, prefix_targ
     return losses, e5m2_satfinite(g), lse
 
 
+def ce_grad_columns(logits_cols: Tensor, cols: Tensor, lse: Tensor, targets: Tensor,
+                    A: float, B: float, C: float, grad_s: float, grad_scale: float) -> Tensor:
+    """The gradient that ce_fwd_bwd stores, for a subset `cols` of the vocabulary columns only
+    (n_predict = 1, no prefix term), given the rows' log-sum-exp.  logits_cols [M, len(cols)] bf16.
+    Same expressions as ce_fwd_bwd above (triton_kernels.py:1100-1123); used by the full-size tests, where
+    whole rows of logits do not fit a CPU run."""
+    A32 = torch.tensor(A, dtype=torch.float32)
+    sig = softcap_sigma(logits_cols, B, C)
+    z = A32 * sig
+    p = torch.exp(z - lse.unsqueeze(1))
+    term2 = (targets.unsqueeze(1) == cols.unsqueeze(0)).float()
+    c32 = torch.tensor(C, dtype=torch.float32)
+    coef = (torch.tensor(grad_scale, dtype=torch.float32) * (1.0 / c32 * A32)
+            * (1.0 / torch.tensor(grad_s, dtype=torch.float32)))
+    return e5m2_satfinite(coef * (p - term2) * sig * (1.0 - sig))
+
+
 # a12: closed form on un-rounded sigma, the pin for ce_fwd_bwd
 
 def _upcast(t: Tensor) -> Tensor:
