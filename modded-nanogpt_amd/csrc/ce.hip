@@ -412,19 +412,19 @@ __global__ void ce_rowf_kernel(const float* __restrict__ lse, CandArgs ca, Softc
 }
 
 // ------------------------------------------------------------------------------------------------
-// dlogits panels.  The e5m2 gradient of a chunk of tokens is consumed twice: as the A operand of
-// dx = dl . W (rows = tokens, contraction = vocabulary) and as an operand of dW = dl^T . x (rows =
-// vocabulary, contraction = tokens).  It is written once in each orientation, panel-blocked (see
-// GemmOperands), and with the contraction bytes of every 128-byte k-step row permuted into the order
-// in which the recompute kernel's accumulator registers already hold them, so that both copies leave
-// the registers as full 16-byte stores without a trip through LDS.  A GEMM is indifferent to the
-// order of its contraction as long as both operands agree, so the other operand of each product
-// (W^T, x^T) is produced with the same permutation by panel_transpose_kernel.
+// dlogits panel.  The e5m2 gradient is consumed twice: as an operand of dW = dl^T . x (rows =
+// vocabulary, contraction = tokens) and as the A operand of dx = dl . W (rows = tokens, contraction =
+// vocabulary).  It is written ONCE, vocabulary-major and panel-blocked (see GemmOperands): blocks
+// [V / 256][tokens / 128], 128-byte rows = 128 tokens of one vocabulary column.  Inside such a row the
+// tokens of every 32-group sit in the order in which the recompute kernel's accumulator registers hold
+// them (dw_pos), so the panel leaves the registers as full 16-byte stores without a trip through
+// LDS; x^T, the other operand of dW, is produced with the same token order by panel_transpose_kernel
+// (a GEMM does not care about the order of its contraction as long as both operands agree).
+// The dx GEMM reads the same panel as the transpose of its A operand and transposes it on the way from
+// LDS to the MFMA registers (FMT_TRANSPOSED); its output rows come out in dw_pos order, which its
+// epilogue undoes (AccCoords::perm).
 //
-// token-major panel ("dx panel"):  vocabulary column vv of a k-step (0..127) sits at byte dx_pos(vv)
-// vocab-major panel ("dw panel"):  token tt of a k-step (0..127) sits at byte dw_pos(tt)
-__host__ __device__ inline int dx_pos(int vv) { return 16 * ((vv & 31) >> 2) + 4 * (vv >> 5) + (vv & 3); }
-__host__ __device__ inline int dx_pos_inv(int p) { return 32 * ((p >> 2) & 3) + 4 * (p >> 4) + (p & 3); }
+// token tt of a k-step (0..127) sits at byte dw_pos(tt) of the row
 __host__ __device__ inline int dw_pos(int tt) { return (tt & ~31) | (((tt >> 2) & 1) << 4) | (((tt >> 3) & 3) << 2) | (tt & 3); }
 __host__ __device__ inline int dw_pos_inv(int p) { return (p & ~31) | (((p >> 2) & 3) << 3) | (((p >> 4) & 1) << 2) | (p & 3); }
 
@@ -432,19 +432,11 @@ __host__ __device__ inline int64_t panel_offset(int row, int kbyte, int nk /* k-
     return ((int64_t)(row >> 8) * nk + (kbyte >> 7)) * kPanelBytes + (row & 255) * 128;
 }
 
-// 4 x 4 byte transpose across the four lanes of a quad: lane m ends up with byte m of lanes 0..3.
-__device__ __forceinline__ uint32_t quad_transpose_u8(uint32_t x, uint32_t sel1, uint32_t sel2) {
-    uint32_t y = (uint32_t)__builtin_amdgcn_mov_dpp((int)x, 0xB1, 0xf, 0xf, true);   // quad_perm [1,0,3,2]
-    uint32_t r = __builtin_amdgcn_perm(x, y, sel1);
-    uint32_t z = (uint32_t)__builtin_amdgcn_mov_dpp((int)r, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
-    return __builtin_amdgcn_perm(r, z, sel2);
-}
-
 // Epilogue of the backward's logits recompute (A = x chunk, rows = tokens; B = W, rows = vocabulary):
-// dl = e5m2_sat(rowf[token] * D(logit)) written to both panels.  Rows past Mc get rowf = 0, i.e. zero codes,
-// so the token padding of the dw panel contracts to nothing.
+// dl = e5m2_sat(rowf[token] * D(logit)) written to the panel.  Rows past Mc get rowf = 0, i.e. zero codes,
+// so the token padding of the panel contracts to nothing.
 struct EpiDlStore {
-    static constexpr int TILE_STORES = 16;   // 8 dw-panel + 8 dx-panel 16-byte stores per wave and tile, always
+    static constexpr int TILE_STORES = 8;    // 16-byte panel stores per wave and tile, always
     static constexpr bool HAS_TILE_BEGIN = true;
     static constexpr int EXTRA_LDS = 2048;   // row factors of the current and the next tile (2 x 256 floats)
     static constexpr bool NEEDS_SCRATCH = false;
@@ -453,10 +445,8 @@ struct EpiDlStore {
     __device__ void job_begin(int) {}
     const float* gtabD;
     const float* rowf;     // already offset to the chunk's first row
-    uint8_t* dx_panel;     // [Mt / 256][V / 128] blocks, Mt = Mc rounded up to 256, plus one more block: the sink
-                           // for the stores of the columns past V in the last vocabulary tile
-    uint8_t* dw_panel;     // [Vp / 256][Mt / 128] blocks, Vp = V rounded up to 256
-    int Mc, V, nkv, nkt;   // k-steps per panel row: V / 128, Mt / 128
+    uint8_t* dw_panel;     // [Vp / 256][Mt / 128] blocks, Vp / Mt = V / Mc rounded up to 256
+    int Mc, V, nkt;        // nkt = k-steps per panel row = Mt / 128
     float scale;
     float* rowf_lds;       // LDS [2][256]
     int rslot;
@@ -492,17 +482,9 @@ struct EpiDlStore {
         const int h = lane >> 5, j = lane & 31;
         const float* tab = lds_table();
         const int wr = co.wave_row0 >> 6, wc = co.wave_col0 >> 7;
-        // dw panel: row = vocabulary column of this lane, 16 bytes = 16 tokens of one (tm, h) group
+        // row = vocabulary column of this lane, 16 bytes = 16 tokens of one (tm, h) group
         uint8_t* dw_base = dw_panel + ((int64_t)(c0 >> 8) * nkt + (r0 >> 7) + (wr >> 1)) * kPanelBytes;
         const uint32_t dw_lane = (uint32_t)((128 * wc + j) * 128 + 64 * (wr & 1) + 16 * h);
-        // dx panel: row = token, 16 bytes = vocabulary columns 4q..4q+3 of the four tn blocks
-        const int ktv = (c0 >> 7) + wc;
-        // the last vocabulary tile may be half empty: its stores go to the sink block behind the panel
-        const int64_t dx_block = ktv < nkv ? (int64_t)(r0 >> 8) * nkv + ktv : (int64_t)((Mc + 255) >> 8) * nkv;
-        uint8_t* dx_base = dx_panel + dx_block * kPanelBytes;
-        const uint32_t dx_lane = (uint32_t)((64 * wr + 4 * h + (j & 3)) * 128 + 16 * (j >> 2));
-        const uint32_t sel1 = (j & 1) ? 0x07030501u : 0x02060004u;
-        const uint32_t sel2 = (j & 2) ? 0x07060302u : 0x01000504u;
 #pragma unroll
         for (int tm = 0; tm < Cfg::TM; ++tm) {
             uint32_t pk[Cfg::TN][4];
@@ -524,13 +506,6 @@ struct EpiDlStore {
             for (int tn = 0; tn < Cfg::TN; ++tn)
                 *(v4i*)(dw_base + (dw_lane + tn * 4096 + tm * 32)) =
                     (v4i){(int)pk[tn][0], (int)pk[tn][1], (int)pk[tn][2], (int)pk[tn][3]};
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                uint32_t t[Cfg::TN];
-#pragma unroll
-                for (int tn = 0; tn < Cfg::TN; ++tn) t[tn] = quad_transpose_u8(pk[tn][g], sel1, sel2);
-                *(v4i*)(dx_base + (dx_lane + (32 * tm + 8 * g) * 128)) = (v4i){(int)t[0], (int)t[1], (int)t[2], (int)t[3]};
-            }
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -538,8 +513,8 @@ struct EpiDlStore {
 
 // Rewrites the (at most MAX_CAND) target columns of every row of the chunk with the exact gradient.
 __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __restrict__ saved_sigma,
-                                 CandArgs ca, Softcap sc, float coef, int m_begin, int Mc, int nkv, int nkt,
-                                 uint8_t* __restrict__ dx_panel, uint8_t* __restrict__ dw_panel) {
+                                 CandArgs ca, Softcap sc, float coef, int m_begin, int Mc, int nkt,
+                                 uint8_t* __restrict__ dw_panel) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= Mc) return;
     int m = m_begin + i;
@@ -556,14 +531,13 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
         float gz = s_w * (softcap_E(sg, sc) * p_scale) - term2;
         float gx = coef * gz * sg * (1.0f - sg);
         uint8_t code = (uint8_t)(f32x2_to_e5m2_sat(gx, gx) & 0xffu);
-        dx_panel[panel_offset(i, t, nkv) + dx_pos(t & 127)] = code;
         dw_panel[panel_offset(t, i, nkt) + dw_pos(i & 127)] = code;
     }
 }
 
 // Panel-blocked transpose of a row-major fp8 matrix: out row = input column c (c < cols), contraction =
 // input rows [row0, row0 + nrows) padded with zeros to nk * 128, contraction bytes of each k-step
-// permuted by PERM (0 none, 1 dx_pos, 2 dw_pos).  One workgroup moves a 128 (rows) x 64 (columns) tile.
+// permuted by PERM (0 none, 2 dw_pos).  One workgroup moves a 128 (rows) x 64 (columns) tile.
 template <int PERM>
 __global__ __launch_bounds__(256) void panel_transpose_kernel(const uint8_t* __restrict__ in, int64_t ld, int row0, int nrows, int cols,
                                                               int nk, uint8_t* __restrict__ out) {
@@ -587,7 +561,7 @@ __global__ __launch_bounds__(256) void panel_transpose_kernel(const uint8_t* __r
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             int p = part * 32 + d * 4 + b;
-            int t = PERM == 1 ? dx_pos_inv(p) : PERM == 2 ? dw_pos_inv(p) : p;
+            int t = PERM == 2 ? dw_pos_inv(p) : p;
             word |= (uint32_t)tile[t][o] << (8 * b);
         }
         w[d] = word;
@@ -608,7 +582,7 @@ static int panel_transpose(const uint8_t* in, int64_t ld, int row0, int nrows, i
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
                float scale, void* out, int64_t ldc, int out_kind, hipStream_t st, int splits);
 int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
-                       float scale, void* out_bf16, int64_t ldc, float* part32, hipStream_t st);
+                       float scale, void* out_bf16, int64_t ldc, float* part32, int a_rows_pad, hipStream_t st);
 int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
                       float scale, float* out, int64_t ldc, bool accumulate, hipStream_t st);
 
@@ -776,12 +750,12 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
 }
 
 // ------------------------------------------------------------------------------------------------
-// backward workspace: tabE | tabD | rowf [M] | x^T panel [Kp, Mt] | W^T panel [Kp, V] | dx panel [Mt, V] + 32 KiB |
-// dw panel [Vp, Mt] | dx fp32 [Mc, K]   (Mc = tokens per pass, Mt / Kp / Vp = Mc / K / V rounded up to 256)
+// backward workspace: tabE | tabD | rowf [M] | x^T panel [Kp, Mt] | W^T panel [Kp, V] | dlogits panel [Vp, Mt] |
+// dx fp32 [Mc, K]   (Mc = tokens per pass, Mt / Kp / Vp = Mc / K / V rounded up to 256)
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
     int64_t Mc = bwd_chunk_rows(M), Mt = round256(Mc), Kp = round256(K), Vp = round256(V);
-    return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)M * 4, 256) + Kp * Mt + Kp * (int64_t)V + Mt * (int64_t)V + kPanelBytes + Vp * Mt +
+    return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)M * 4, 256) + Kp * Mt + Kp * (int64_t)V + Vp * Mt +
            align_up(Mc * K * 4, 256);
 }
 
@@ -813,10 +787,8 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     ws += align_up((int64_t)M * 4, 256);
     uint8_t* x_t = ws;       // x^T panel of the pass: rows = K features, contraction = tokens (dw_pos order)
     ws += Kp * Mt_max;
-    uint8_t* w_t = ws;       // W^T panel: rows = K features, contraction = vocabulary (dx_pos order)
+    uint8_t* w_t = ws;       // W^T panel: rows = K features, contraction = vocabulary
     ws += Kp * (int64_t)V;
-    uint8_t* dx_panel = ws;
-    ws += Mt_max * (int64_t)V + kPanelBytes;     // + the sink block
     uint8_t* dw_panel = ws;
     ws += Vp * Mt_max;
     float* dx32 = (float*)ws;
@@ -828,7 +800,7 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     ce_rowf_kernel<<<(M + 255) / 256, 256, 0, st>>>(lse, ca, sc, coef, rowf);
     if (int e = check_launch("ce_rowf_kernel")) return e;
     const int nkv = V / 128;
-    if (int e = panel_transpose<1>((const uint8_t*)w_f8_vk, K, 0, V, K, nkv, w_t, st)) return e;
+    if (int e = panel_transpose<0>((const uint8_t*)w_f8_vk, K, 0, V, K, nkv, w_t, st)) return e;
     const bool several = M > Mc_max;       // dw then accumulates over the passes
     if (several) fill_f32_kernel<<<(int)(((int64_t)V * K + 255) / 256), 256, 0, st>>>((float*)dw_f32, (int64_t)V * K, 0.0f);
 
@@ -836,27 +808,25 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         const int Mc = (M - m0 < Mc_max) ? (M - m0) : Mc_max;
         const int Mt = (int)round256(Mc), nkt = Mt / 128;
         if (int e = panel_transpose<2>((const uint8_t*)x_f8, K, m0, Mc, K, nkt, x_t, st)) return e;
-        // 1. recompute the pass's logits and turn them into e5m2 dlogits (both panels)
+        // 1. recompute the pass's logits and turn them into the e5m2 dlogits panel
         GemmOperands g{(const uint8_t*)x_f8 + (int64_t)m0 * K, (const uint8_t*)w_f8_vk, K, K, Mc, V, K, 1, 0};
         EpiDlStore epi{};
         epi.gtabD = tabD;
         epi.rowf = rowf + m0;
-        epi.dx_panel = dx_panel;
         epi.dw_panel = dw_panel;
         epi.Mc = Mc;
         epi.V = V;
-        epi.nkv = nkv;
         epi.nkt = nkt;
         epi.scale = x_s * w_s;
         if (int e = launch_grid_kernel<MainCfg>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
-        ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, nkv, nkt, dx_panel, dw_panel);
+        ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, nkt, dw_panel);
         if (int e = check_launch("ce_dl_fix_kernel")) return e;
-        // 3. dx[pass] = dl [Mc, V] . (W^T [K, V])^T
+        // 3. dx[pass] = dl [Mc, V] . (W^T [K, V])^T, dl read transposed from the panel
         {
             GemmSlot slot(PROF_CE_DX);
-            if (int e = gemm_balanced_bf16(dx_panel, FMT_E5M2, 0, w_t, FMT_E4M3, 0, kBlockedA | kBlockedB, Mc, K, V, grad_s * w_s,
-                                           (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, dx32, st)) return e;
+            if (int e = gemm_balanced_bf16(dw_panel, FMT_E5M2 | FMT_TRANSPOSED, 0, w_t, FMT_E4M3, 0, kBlockedB, Mc, K, V, grad_s * w_s,
+                                           (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, dx32, Mt, st)) return e;
         }
         // 4. dw (+)= dl^T . x over the tokens of the pass (zero padded to Mt)
         GemmSlot slot(PROF_CE_DW);

@@ -12,6 +12,9 @@ typedef float v4f  __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 enum : int { FMT_E4M3 = 0, FMT_E5M2 = 1, FMT_BF16 = 2 };   // FMT_BF16: both operands bf16, contraction counted in bytes
+// Added to the A format of the GEMM kernel: the A operand is given as the panel of its TRANSPOSE (rows =
+// contraction index) and is transposed on the way from LDS to the MFMA registers.
+constexpr int FMT_TRANSPOSED = 4;
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 constexpr int kWave = 64;

@@ -84,7 +84,7 @@ __device__ __forceinline__ void store_tile_f32(v16f (&acc)[Cfg::TM][Cfg::TN], fl
         for (int tn = 0; tn < Cfg::TN; ++tn) {
 #pragma unroll
             for (int v = 0; v < 16; v += 2) {
-                const int dr = tm * 32 + 8 * (v >> 2) + (v & 3), dc = tn * 32;
+                const int dr = co.dr(tm, v), dc = tn * 32;
                 float* pu = origin + ((int64_t)dr * ld + dc);
                 float v0 = acc[tm][tn][v] * scale, v1 = acc[tm][tn][v + 1] * scale;
                 if (full || (dr < rlim && dc < clim)) {
@@ -141,7 +141,7 @@ struct EpiStoreBf16 {
             for (int tn = 0; tn < Cfg::TN; ++tn) {
 #pragma unroll
                 for (int v = 0; v < 16; v += 2) {
-                    const int dr = tm * 32 + 8 * (v >> 2) + (v & 3), dc = tn * 32;
+                    const int dr = co.dr(tm, v), dc = tn * 32;
                     uint16_t* pu = origin + ((int64_t)dr * ld + dc);
                     uint32_t pk = cvt_pk_bf16(acc[tm][tn][v] * scale, acc[tm][tn][v + 1] * scale);
                     if (full || (dr < rlim && dc < clim)) pu[lane_off] = (uint16_t)pk;

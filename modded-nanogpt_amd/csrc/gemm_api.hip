@@ -129,15 +129,16 @@ __global__ void rem_tiles_kernel(float* part32, int64_t ld32, uint16_t* out, int
 
 // C[R, C] = scale * A . B^T with the balanced walk.  `layout`: kBlockedA | kBlockedB.
 // bf16 output: part32 is an fp32 [R, C] scratch matrix (row stride C) that only the split tiles touch.
+// fa may carry FMT_TRANSPOSED (A = panel of the transpose, a_rows_pad = R rounded up to 256).
 int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
-                       float scale, void* out_bf16, int64_t ldc, float* part32, hipStream_t st) {
+                       float scale, void* out_bf16, int64_t ldc, float* part32, int a_rows_pad, hipStream_t st) {
     if (R <= 0 || C <= 0 || K <= 0 || K % 128 || C % 4 || ldc % 4)
         return fail(NGPT_EALIGN, "gemm_balanced_bf16: R=%d C=%d K=%d ldc=%lld", R, C, K, (long long)ldc);
     BalancePlan p = plan_balance(R, C, K);
     if (p.splits > 1 && !part32) return fail(NGPT_EINVAL, "gemm_balanced_bf16: split tiles need the fp32 scratch matrix");
     ProfileScope prof(g_gemm_slot, st);
     if (p.splits > 1) rem_tiles_kernel<0><<<p.rem, 256, 0, st>>>(part32, C, nullptr, 0, R, C, p.full);
-    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full};
+    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full, a_rows_pad};
     EpiStoreBf16 epi{(uint16_t*)out_bf16, ldc, scale, R, C, part32, C, false};
     if (int e = launch_gemm<MainCfg>(g, fa, fb, epi, st)) return e;
     if (p.splits > 1) rem_tiles_kernel<1><<<p.rem, 256, 0, st>>>(part32, C, (uint16_t*)out_bf16, ldc, R, C, p.full);

@@ -32,6 +32,10 @@ namespace ngpt {
 // (r % 256) * 128 + c % 128.  A blocked operand is allocated for whole tiles (rows padded to 256).
 // One k-step then reads 2 x 32 KiB of consecutive addresses instead of 512 rows that lie a full
 // matrix row apart, which for long rows costs a TLB entry and a DRAM page per 128 bytes.
+// Transposed A (kernel instantiations with FMT_TRANSPOSED): `A` points at the panel-blocked TRANSPOSE of
+// the A matrix -- rows = the contraction index of this GEMM, 128-byte k-step rows = 128 rows of this
+// GEMM's output, blocks [contraction / 256][R / 128] -- and `a_rows_pad` is R rounded up to 256.  One
+// k-step of a tile then reads two contiguous 16 KiB pieces (128 contraction rows x 128 output rows each).
 constexpr int kBlockedA = 1, kBlockedB = 2;
 constexpr int kPanelRows = 256, kPanelBytes = kPanelRows * 128;
 
@@ -44,6 +48,7 @@ struct GemmOperands {
     int ablate;         // timing aid: bit 0 = issue no operand loads after the first, bit 1 = no MFMA work, bit 2 = no k-loop barrier
     int layout;         // kBlockedA | kBlockedB
     int full_tiles;     // the first full_tiles tiles (in walk order) are never split; 0 = `splits` applies to every tile
+    int a_rows_pad;     // transposed A only: R rounded up to 256
 };
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1>
@@ -120,10 +125,18 @@ __device__ __forceinline__ void wait_vmem_le() {
 template <class Cfg>
 struct LaneOffsets {
     uint32_t a_off[Cfg::A_LOADS], b_off[Cfg::B_LOADS];   // byte offset of this lane's chunk from the tile's first row
-    __device__ void init(const GemmOperands& g, int wave, int lane, int r0, int c0) {
+    __device__ void init(const GemmOperands& g, int wave, int lane, int r0, int c0, bool a_transposed) {
         int lrow = lane / Cfg::CPR, lchunk = lane % Cfg::CPR;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i) {
+            if (a_transposed) {
+                // 1 KiB piece `c32` of the k-step's 32: half (token block) c32 / 16, contraction rows 8 * (c32 % 16) ..+7;
+                // the 16-byte chunk q of contraction row r lands at chunk position q ^ (r & 7)
+                const int c32 = wave + i * Cfg::NWAVES;
+                const int r = 8 * (c32 & 15) + lrow;
+                a_off[i] = (uint32_t)((c32 >> 4) * kPanelBytes + r * 128 + ((lchunk ^ (r & 7)) << 4));
+                continue;
+            }
             int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
             int q = lchunk ^ Cfg::swz(R);
             if (g.layout & kBlockedA) { a_off[i] = (uint32_t)(R * 128 + q * 16); continue; }   // padded: no clamp
@@ -149,7 +162,10 @@ struct TileMainloop {
     int frag_a[Cfg::TM];     // LDS byte offset of this lane's first 16-byte chunk, stage 0, ksub 0
     int frag_b[Cfg::TN];
     int a_step, b_step;      // bytes from one k-step's slab to the next
+    int a_kt;                // transposed A: index of the next k-step to load; a_next then is the tile's base
+    int64_t a_pair_stride;   // transposed A: bytes between the panel rows of two consecutive 256-blocks of the contraction
     int wave, lane, wr, wc;
+    static constexpr bool ATR = (AFMT & FMT_TRANSPOSED) != 0;
 
     __device__ void init() {
         int tid = threadIdx.x;
@@ -164,6 +180,18 @@ struct TileMainloop {
         for (int t = 0; t < Cfg::TM; ++t) {
             int row = wr * Cfg::WTM + t * 32 + (lane & 31);
             frag_a[t] = row * Cfg::BK + ((q0 ^ Cfg::swz(row)) << 4);
+            if (ATR) {
+                // Source address of this lane for the transposing read (ds_read_b64_tr_b8: inside each block
+                // of 16 lanes, lane i receives byte i % 8 of the 8-byte rows of lanes 2j + i / 8, j = 0..7).
+                // Lane s' of a block supplies contraction row s' / 2 and output rows 8 * (s' % 2) ..+7, so lane i
+                // ends up with 8 consecutive contraction bytes of output row i.  Blocks 0, 1 serve MFMA rows
+                // 0..15, 16..31 of the first 32 contraction bytes, blocks 2, 3 the same rows of the second 32.
+                static_assert(!ATR || (Cfg::BM == 256 && Cfg::BK == 128 && Cfg::WTM == 64), "transposed A geometry");
+                const int sl = lane & 15, blk = lane >> 4;
+                const int krow = 32 * (blk >> 1) + (sl >> 1);
+                const int pos = (wr & 1) * 64 + 32 * t + 16 * (blk & 1) + 8 * (sl & 1);   // byte inside the 128-byte row
+                frag_a[t] = (wr >> 1) * (kPanelBytes / 2) + krow * 128 + ((((pos >> 4) ^ (sl >> 1)) << 4) | (pos & 15));
+            }
         }
 #pragma unroll
         for (int t = 0; t < Cfg::TN; ++t) {
@@ -181,7 +209,13 @@ struct TileMainloop {
         // a blocked operand's tile starts r0 / 256 * (K / 128) blocks in, which is r0 * K bytes
         a_next = g.A + (int64_t)r0 * ((g.layout & kBlockedA) ? (int64_t)g.K : g.lda) + (int64_t)kt * a_step;
         b_next = g.B + (int64_t)c0 * ((g.layout & kBlockedB) ? (int64_t)g.K : g.ldb) + (int64_t)kt * b_step;
-        lo.init(g, wave, lane, r0, c0);
+        if (ATR) {
+            // block (contraction / 256, output row / 128): the tile's two output-row blocks are adjacent
+            a_next = g.A + (int64_t)(r0 >> 7) * kPanelBytes;
+            a_pair_stride = (int64_t)(g.a_rows_pad >> 7) * kPanelBytes;
+            a_kt = kt;
+        }
+        lo.init(g, wave, lane, r0, c0, ATR);
     }
 
     // Loads the next k-step of the current tile into LDS slot `stage` and moves on to the one after.
@@ -189,7 +223,12 @@ struct TileMainloop {
         uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
         const uint8_t* ab = a_next;
         const uint8_t* bb = b_next;
-        a_next += a_step;
+        if (ATR) {   // contraction rows 128 * a_kt ..+127: block a_kt / 2, upper or lower half of its 256 rows
+            ab = a_next + (int64_t)(a_kt >> 1) * a_pair_stride + (a_kt & 1) * (kPanelBytes / 2);
+            ++a_kt;
+        } else {
+            a_next += a_step;
+        }
         b_next += b_step;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i)
@@ -205,6 +244,21 @@ struct TileMainloop {
         v4i lo = *(const v4i*)(s + o);
         v4i hi = *(const v4i*)(s + (o ^ 16));
         return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+
+    // A fragment through the transposing LDS read: four 8-byte reads, 8 contraction rows (1 KiB of LDS) apart.
+    __device__ __forceinline__ v8i frag_a_at(const uint8_t* s, int t, int ks) const {
+        if constexpr (ATR) {
+            typedef __attribute__((address_space(3))) v2i* lds_v2i;
+            const uint8_t* p = s + frag_a[t] + ks * 8192;
+            v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p));
+            v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 1024));
+            v2i r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 2048));
+            v2i r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 3072));
+            return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
+        } else {
+            return frag(s, frag_a[t], ks);
+        }
     }
 
     // One k-step of MFMAs on the operands in LDS slot `stage`, software-pipelined by hand.
@@ -224,7 +278,7 @@ struct TileMainloop {
                                             Refill&& refill) {
         const uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
         const uint8_t* sn = smem + next_stage * Cfg::STAGE_BYTES;
-        if constexpr (AFMT == FMT_BF16) {
+        if constexpr ((AFMT & 3) == FMT_BF16) {
             // bf16 operands: 32 contraction bytes (16 elements) per MFMA, one 16-byte chunk per lane;
             // no fragment hand-over between k-steps
             constexpr int KS = Cfg::BK / 32;
@@ -250,7 +304,7 @@ struct TileMainloop {
             v8i bcur = b0;
             if (!have) {
 #pragma unroll
-                for (int t = 0; t < Cfg::TM; ++t) a[t] = frag(s, frag_a[t], 0);
+                for (int t = 0; t < Cfg::TM; ++t) a[t] = frag_a_at(s, t, 0);
                 bcur = frag(s, frag_b[0], 0);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -264,13 +318,13 @@ struct TileMainloop {
                         bnext = frag(s, frag_b[tn + 1], ks);
                     } else if (ks + 1 < Cfg::KSUB) {
 #pragma unroll
-                        for (int t = 0; t < Cfg::TM; ++t) an[t] = frag(s, frag_a[t], ks + 1);
+                        for (int t = 0; t < Cfg::TM; ++t) an[t] = frag_a_at(s, t, ks + 1);
                         bnext = frag(s, frag_b[0], ks + 1);
                     } else {
                         sync();
                         if (want_next) {
 #pragma unroll
-                            for (int t = 0; t < Cfg::TM; ++t) an[t] = frag(sn, frag_a[t], 0);
+                            for (int t = 0; t < Cfg::TM; ++t) an[t] = frag_a_at(sn, t, 0);
                             bnext = frag(sn, frag_b[0], 0);
                         } else {
 #pragma unroll
@@ -298,14 +352,24 @@ struct TileMainloop {
 };
 
 // Coordinates of accumulator element (tm, tn, v) of this lane inside the workgroup tile.
+// `perm`: the kernel read its A operand transposed from a panel whose 128-byte rows hold the output rows
+// of every 32-group in the order position 16h + 4g + i <-> row 8g + 4h + i (the order in which the producer's
+// accumulator registers held them).  MFMA row 8a + 4H + b (register group a, lane half H) then is output
+// row {0, 16, 4, 20}[a] + 8H + b of its 32-group.
 template <class Cfg>
 struct AccCoords {
     int wave_row0, wave_col0;   // origin of this wave's sub-tile
     int row_base, col_base;     // this lane's element for tm = tn = 0, v = 0
-    __device__ AccCoords(int wr, int wc, int lane)
+    bool perm;
+    __device__ AccCoords(int wr, int wc, int lane, bool perm_ = false)
         : wave_row0(wr * Cfg::WTM), wave_col0(wc * Cfg::WTN),
-          row_base(wr * Cfg::WTM + 4 * (lane >> 5)), col_base(wc * Cfg::WTN + (lane & 31)) {}
-    __device__ int row(int tm, int v) const { return row_base + tm * 32 + 8 * (v >> 2) + (v & 3); }
+          row_base(wr * Cfg::WTM + (perm_ ? 8 : 4) * (lane >> 5)), col_base(wc * Cfg::WTN + (lane & 31)), perm(perm_) {}
+    // row of accumulator register v of MFMA tile tm, relative to row_base
+    __device__ int dr(int tm, int v) const {
+        const int a = v >> 2;
+        return tm * 32 + (perm ? ((a & 1) * 16 + (a >> 1) * 4) : 8 * a) + (v & 3);
+    }
+    __device__ int row(int tm, int v) const { return row_base + dr(tm, v); }
     __device__ int col(int tn) const { return col_base + tn * 32; }
 };
 
@@ -432,7 +496,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     ml.init();
     const int bid = blockIdx.x, G = gridDim.x;
     const int nk = g.K / Cfg::BK;
-    AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane);
+    AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane, (AFMT & FMT_TRANSPOSED) != 0);
     Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
 
     // `pre` walks the (job, k-step) sequence of this workgroup ahead of the MFMAs; `ahead` counts the
@@ -501,7 +565,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
                 sync();
                 refill_here();
             }
-            have = more && AFMT != FMT_BF16 && !(ablate & 2);
+            have = more && (AFMT & 3) != FMT_BF16 && !(ablate & 2);
             --ahead;
             slot ^= 1;
         };

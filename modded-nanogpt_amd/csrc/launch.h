@@ -34,8 +34,17 @@ int launch_gemm_fmt(const GemmOperands& g, const Epi& epi, hipStream_t st, int m
     return check_launch("gemm_tn_kernel");
 }
 
+struct EpiStoreBf16;
+
 template <class Cfg, class Epi>
 int launch_gemm_cfg(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {
+    if (fa & FMT_TRANSPOSED) {   // only the combination the fused CE backward uses is instantiated
+        if constexpr (std::is_same<Epi, EpiStoreBf16>::value) {
+            if (fa == (FMT_E5M2 | FMT_TRANSPOSED) && fb == FMT_E4M3)
+                return launch_gemm_fmt<Cfg, FMT_E5M2 | FMT_TRANSPOSED, FMT_E4M3>(g, epi, st, max_grid);
+        }
+        return fail(NGPT_EINVAL, "transposed A operand: unsupported format / output combination");
+    }
     if (fa == FMT_E4M3 && fb == FMT_E4M3) return launch_gemm_fmt<Cfg, FMT_E4M3, FMT_E4M3>(g, epi, st, max_grid);
     if (fa == FMT_E5M2 && fb == FMT_E4M3) return launch_gemm_fmt<Cfg, FMT_E5M2, FMT_E4M3>(g, epi, st, max_grid);
     if (fa == FMT_E4M3 && fb == FMT_E5M2) return launch_gemm_fmt<Cfg, FMT_E4M3, FMT_E5M2>(g, epi, st, max_grid);
