@@ -247,17 +247,36 @@ struct TileMainloop {
     }
 
     // A fragment through the transposing LDS read: four 8-byte reads, 8 contraction rows (1 KiB of LDS) apart.
+    // Written as inline assembly: behind the builtin the compiler cannot tell these reads from the LDS
+    // destinations of the direct-to-LDS loads still in flight and makes every one of them wait for
+    // vmcnt(0), which serialises the operand prefetch.  The price is that the compiler does not count
+    // them in lgkmcnt either: frag_fence() must stand between such a read and the first use of its result.
+    template <int OFF>
+    static __device__ __forceinline__ v2i read_tr8(uint32_t lds_addr) {
+        v2i r;
+        asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(r) : "v"(lds_addr), "n"(OFF));
+        return r;
+    }
+    template <int KS>
+    __device__ __forceinline__ v8i frag_a_tr(const uint8_t* s, int t) const {
+        const uint32_t p = (uint32_t)(size_t)((const __attribute__((address_space(3))) uint8_t*)s) + (uint32_t)frag_a[t];
+        v2i r0 = read_tr8<KS * 8192>(p), r1 = read_tr8<KS * 8192 + 1024>(p);
+        v2i r2 = read_tr8<KS * 8192 + 2048>(p), r3 = read_tr8<KS * 8192 + 3072>(p);
+        return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
+    }
     __device__ __forceinline__ v8i frag_a_at(const uint8_t* s, int t, int ks) const {
         if constexpr (ATR) {
-            typedef __attribute__((address_space(3))) v2i* lds_v2i;
-            const uint8_t* p = s + frag_a[t] + ks * 8192;
-            v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p));
-            v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 1024));
-            v2i r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 2048));
-            v2i r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 3072));
-            return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
+            static_assert(!ATR || Cfg::KSUB == 2, "two contraction sub-steps");
+            return ks == 0 ? frag_a_tr<0>(s, t) : frag_a_tr<1>(s, t);
         } else {
             return frag(s, frag_a[t], ks);
+        }
+    }
+    // All LDS reads issued so far have returned; ties the A fragments to that point.
+    static __device__ __forceinline__ void frag_fence(v8i (&a)[Cfg::TM]) {
+        if constexpr (ATR) {
+            static_assert(!ATR || Cfg::TM == 2, "two A fragments");
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]));
         }
     }
 
@@ -310,6 +329,7 @@ struct TileMainloop {
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int ks = 0; ks < Cfg::KSUB; ++ks) {
+                frag_fence(a);
                 v8i an[Cfg::TM];
 #pragma unroll
                 for (int tn = 0; tn < Cfg::TN; ++tn) {
@@ -317,8 +337,10 @@ struct TileMainloop {
                     if (tn + 1 < Cfg::TN) {
                         bnext = frag(s, frag_b[tn + 1], ks);
                     } else if (ks + 1 < Cfg::KSUB) {
+                        if (!ATR) {
 #pragma unroll
-                        for (int t = 0; t < Cfg::TM; ++t) an[t] = frag_a_at(s, t, ks + 1);
+                            for (int t = 0; t < Cfg::TM; ++t) an[t] = frag_a_at(s, t, ks + 1);
+                        }
                         bnext = frag(s, frag_b[0], ks + 1);
                     } else {
                         sync();
@@ -337,6 +359,14 @@ struct TileMainloop {
                         const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                         acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                             a[tm], bcur, (FIRST && ks == 0) ? zero : acc[tm][tn], AFMT & 1, BFMT & 1, 0, 0, 0, 0);
+                    }
+                    // Transposing reads (twice as many instructions) of the next sub-step's A fragments: one
+                    // fragment per group from the first on, issued behind the group's MFMAs and after its B
+                    // read, so that the next group waits for that B fragment only (LDS reads return in order).
+                    if (ATR && ks + 1 < Cfg::KSUB) {
+#pragma unroll
+                        for (int t = 0; t < Cfg::TM; ++t)
+                            if (tn == (t < Cfg::TN - 1 ? t : Cfg::TN - 1)) an[t] = frag_a_at(s, t, ks + 1);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     bcur = bnext;
