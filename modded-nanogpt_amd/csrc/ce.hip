@@ -15,6 +15,7 @@
 #include "epilogues.h"
 #include "host_util.h"
 #include "launch.h"
+#include "panel.h"
 
 namespace ngpt {
 
@@ -424,14 +425,6 @@ __global__ void ce_rowf_kernel(const float* __restrict__ lse, CandArgs ca, Softc
 // LDS to the MFMA registers (FMT_TRANSPOSED); its output rows come out in dw_pos order, which its
 // epilogue undoes (AccCoords::perm).
 //
-// token tt of a k-step (0..127) sits at byte dw_pos(tt) of the row
-__host__ __device__ inline int dw_pos(int tt) { return (tt & ~31) | (((tt >> 2) & 1) << 4) | (((tt >> 3) & 3) << 2) | (tt & 3); }
-__host__ __device__ inline int dw_pos_inv(int p) { return (p & ~31) | (((p >> 2) & 3) << 3) | (((p >> 4) & 1) << 2) | (p & 3); }
-
-__host__ __device__ inline int64_t panel_offset(int row, int kbyte, int nk /* k-steps per row */) {
-    return ((int64_t)(row >> 8) * nk + (kbyte >> 7)) * kPanelBytes + (row & 255) * 128;
-}
-
 // Epilogue of the backward's logits recompute (A = x chunk, rows = tokens; B = W, rows = vocabulary):
 // dl = e5m2_sat(rowf[token] * D(logit)) written to the panel.  Rows past Mc get rowf = 0, i.e. zero codes,
 // so the token padding of the panel contracts to nothing.
@@ -535,49 +528,6 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
     }
 }
 
-// Panel-blocked transpose of a row-major fp8 matrix: out row = input column c (c < cols), contraction =
-// input rows [row0, row0 + nrows) padded with zeros to nk * 128, contraction bytes of each k-step
-// permuted by PERM (0 none, 2 dw_pos).  One workgroup moves a 128 (rows) x 64 (columns) tile.
-template <int PERM>
-__global__ __launch_bounds__(256) void panel_transpose_kernel(const uint8_t* __restrict__ in, int64_t ld, int row0, int nrows, int cols,
-                                                              int nk, uint8_t* __restrict__ out) {
-    __shared__ __attribute__((aligned(16))) uint8_t tile[128][80];
-    const int kt = blockIdx.x, cg = blockIdx.y, tid = threadIdx.x;
-    for (int i = tid; i < 512; i += 256) {
-        int r = i >> 2, ch = i & 3;
-        int gr = kt * 128 + r;
-        v4i v = {0, 0, 0, 0};
-        if (gr < nrows && cg * 64 + ch * 16 < cols) v = *(const v4i*)(in + (int64_t)(row0 + gr) * ld + cg * 64 + ch * 16);
-        *(v4i*)&tile[r][ch * 16] = v;
-    }
-    __syncthreads();
-    const int o = tid >> 2, part = tid & 3;
-    const int c = cg * 64 + o;
-    if (c >= cols) return;
-    uint32_t w[8];
-#pragma unroll
-    for (int d = 0; d < 8; ++d) {
-        uint32_t word = 0;
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            int p = part * 32 + d * 4 + b;
-            int t = PERM == 2 ? dw_pos_inv(p) : p;
-            word |= (uint32_t)tile[t][o] << (8 * b);
-        }
-        w[d] = word;
-    }
-    uint8_t* dst = out + panel_offset(c, kt * 128, nk) + part * 32;
-    *(v4i*)dst = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-    *(v4i*)(dst + 16) = (v4i){(int)w[4], (int)w[5], (int)w[6], (int)w[7]};
-}
-
-template <int PERM>
-static int panel_transpose(const uint8_t* in, int64_t ld, int row0, int nrows, int cols, int nk, uint8_t* out, hipStream_t st) {
-    if (cols % 16 || ld % 16) return fail(NGPT_EALIGN, "panel_transpose: cols=%d ld=%lld", cols, (long long)ld);
-    dim3 grid(nk, (cols + 63) / 64);
-    panel_transpose_kernel<PERM><<<grid, 256, 0, st>>>(in, ld, row0, nrows, cols, nk, out);
-    return check_launch("panel_transpose_kernel");
-}
 
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
                float scale, void* out, int64_t ldc, int out_kind, hipStream_t st, int splits);
@@ -825,7 +775,7 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         // 3. dx[pass] = dl [Mc, V] . (W^T [K, V])^T, dl read transposed from the panel
         {
             GemmSlot slot(PROF_CE_DX);
-            if (int e = gemm_balanced_bf16(dw_panel, FMT_E5M2 | FMT_TRANSPOSED, 0, w_t, FMT_E4M3, 0, kBlockedB, Mc, K, V, grad_s * w_s,
+            if (int e = gemm_balanced_bf16(dw_panel, FMT_E5M2 | FMT_TRANSPOSED, 0, w_t, FMT_E4M3, 0, kBlockedB | kRowsPermuted, Mc, K, V, grad_s * w_s,
                                            (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, dx32, Mt, st)) return e;
         }
         // 4. dw (+)= dl^T . x over the tokens of the pass (zero padded to Mt)

@@ -95,6 +95,28 @@ __device__ __forceinline__ uint32_t f32_to_e4m3_sat(float v) {
     return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v, v, 0, false) & 0xffu;
 }
 
+// fp8(bf16_rne(fp32(x) / s)): the division is IEEE fp32 and is rounded to bf16 before the cast.
+template <int FMT>
+__device__ __forceinline__ uint32_t quant_one(uint32_t bf16_bits, float s) {
+    float q = round_to_bf16(__fdiv_rn(bf16_bits_to_f32(bf16_bits), s));
+    return FMT == FMT_E4M3 ? f32_to_e4m3_torch(q) : f32_to_e5m2_torch(q);
+}
+
+template <int FMT>
+__device__ __forceinline__ v2i quant8(v4i in, float s) {
+    uint32_t w[4] = {(uint32_t)in.x, (uint32_t)in.y, (uint32_t)in.z, (uint32_t)in.w};
+    uint32_t c[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        c[2 * i] = quant_one<FMT>(w[i] & 0xffffu, s);
+        c[2 * i + 1] = quant_one<FMT>(w[i] >> 16, s);
+    }
+    v2i o;
+    o.x = (int)(c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24));
+    o.y = (int)(c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24));
+    return o;
+}
+
 // ---------------------------------------------------------------- wave helpers
 __device__ __forceinline__ int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
 

@@ -3,6 +3,7 @@
 #include "epilogues.h"
 #include "host_util.h"
 #include "launch.h"
+#include "panel.h"
 #include <mutex>
 #include <vector>
 
@@ -277,11 +278,16 @@ extern "C" int ngpt_mm_fwd(const void* x_bf16, const void* w_bf16, int M, int N,
 }
 
 // ------------------------------------------------------------------------------------------ mm backward
-// workspace: g_f8 [M,N] | g_f8^T [N,M] | x_f8^T [K,M] | (OUT_IN only) w_f8^T [K,N]
+// The incoming gradient is quantised ONCE, into a panel-blocked e5m2 matrix with rows = N and 128-byte
+// rows = 128 consecutive rows of g (tokens): dW = x^T . g consumes it directly as its B operand, dx = g . w
+// reads it as the transpose of its A operand (transposed on the way from LDS to the MFMA registers).
+// Both GEMMs use the balanced walk.
+// workspace: g^T panel [Np, Mt] | x_f8^T panel [Kp, Mt] | w^T panel [Kp, N] | dx fp32 [M, K]   (p / t = rounded up to 256)
+static int64_t round256(int64_t n) { return (n + 255) / 256 * 256; }
 extern "C" int64_t ngpt_mm_bwd_workspace_bytes(int M, int N, int K, int w_layout) {
-    int64_t b = 2 * align_up((int64_t)M * N, 256) + align_up((int64_t)K * M, 256);
-    if (w_layout == NGPT_W_OUT_IN) b += align_up((int64_t)K * N, 256);
-    return b;
+    (void)w_layout;
+    const int64_t Mt = round256(M), Np = round256(N), Kp = round256(K);
+    return Np * Mt + Kp * Mt + Kp * (int64_t)N + align_up((int64_t)M * K * 4, 256);
 }
 
 extern "C" int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f8, int M, int N, int K,
@@ -296,22 +302,26 @@ extern "C" int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f
     if (workspace_bytes < need)
         return fail(NGPT_EWORKSPACE, "ngpt_mm_bwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
     hipStream_t st = (hipStream_t)stream;
+    const int64_t Mt = round256(M), Np = round256(N), Kp = round256(K);
+    const int nkt = (int)(Mt / 128), nkn = N / 128;
     uint8_t* ws = (uint8_t*)workspace;
-    uint8_t* g_f8 = ws;
-    uint8_t* g_f8_t = g_f8 + align_up((int64_t)M * N, 256);
-    uint8_t* x_f8_t = g_f8_t + align_up((int64_t)M * N, 256);
-    uint8_t* w_f8_t = x_f8_t + align_up((int64_t)K * M, 256);
-    if (int e = ngpt_quant_fp8_2d(g_bf16, M, N, grad_s, NGPT_FMT_E5M2, g_f8, g_f8_t, stream)) return e;
-    if (int e = ngpt_transpose_u8(x_f8, M, K, x_f8_t, stream)) return e;
-    const void* w_kn = w_f8;
-    if (w_layout == NGPT_W_OUT_IN) {
-        if (int e = ngpt_transpose_u8(w_f8, N, K, w_f8_t, stream)) return e;
-        w_kn = w_f8_t;
+    uint8_t* g_panel = ws;
+    uint8_t* x_t = g_panel + Np * Mt;
+    uint8_t* w_t = x_t + Kp * Mt;
+    float* dx32 = (float*)(w_t + Kp * (int64_t)N);
+    if (int e = (panel_transpose<0, FMT_E5M2>(g_bf16, N, 0, M, N, nkt, g_panel, st, grad_s))) return e;
+    if (int e = panel_transpose<0>(x_f8, K, 0, M, K, nkt, x_t, st)) return e;
+    if (w_layout == NGPT_W_OUT_IN) {   // w [N, K]  ->  rows = K, contraction = N
+        if (int e = panel_transpose<0>(w_f8, K, 0, N, K, nkn, w_t, st)) return e;
+    } else {                           // w [K, N] already has the contraction contiguous
+        if (int e = panel_pack(w_f8, N, K, N, w_t, st)) return e;
     }
-    // dx [M,K] = g_f8 [M,N] . (w [K,N])^T, contraction over N
-    if (int e = gemm_store(g_f8, FMT_E5M2, N, w_kn, FMT_E4M3, N, M, K, N, grad_s * w_s, dx_bf16, K, 0, st, 1)) return e;
-    // dw [K,N] = x_f8^T [K,M] . (g_f8^T [N,M])^T, contraction over M
-    return gemm_store(x_f8_t, FMT_E4M3, M, g_f8_t, FMT_E5M2, M, K, N, M, x_s * grad_s, dw_kn_f32, N, 1, st, 1);
+    // dx [M,K] = g [M,N] . (w^T [K,N])^T, contraction over N, g read transposed from the panel
+    if (int e = gemm_balanced_bf16(g_panel, FMT_E5M2 | FMT_TRANSPOSED, 0, w_t, FMT_E4M3, 0, kBlockedB, M, K, N, grad_s * w_s,
+                                   dx_bf16, K, dx32, (int)Mt, st)) return e;
+    // dw [K,N] = x_f8^T [K,Mt] . (g^T [N,Mt])^T, contraction over the (zero padded) rows of g
+    return gemm_balanced_f32(x_t, FMT_E4M3, 0, g_panel, FMT_E5M2, 0, kBlockedA | kBlockedB, K, N, (int)Mt, x_s * grad_s,
+                             (float*)dw_kn_f32, N, false, st);
 }
 
 // ------------------------------------------------------------------------------------------ dpre (bf16)

@@ -36,7 +36,9 @@ namespace ngpt {
 // the A matrix -- rows = the contraction index of this GEMM, 128-byte k-step rows = 128 rows of this
 // GEMM's output, blocks [contraction / 256][R / 128] -- and `a_rows_pad` is R rounded up to 256.  One
 // k-step of a tile then reads two contiguous 16 KiB pieces (128 contraction rows x 128 output rows each).
-constexpr int kBlockedA = 1, kBlockedB = 2;
+// kRowsPermuted: the 128-byte rows of a transposed A panel hold the output rows of every 32-group in dw_pos
+// order (panel.h); the epilogue's row arithmetic undoes it (AccCoords::perm).
+constexpr int kBlockedA = 1, kBlockedB = 2, kRowsPermuted = 4;
 constexpr int kPanelRows = 256, kPanelBytes = kPanelRows * 128;
 
 struct GemmOperands {
@@ -46,7 +48,7 @@ struct GemmOperands {
     int R, C, K;        // K % 128 == 0
     int splits;         // split-K: the contraction of a split tile is cut into this many jobs (>= 1); needs an accumulating epilogue if > 1
     int ablate;         // timing aid: bit 0 = issue no operand loads after the first, bit 1 = no MFMA work, bit 2 = no k-loop barrier
-    int layout;         // kBlockedA | kBlockedB
+    int layout;         // kBlockedA | kBlockedB | kRowsPermuted
     int full_tiles;     // the first full_tiles tiles (in walk order) are never split; 0 = `splits` applies to every tile
     int a_rows_pad;     // transposed A only: R rounded up to 256
 };
@@ -526,7 +528,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     ml.init();
     const int bid = blockIdx.x, G = gridDim.x;
     const int nk = g.K / Cfg::BK;
-    AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane, (AFMT & FMT_TRANSPOSED) != 0);
+    AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane, (g.layout & kRowsPermuted) != 0);
     Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
 
     // `pre` walks the (job, k-step) sequence of this workgroup ahead of the MFMAs; `ahead` counts the

@@ -135,3 +135,36 @@ def test_config2_mlp_forward_full_size(amd, oracle):
     assert _rel(post.cpu()[rows], post_ref) <= GEMM_TOL
     out_ref = (post_ref.float() @ w_proj_t.float()).bfloat16()
     assert _rel(out.cpu()[0, rows], out_ref) <= GEMM_TOL
+
+
+@pytest.mark.parametrize("layout", ["out_in", "in_out"])
+def test_mm_forward_backward_lm_head_shape(amd, oracle, layout):
+    """nanogpt::mm / mm_t forward + backward at an lm_head-sized problem (N = 50304): row / column subsets
+    against the oracle's quantise-dequantise-matmul restatement."""
+    g = torch.Generator().manual_seed(11)
+    M, N, K = 8192, 50304, 768
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    grad = (torch.randn(M, N, generator=g) * 1e-3).bfloat16()
+    x_s, w_s, grad_s = 100 / 448, 1.6 / 448, 0.75 / 448 * 1e-2
+    d = "cuda"
+    if layout == "out_in":
+        out, x_f8, w_f8 = torch.ops.nanogpt.mm(x.to(d), w.to(d), x_s, w_s, grad_s)
+        dx, dw = torch.ops.nanogpt.mm_backward(grad.to(d), x_f8, w_f8, x_s, w_s, grad_s)
+        dw_nk = dw                                   # [N, K] (a transposed view of the [K, N] result)
+    else:
+        out, x_f8, w_f8 = torch.ops.nanogpt.mm_t(x.to(d), w.T.contiguous().to(d), x_s, w_s, grad_s)
+        dx, dw = torch.ops.nanogpt.mm_t_backward(grad.to(d), x_f8, w_f8, x_s, w_s, grad_s)
+        dw_nk = dw.T                                 # [K, N] -> [N, K]
+    torch.cuda.synchronize()
+    xq, wq = oracle.quant_e4m3(x, x_s).float(), oracle.quant_e4m3(w, w_s).float()
+    rows = torch.cat([torch.arange(0, M, 509), torch.arange(M - 8, M)]).unique()
+    cols = torch.cat([torch.arange(0, N, 3001), torch.arange(N - 8, N)]).unique()
+    out_ref = ((xq[rows] @ wq.T) * (x_s * w_s)).bfloat16()
+    assert _rel(out.cpu()[rows], out_ref) <= GEMM_TOL
+    gq_rows = oracle.quant_e5m2(grad[rows], grad_s).float()
+    dx_ref = ((gq_rows @ wq) * (grad_s * w_s)).bfloat16()
+    assert _rel(dx.cpu()[rows], dx_ref) <= GEMM_TOL
+    gq_cols = oracle.quant_e5m2(grad[:, cols].contiguous(), grad_s).float()
+    dw_ref = (gq_cols.T @ xq) * (x_s * grad_s)
+    assert _rel(dw_nk.cpu()[cols], dw_ref) <= GEMM_TOL
