@@ -68,8 +68,82 @@ def cpu_baseline(oracle, x, w, t, sc, budget_s=20.0):
     }
 
 
+def secondary(args, amd, oracle) -> int:
+    """Other workloads of the path, same JSON shape; timed with events on the current stream."""
+    import math
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    wl = args.workload
+    if wl == "mm_cfg1":
+        x, w, x_s, w_s = oracle.make_cfg1(seed=0)
+        xd, wd = x.to(dev), w.to(dev)
+        step = lambda: torch.ops.nanogpt.mm(xd, wd, x_s, w_s, 1.0)
+        flops, desc, tokens = 2.0 * x.shape[0] * w.shape[0] * x.shape[1], "config 1: nanogpt::mm forward, M=1024 N=3072 K=768", x.shape[0]
+    elif wl == "mm_lmhead":
+        Mm, Nn, Kk = 16384, 50304, 768
+        xd = torch.randn(Mm, Kk, generator=g).bfloat16().to(dev)
+        wd = (torch.randn(Nn, Kk, generator=g) / math.sqrt(Kk)).bfloat16().to(dev)
+        gd = (torch.randn(Mm, Nn, generator=g) * 1e-3).bfloat16().to(dev)
+        x_s, w_s, grad_s = 100 / 448, 1.6 / 448, 0.75 / 448 * 1e-2
+
+        def step():
+            out, x_f8, w_f8 = torch.ops.nanogpt.mm(xd, wd, x_s, w_s, grad_s)
+            return torch.ops.nanogpt.mm_backward(gd, x_f8, w_f8, x_s, w_s, grad_s)
+        flops, desc, tokens = 6.0 * Mm * Nn * Kk, "nanogpt::mm forward + mm_backward at the lm_head shape, M=16384 N=50304 K=768", Mm
+    elif wl in ("mlp_fwd", "mlp_fwd_bwd"):
+        Mm, D, H = 49152, 768, 3072
+        xr = (torch.randn(Mm, D, generator=g) * 2).bfloat16().to(dev)
+        w_fc = (torch.randn(H, D, generator=g) / math.sqrt(D)).bfloat16().to(dev)
+        w_pt = (torch.randn(D, H, generator=g) / math.sqrt(H)).bfloat16().T.contiguous().to(dev)
+        dy = (torch.randn(1, Mm, D, generator=g) * 1e-3).bfloat16().to(dev)
+        w_f8, scales = torch.ops.nanogpt.quant_up_weights(w_fc[None])
+        bwd = wl == "mlp_fwd_bwd"
+        if bwd:
+            xr.requires_grad_(True); w_fc.requires_grad_(True); w_pt.requires_grad_(True)
+
+        def step():
+            normed, x_f8, dequant = torch.ops.nanogpt.mlp_input_quant(xr, scales[0:1])
+            out = amd.ReLUSqrdMLP(normed[None], w_fc, w_pt, w_f8[0], dequant, x_f8[None])
+            if bwd:
+                xr.grad = w_fc.grad = w_pt.grad = None
+                out.backward(dy)
+            return out
+        flops = (12.0 if bwd else 4.0) * Mm * D * H
+        desc = ("config 4 (one layer): " if bwd else "config 2: ") + "norm + quantise + FP8 c_fc with ReLU^2 + bf16 c_proj" + \
+               (", forward+backward" if bwd else ", forward") + ", M=49152 D=768 H=3072"
+        tokens = Mm
+    else:
+        print(f"bench.py: unknown workload {wl}", file=sys.stderr)
+        return 2
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = dt / args.steps * 1e3
+    tflops = flops / (ms * 1e-3) / 1e12
+    peak = PEAK_FP8_TFLOPS
+    print(json.dumps({
+        "metric": "tokens/s (secondary workload of the FP8 path)", "value": tokens / (ms * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp8", "data": "synthetic", "config": {"workload": desc},
+        "tflops": tflops, "event_ms_per_step": e0.elapsed_time(e1) / args.steps,
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak, "traffic": None,
+                     "note": "whole step against the dense FP8 peak; bf16 GEMMs inside count at the same peak"},
+    }))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--workload", default="lmhead_ce",
+                    help="lmhead_ce (default, the headline configuration 3) | mm_cfg1 | mm_lmhead | mlp_fwd | mlp_fwd_bwd")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
@@ -89,6 +163,8 @@ def main() -> int:
 
     lib = amd._lib.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.workload != "lmhead_ce":
+        return secondary(args, amd, oracle)
     dev = torch.device("cuda:0")
     x, w, t, sc = oracle.make_cfg3(seed=0)
     xd, wd, td = x.to(dev), w.to(dev), t.to(dev)

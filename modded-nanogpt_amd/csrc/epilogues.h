@@ -152,13 +152,18 @@ struct EpiStoreBf16 {
     }
 };
 
-// dpre[r, c] = bf16(2 * bf16(acc) * sqrt(post[r, c])): the backward of relu(pre)^2 through the down
-// projection, with relu(pre) recovered as sqrt(post) (linear_relu_square_kernel, FORWARD = False).
+// dpre = bf16(2 * bf16(acc) * sqrt(post)): the backward of relu(pre)^2 through the down projection, with
+// relu(pre) recovered as sqrt(post) (linear_relu_square_kernel, FORWARD = False).
+// The GEMM runs TRANSPOSED: tile rows = hidden units (A = W2), tile columns = tokens (B = dY), while post
+// and dpre are [tokens, hidden] row-major.  A lane then owns one token and, per accumulator register
+// group, four consecutive hidden units, i.e. 8 contiguous bytes of post / dpre: 32 wide loads and stores
+// per wave tile instead of 128 two-byte ones.  All loads are issued before the first store (the memory
+// counter retires in issue order: a load behind a store would wait for it to reach memory).
 struct EpiDpre {
-    uint16_t* out;
-    const uint16_t* post;
+    uint16_t* out;          // dpre [C = tokens, R = hidden], row stride ld
+    const uint16_t* post;   // same shape
     int64_t ld;
-    int R, C;
+    int R, C;               // R % 4 == 0
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
@@ -172,29 +177,39 @@ struct EpiDpre {
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t*, int) {
-        const int64_t tile_off = (int64_t)r0 * ld + c0;
+        const int64_t tile_off = (int64_t)c0 * ld + r0;
         uint16_t* origin = out + tile_off;
         const uint16_t* porigin = post + tile_off;
-        const uint32_t lane_off = (uint32_t)co.row_base * (uint32_t)ld + (uint32_t)co.col_base;
+        const uint32_t lane_off = (uint32_t)co.col_base * (uint32_t)ld + (uint32_t)co.row_base;
         const int rlim = R - r0 - co.row_base, clim = C - c0 - co.col_base;
         const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
+        v2i pp[Cfg::TM][Cfg::TN][4];
+#pragma unroll
+        for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < Cfg::TN; ++tn)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const int dr = tm * 32 + 8 * a, dc = tn * 32;
+                    const bool ok = full || (dr < rlim && dc < clim);
+                    pp[tm][tn][a] = ok ? *(const v2i*)(porigin + ((int64_t)dc * ld + dr) + lane_off) : (v2i){0, 0};
+                }
 #pragma unroll
         for (int tm = 0; tm < Cfg::TM; ++tm)
 #pragma unroll
             for (int tn = 0; tn < Cfg::TN; ++tn) {
 #pragma unroll
-                for (int v = 0; v < 16; v += 2) {
-                    const int dr = tm * 32 + 8 * (v >> 2) + (v & 3), dc = tn * 32;
-                    const int64_t uo = (int64_t)dr * ld + dc;
-                    const bool ok0 = full || (dr < rlim && dc < clim), ok1 = full || (dr + 1 < rlim && dc < clim);
-                    float p0 = ok0 ? bf16_bits_to_f32(porigin[uo + lane_off]) : 0.0f;
-                    float p1 = ok1 ? bf16_bits_to_f32(porigin[uo + lane_off + (uint32_t)ld]) : 0.0f;
-                    uint32_t c01 = cvt_pk_bf16(acc[tm][tn][v], acc[tm][tn][v + 1]);        // c = bf16(acc)
-                    float d0 = 2.0f * bf16_bits_to_f32(c01 & 0xffffu) * __fsqrt_rn(p0);
-                    float d1 = 2.0f * bf16_bits_to_f32(c01 >> 16) * __fsqrt_rn(p1);
-                    uint32_t pk = cvt_pk_bf16(d0, d1);
-                    if (ok0) origin[uo + lane_off] = (uint16_t)pk;
-                    if (ok1) origin[uo + lane_off + (uint32_t)ld] = (uint16_t)(pk >> 16);
+                for (int a = 0; a < 4; ++a) {
+                    const int dr = tm * 32 + 8 * a, dc = tn * 32;
+                    const bool ok = full || (dr < rlim && dc < clim);
+                    const uint32_t p01 = (uint32_t)pp[tm][tn][a].x, p23 = (uint32_t)pp[tm][tn][a].y;
+                    const v16f& c = acc[tm][tn];
+                    uint32_t c01 = cvt_pk_bf16(c[4 * a], c[4 * a + 1]), c23 = cvt_pk_bf16(c[4 * a + 2], c[4 * a + 3]);   // bf16(acc)
+                    float d0 = 2.0f * bf16_bits_to_f32(c01 & 0xffffu) * __fsqrt_rn(bf16_bits_to_f32(p01 & 0xffffu));
+                    float d1 = 2.0f * bf16_bits_to_f32(c01 >> 16) * __fsqrt_rn(bf16_bits_to_f32(p01 >> 16));
+                    float d2 = 2.0f * bf16_bits_to_f32(c23 & 0xffffu) * __fsqrt_rn(bf16_bits_to_f32(p23 & 0xffffu));
+                    float d3 = 2.0f * bf16_bits_to_f32(c23 >> 16) * __fsqrt_rn(bf16_bits_to_f32(p23 >> 16));
+                    if (ok) *(v2i*)(origin + ((int64_t)dc * ld + dr) + lane_off) = (v2i){(int)cvt_pk_bf16(d0, d1), (int)cvt_pk_bf16(d2, d3)};
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
