@@ -1,13 +1,14 @@
 // Persistent FP8 "TN" GEMM core for gfx950:  C[r, c] = sum_k A[r, k] * B[c, k]
 //
-// Both operands are fp8 bytes with the contraction index contiguous.  One workgroup owns a
-// BM x BN tile at a time and walks a list of tiles; the k-loop of consecutive tiles is one
-// continuous software pipeline, so the first operand slab of the next tile is already in flight
-// while the current tile's epilogue runs.
+// Both operands are fp8 bytes (or bf16 pairs, FMT_BF16) with the contraction index contiguous.  One
+// workgroup owns a BM x BN tile at a time and walks a list of jobs (tiles, or contraction ranges of
+// tiles); the k-loop of consecutive jobs is one continuous software pipeline: operand loads run two
+// k-steps ahead of the MFMAs, across job boundaries and epilogues.
 //
 // Data path per k-step (BK = 128 bytes of contraction):
-//   HBM/L2 --global_load_lds_dwordx4--> LDS (two stages, no register staging)
+//   HBM/L2 --global_load_lds_dwordx4--> LDS (two 64 KiB slots, no register staging)
 //   LDS --ds_read_b128--> MFMA operand registers --v_mfma_f32_32x32x64_f8f6f4--> fp32 accumulators
+// (A operand given as the panel of its transpose, FMT_TRANSPOSED: LDS --ds_read_b64_tr_b8--> registers.)
 //
 // LDS layout of an operand slab: rows of 128 bytes; the eight 16-byte chunks of row r are stored
 // at chunk position q ^ ((r >> 1) & 7).  A direct-to-LDS load writes 1 KiB (8 rows) per wave
