@@ -165,6 +165,8 @@ struct TileMainloop {
     int frag_a[Cfg::TM];     // LDS byte offset of this lane's first 16-byte chunk, stage 0, ksub 0
     int frag_b[Cfg::TN];
     int a_step, b_step;      // bytes from one k-step's slab to the next
+    const uint8_t* b_pending;   // B slab whose loads issue_loads_b() still has to issue, or null
+    int pending_stage;
     int a_kt;                // transposed A: index of the next k-step to load; a_next then is the tile's base
     int64_t a_pair_stride;   // transposed A: bytes between the panel rows of two consecutive 256-blocks of the contraction
     int wave, lane, wr, wc;
@@ -173,6 +175,8 @@ struct TileMainloop {
     __device__ void init() {
         int tid = threadIdx.x;
         lane = tid & 63;
+        b_pending = nullptr;
+        pending_stage = 0;
         wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         wr = wave / Cfg::WAVES_N;
         wc = wave % Cfg::WAVES_N;
@@ -206,6 +210,7 @@ struct TileMainloop {
     // Point the loads at tile (r0, c0).  Rows past the end are clamped to the last row: they are
     // loaded (valid memory) and their results discarded by the epilogue.
     // `kt`: first k-step that will be loaded from this tile.
+    // (The caller flushes issue_loads_b() first: the pending B loads use the old tile's lane offsets.)
     __device__ void set_tile(const GemmOperands& g, int r0, int c0, int kt) {
         a_step = (g.layout & kBlockedA) ? kPanelBytes : Cfg::BK;
         b_step = (g.layout & kBlockedB) ? kPanelBytes : Cfg::BK;
@@ -221,11 +226,14 @@ struct TileMainloop {
         lo.init(g, wave, lane, r0, c0, ATR);
     }
 
-    // Loads the next k-step of the current tile into LDS slot `stage` and moves on to the one after.
+    // Loads the next k-step of the current tile into LDS slot `stage` and moves on to the one after: the A
+    // slab now, the B slab when issue_loads_b() is called (behind the next k-step's first MFMAs, so that the
+    // loads of one k-step do not leave the compute unit in a single burst).
     __device__ void issue_loads(uint8_t* smem, int stage) {
         uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
         const uint8_t* ab = a_next;
-        const uint8_t* bb = b_next;
+        b_pending = b_next;
+        pending_stage = stage;
         if (ATR) {   // contraction rows 128 * a_kt ..+127: block a_kt / 2, upper or lower half of its 256 rows
             ab = a_next + (int64_t)(a_kt >> 1) * a_pair_stride + (a_kt & 1) * (kPanelBytes / 2);
             ++a_kt;
@@ -236,9 +244,14 @@ struct TileMainloop {
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i)
             global_to_lds16(ab + lo.a_off[i], s + (wave + i * Cfg::NWAVES) * 1024);
+    }
+    __device__ void issue_loads_b(uint8_t* smem) {
+        if (b_pending == nullptr) return;
+        uint8_t* s = smem + pending_stage * Cfg::STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < Cfg::B_LOADS; ++i)
-            global_to_lds16(bb + lo.b_off[i], s + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
+            global_to_lds16(b_pending + lo.b_off[i], s + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
+        b_pending = nullptr;
     }
 
     // Operand fragment of one 32-row MFMA tile for contraction sub-step ks (two 16-byte chunks).
@@ -295,7 +308,7 @@ struct TileMainloop {
     //    `refill` (issue of the operand loads two k-steps ahead into the slot just freed) runs behind the
     //    last group's MFMAs, so that its address arithmetic is hidden too.
     template <bool FIRST, class Sync, class Refill>
-    __device__ __forceinline__ void compute(const uint8_t* smem, int stage, int next_stage, bool have, bool want_next,
+    __device__ __forceinline__ void compute(uint8_t* smem, int stage, int next_stage, bool have, bool want_next,
                                             v16f (&acc)[Cfg::TM][Cfg::TN], v8i (&a)[Cfg::TM], v8i& b0, Sync&& sync,
                                             Refill&& refill) {
         const uint8_t* s = smem + stage * Cfg::STAGE_BYTES;
@@ -304,6 +317,7 @@ struct TileMainloop {
             // bf16 operands: 32 contraction bytes (16 elements) per MFMA, one 16-byte chunk per lane;
             // no fragment hand-over between k-steps
             constexpr int KS = Cfg::BK / 32;
+            issue_loads_b(smem);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 v8bf fa[Cfg::TM], fb[Cfg::TN];
@@ -363,6 +377,7 @@ struct TileMainloop {
                         acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                             a[tm], bcur, (FIRST && ks == 0) ? zero : acc[tm][tn], AFMT & 1, BFMT & 1, 0, 0, 0, 0);
                     }
+                    if (ks == 0 && tn == 0) issue_loads_b(smem);   // second half of the loads issued at the end of the previous k-step
                     // Transposing reads (twice as many instructions) of the next sub-step's A fragments: one
                     // fragment per group from the first on, issued behind the group's MFMAs and after its B
                     // read, so that the next group waits for that B fragment only (LDS reads return in order).
@@ -540,6 +555,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         if (pre.valid()) {
             if (pre.at_job_start()) {
                 asm volatile("; new tile" ::: "memory");   // rare: keep it a branch, out of the k-loop's straight path
+                ml.issue_loads_b(smem);
                 ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN, pre.kt);
             }
             if (!(ablate & 1) || ahead == 0) ml.issue_loads(smem, into_slot);
@@ -548,7 +564,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         }
     };
     refill(0);
+    ml.issue_loads_b(smem);
     refill(1);
+    ml.issue_loads_b(smem);
     epi.begin(bid, G, smem_all);
     // operands of the first k-step
     if (ahead == 2) wait_vmem_le<Cfg::LOADS>();
@@ -591,10 +609,14 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
             };
             auto refill_here = [&]() {
                 if (!(last_kt && keep_slot)) refill(slot);
+                // before an epilogue both halves go out at once: the relaxed wait of the next job's first
+                // k-step counts on every operand load having been issued before the epilogue's stores
+                if (last_kt) ml.issue_loads_b(smem);
             };
             if (!(ablate & 2)) {
                 ml.template compute<decltype(first)::value>(smem, slot, slot ^ 1, have, more, acc, fa, fb, sync, refill_here);
             } else {
+                ml.issue_loads_b(smem);
                 sync();
                 refill_here();
             }
@@ -618,6 +640,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         if (keep_slot) {
             wg_barrier();          // all waves are done with the scratch
             refill(slot ^ 1);
+            ml.issue_loads_b(smem);
         }
         cur.advance();
     }
