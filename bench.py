@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload: BASELINE config 3 -- x bf16 [49152, 768] ~ N(0,1), W bf16 [50304, 768] ~ N(0, 1/768),
+Workload: Benchmark configuration 3 -- x bf16 [49152, 768] ~ N(0,1), W bf16 [50304, 768] ~ N(0, 1/768),
 lm_head scales x_s = 100/448, w_s = 1.6/448, grad_s = 0.75/448, int64 targets uniform in [0, 50257),
 outputs per-token losses, dx bf16, dW fp32.  One "step" = one forward + one backward of the path
 with all inputs already resident in HBM.  Algorithmic work per step: 6*M*K*V FLOP (three GEMMs;

@@ -1,4 +1,4 @@
-"""Full-size runs of the fused lm_head + cross-entropy (BASELINE configs 3 and 5 shapes) on the GPU.
+"""Full-size runs of the fused lm_head + cross-entropy (benchmark configurations 3 and 5) on the GPU.
 
 The CPU oracle cannot process 49152 x 50304 logits in seconds, so parity at this size is checked on what
 the problem's structure allows: rows are independent in the forward and in dx (row subsets against the

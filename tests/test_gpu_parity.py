@@ -119,7 +119,7 @@ def test_gemm_operand_orientation(amd):
 
 # ------------------------------------------------------------------------------------------ nanogpt::mm
 def test_mm_forward_config1(amd, oracle):
-    """BASELINE config 1: x [1024,768], W [3072,768], x_s=1, w_s=1/32, seed 0."""
+    """Benchmark configuration 1: x [1024,768], W [3072,768], x_s=1, w_s=1/32, seed 0."""
     x, w, x_s, w_s = oracle.make_cfg1(seed=0)
     out_ref, xf_ref, wf_ref = oracle.mm_fwd(x, w, x_s, w_s)
     out, x_f8, w_f8 = torch.ops.nanogpt.mm(dev(x), dev(w), x_s, w_s, 1.0)
