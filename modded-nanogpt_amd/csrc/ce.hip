@@ -50,8 +50,15 @@ __device__ __forceinline__ uint32_t tab_offsets2(uint32_t pk) {
     u16x2_t u = __builtin_bit_cast(u16x2_t, pk);
     u16x2_t t = __builtin_elementwise_sub_sat(u & (u16x2_t){0x7fff, 0x7fff}, (u16x2_t){TAB_LO, TAB_LO});
     t = __builtin_elementwise_min(t, (u16x2_t){TAB_N - 1, TAB_N - 1});
-    u16x2_t off = (t << (u16x2_t){2, 2}) | ((u >> (u16x2_t){1, 1}) & (u16x2_t){4 * TAB_NEG, 4 * TAB_NEG});
-    return __builtin_bit_cast(uint32_t, off);
+    // sign bits (bit 15 of each half) to the table's sign bit and merged in one instruction: written as
+    // assembly because the compiler otherwise separates the merge from the extraction of the two halves
+    // at the price of an extra instruction.  (A 32-bit shift moves bit 16 into bit 15, which the mask
+    // drops: same as shifting the halves.)
+    uint32_t off;
+    asm("v_and_or_b32 %0, %1, %2, %3"
+        : "=v"(off)
+        : "v"(pk >> 1), "s"((uint32_t)(4 * TAB_NEG) * 0x10001u), "v"(__builtin_bit_cast(uint32_t, t << (u16x2_t){2, 2})));
+    return off;
 }
 __device__ __forceinline__ float tab_at(const float* tab, uint32_t byte_off) {
     return *(const float*)((const uint8_t*)tab + byte_off);
@@ -405,11 +412,18 @@ __global__ void ce_finalize_kernel(const float* __restrict__ part, const float* 
 
 // =====================================================================================================
 // Backward, recomputing the logits.  rowf[m] = coef * S_w[m] * exp(A - lse[m]).
+// One 256-thread block per 256 rows (one token tile of the recompute kernel).  rowf is written for the
+// whole block, zero past M (zero codes in the panel's padding without any masking in the epilogue);
+// big[block] says whether any |rowf| of the block is large enough for rowf * D to leave the e5m2 range:
+// D = E * sigma * (1 - sigma) <= 1/4, so |rowf| <= 4 * 57344 needs no clamp.
 __global__ void ce_rowf_kernel(const float* __restrict__ lse, CandArgs ca, Softcap sc, float coef,
-                               float* __restrict__ rowf) {
+                               float* __restrict__ rowf, int* __restrict__ big) {
     int m = blockIdx.x * blockDim.x + threadIdx.x;
-    if (m >= ca.M) return;
-    rowf[m] = coef * (row_weight_sum(ca, m) * expf(sc.A - lse[m]));
+    float f = 0.0f;
+    if (m < ca.M) f = coef * (row_weight_sum(ca, m) * expf(sc.A - lse[m]));
+    rowf[m] = f;
+    int b = __syncthreads_or(!(fabsf(f) <= 4.0f * 57344.0f));   // NaN counts as big
+    if (threadIdx.x == 0) big[blockIdx.x] = b;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -426,8 +440,8 @@ __global__ void ce_rowf_kernel(const float* __restrict__ lse, CandArgs ca, Softc
 // epilogue undoes (AccCoords::perm).
 //
 // Epilogue of the backward's logits recompute (A = x chunk, rows = tokens; B = W, rows = vocabulary):
-// dl = e5m2_sat(rowf[token] * D(logit)) written to the panel.  Rows past Mc get rowf = 0, i.e. zero codes,
-// so the token padding of the panel contracts to nothing.
+// dl = e5m2_sat(rowf[token] * D(logit)) written to the panel.  Rows past the last one have rowf = 0, i.e. zero
+// codes, so the token padding of the panel contracts to nothing.
 struct EpiDlStore {
     static constexpr int TILE_STORES = 8;    // 16-byte panel stores per wave and tile, always
     static constexpr bool HAS_TILE_BEGIN = true;
@@ -437,12 +451,14 @@ struct EpiDlStore {
     template <class Cfg>
     __device__ void job_begin(int) {}
     const float* gtabD;
-    const float* rowf;     // already offset to the chunk's first row
+    const float* rowf;     // already offset to the chunk's first row; zero past the last row up to a multiple of 256
+    const int* big;        // per 256 rows of the chunk: some row factor may push a gradient out of the e5m2 range
     uint8_t* dw_panel;     // [Vp / 256][Mt / 128] blocks, Vp / Mt = V / Mc rounded up to 256
     int Mc, V, nkt;        // nkt = k-steps per panel row = Mt / 128
     float scale;
     float* rowf_lds;       // LDS [2][256]
     int rslot;
+    int tile_big;
 
     __device__ void partial(bool) {}
     __device__ void begin(int, int, uint8_t* extra) {
@@ -461,15 +477,20 @@ struct EpiDlStore {
     template <class Cfg>
     __device__ void tile_begin(int r0, int) {
         rslot ^= 1;
-        if ((threadIdx.x >> 6) == 0) {
-            int row = min(r0 + 4 * (int)(threadIdx.x & 63), Mc - 4);   // rows past Mc are masked in tile()
-            global_to_lds16(rowf + row, rowf_lds + rslot * 256);
-        }
+        // wave-uniform and written by an earlier kernel: read through the constant address space so that it is a
+        // scalar load, which stays out of the vector memory counter the k-loop's waits are built on
+        tile_big = ((const __attribute__((address_space(4))) int*)(uintptr_t)big)[r0 >> 8];
+        if ((threadIdx.x >> 6) == 0) global_to_lds16(rowf + r0 + 4 * (int)(threadIdx.x & 63), rowf_lds + rslot * 256);
     }
 
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t*, int lane) {
+        if (tile_big) tile_impl<Cfg, true>(acc, r0, c0, co, lane);
+        else tile_impl<Cfg, false>(acc, r0, c0, co, lane);
+    }
+    template <class Cfg, bool SAT>
+    __device__ __forceinline__ void tile_impl(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co, int lane) {
         static_assert(Cfg::BM == kPanelRows && Cfg::BN == kPanelRows && Cfg::WTM == 64 && Cfg::WTN == 128,
                       "the panel stores assume a 256 x 256 tile of 64 x 128 wave tiles");
         const int h = lane >> 5, j = lane & 31;
@@ -484,15 +505,14 @@ struct EpiDlStore {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int lrow = co.wave_row0 + tm * 32 + 8 * g + 4 * h;
-                v4f rf = *(const v4f*)(rowf_lds + rslot * 256 + lrow);
-                if (r0 + lrow + 4 > Mc) rf = (v4f){0.f, 0.f, 0.f, 0.f};
+                const v4f rf = *(const v4f*)(rowf_lds + rslot * 256 + lrow);
 #pragma unroll
                 for (int tn = 0; tn < Cfg::TN; ++tn) {
                     const v16f& a = acc[tm][tn];
                     uint32_t o01 = tab_offsets2(pack_logits(a[4 * g] * scale, a[4 * g + 1] * scale));
                     uint32_t o23 = tab_offsets2(pack_logits(a[4 * g + 2] * scale, a[4 * g + 3] * scale));
-                    pk[tn][g] = f32x4_to_e5m2_sat(rf[0] * tab_at(tab, o01 & 0xffffu), rf[1] * tab_at(tab, o01 >> 16),
-                                                  rf[2] * tab_at(tab, o23 & 0xffffu), rf[3] * tab_at(tab, o23 >> 16));
+                    pk[tn][g] = f32x4_to_e5m2_sat<SAT>(rf[0] * tab_at(tab, o01 & 0xffffu), rf[1] * tab_at(tab, o01 >> 16),
+                                                       rf[2] * tab_at(tab, o23 & 0xffffu), rf[3] * tab_at(tab, o23 >> 16));
                 }
             }
 #pragma unroll
@@ -700,12 +720,12 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
 }
 
 // ------------------------------------------------------------------------------------------------
-// backward workspace: tabE | tabD | rowf [M] | x^T panel [Kp, Mt] | W^T panel [Kp, V] | dlogits panel [Vp, Mt] |
+// backward workspace: tabE | tabD | rowf [M rounded up to 256] | big [same, one int per 256 rows used] | x^T panel [Kp, Mt] | W^T panel [Kp, V] | dlogits panel [Vp, Mt] |
 // dx fp32 [Mc, K]   (Mc = tokens per pass, Mt / Kp / Vp = Mc / K / V rounded up to 256)
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
     int64_t Mc = bwd_chunk_rows(M), Mt = round256(Mc), Kp = round256(K), Vp = round256(V);
-    return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)M * 4, 256) + Kp * Mt + Kp * (int64_t)V + Vp * Mt +
+    return align_up(2 * TAB_BYTES, 256) + 2 * round256(M) * 4 + Kp * Mt + Kp * (int64_t)V + Vp * Mt +
            align_up(Mc * K * 4, 256);
 }
 
@@ -734,7 +754,9 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     float* tabD = tabE + TAB_ENTRIES;
     ws += align_up(2 * TAB_BYTES, 256);
     float* rowf = (float*)ws;
-    ws += align_up((int64_t)M * 4, 256);
+    ws += round256(M) * 4;
+    int* big = (int*)ws;
+    ws += round256(M) * 4;
     uint8_t* x_t = ws;       // x^T panel of the pass: rows = K features, contraction = tokens (dw_pos order)
     ws += Kp * Mt_max;
     uint8_t* w_t = ws;       // W^T panel: rows = K features, contraction = vocabulary
@@ -747,7 +769,7 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     const float coef = make_coef(A, C, grad_s, grad_scale);
     CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
     ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
-    ce_rowf_kernel<<<(M + 255) / 256, 256, 0, st>>>(lse, ca, sc, coef, rowf);
+    ce_rowf_kernel<<<(M + 255) / 256, 256, 0, st>>>(lse, ca, sc, coef, rowf, big);
     if (int e = check_launch("ce_rowf_kernel")) return e;
     const int nkv = V / 128;
     if (int e = panel_transpose<0>((const uint8_t*)w_f8_vk, K, 0, V, K, nkv, w_t, st)) return e;
@@ -763,6 +785,7 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         EpiDlStore epi{};
         epi.gtabD = tabD;
         epi.rowf = rowf + m0;
+        epi.big = big + (m0 >> 8);
         epi.dw_panel = dw_panel;
         epi.Mc = Mc;
         epi.V = V;

@@ -79,12 +79,18 @@ __device__ __forceinline__ uint32_t f32x2_to_e5m2_sat(float a, float b) {
     return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false) & 0xffffu;
 }
 
+// SAT = false: the caller knows that |value| <= 57344 and saves the clamps.  The converter writes one half
+// of its destination and keeps the other: the first of the two conversions gets its own first source (dead
+// afterwards) as the "old" value -- all 32 bits are overwritten in the end -- instead of a fresh zero.
+template <bool SAT = true>
 __device__ __forceinline__ uint32_t f32x4_to_e5m2_sat(float a, float b, float c, float d) {
-    a = __builtin_fminf(__builtin_fmaxf(a, -57344.0f), 57344.0f);
-    b = __builtin_fminf(__builtin_fmaxf(b, -57344.0f), 57344.0f);
-    c = __builtin_fminf(__builtin_fmaxf(c, -57344.0f), 57344.0f);
-    d = __builtin_fminf(__builtin_fmaxf(d, -57344.0f), 57344.0f);
-    int r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+    if (SAT) {
+        a = __builtin_fminf(__builtin_fmaxf(a, -57344.0f), 57344.0f);
+        b = __builtin_fminf(__builtin_fmaxf(b, -57344.0f), 57344.0f);
+        c = __builtin_fminf(__builtin_fmaxf(c, -57344.0f), 57344.0f);
+        d = __builtin_fminf(__builtin_fmaxf(d, -57344.0f), 57344.0f);
+    }
+    int r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, __builtin_bit_cast(int, a), false);
     r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
     return (uint32_t)r;
 }

@@ -314,6 +314,28 @@ def test_fused_lmhead_ce(amd, oracle, layout, M, K, V, n_predict, prefix):
     assert_close_gemm(dw, dw_ref)
 
 
+@pytest.mark.parametrize("grad_scale", [3.0e5, 3.0e7])
+def test_fused_lmhead_ce_gradient_saturates(amd, oracle, grad_scale):
+    """Row factors large enough for the e5m2 gradient to clamp at +-57344 (the recompute kernel then takes
+    its clamping epilogue for those token tiles); M = 640 also leaves half of the last token tile as padding.
+    At 3e5 only part of the entries clamp, at 3e7 nearly all."""
+    M, K, V = 640, 256, 2432
+    x, w, t, sc, mtp, pt, pw = _fused_case(oracle, M, K, V, seed=5)
+    l_ref, ctx = oracle.lm_head_ce_fwd(x, t, mtp, pt, pw, w, sc["x_s"], sc["w_s"], sc["grad_s"], grad_scale, w_layout="out_in")
+    dx_ref, dw_ref = oracle.lm_head_ce_bwd(ctx)
+    clamped = (ctx["dl_f8"].float().abs() == 57344.0).float().mean()
+    assert clamped > (0.5 if grad_scale > 1e7 else 0.0) and (grad_scale > 1e7 or clamped < 0.5)
+    ptd = torch.full((M,), -1, dtype=torch.int64, device="cuda")
+    pwd = torch.zeros(1, device="cuda")
+    _, lse, sig, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(dev(x), dev(w), dev(t), dev(mtp), ptd, pwd,
+                                                              sc["x_s"], sc["w_s"], 23.0, 5.0, 7.5, False)
+    dx, dw = torch.ops.nanogpt.lmhead_ce_bwd(x_f8, w_f8, dev(t), dev(mtp), ptd, pwd, lse, sig, sc["x_s"], sc["w_s"],
+                                             sc["grad_s"], grad_scale, 23.0, 5.0, 7.5, False)
+    assert torch.isfinite(dx.float()).all() and torch.isfinite(dw).all()
+    assert_close_gemm(dx, dx_ref)
+    assert_close_gemm(dw, dw_ref)
+
+
 def test_fused_lmhead_ce_reduces_to_cross_entropy(amd, oracle):
     """Independent of the oracle's kernel restatement: n_predict = 1, no prefix => the closed form
     F.cross_entropy(23*sigmoid((l+5)/7.5)) on the dequantised operands."""
