@@ -309,20 +309,32 @@ struct EpiCEFwd {
         const int V = ca.V, M = ca.M;
         const float* tab = lds_table();
         if (r0 + Cfg::BM <= V) {
+            // Batches of 8 accumulator registers, software-pipelined by hand: index arithmetic of batch b, its 8
+            // table reads, then the additions of batch b - 1, whose reads have had the arithmetic of b to return.
+            // (Left to itself the scheduler sometimes waits for every pair of reads right behind their issue.)
+            constexpr int NB = Cfg::TN * Cfg::TM * 2;
+            float pv[8];
 #pragma unroll
-            for (int tn = 0; tn < Cfg::TN; ++tn)
+            for (int b = 0; b <= NB; ++b) {
+                float nv[8];
+                if (b < NB) {
+                    const v16f& a = acc[(b >> 1) % Cfg::TM][b / (2 * Cfg::TM)];
+                    uint32_t off[4];
 #pragma unroll
-                for (int tm = 0; tm < Cfg::TM; ++tm) {
-                    float s0 = 0.0f, s1 = 0.0f;
+                    for (int k = 0; k < 4; ++k)
+                        off[k] = tab_offsets2(pack_logits(a[8 * (b & 1) + 2 * k] * scale, a[8 * (b & 1) + 2 * k + 1] * scale));
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int v = 0; v < 16; v += 2) {
-                        uint32_t off = tab_offsets2(pack_logits(acc[tm][tn][v] * scale, acc[tm][tn][v + 1] * scale));
-                        s0 += tab_at(tab, off & 0xffffu);
-                        s1 += tab_at(tab, off >> 16);
+                    for (int k = 0; k < 4; ++k) {
+                        nv[2 * k] = tab_at(tab, off[k] & 0xffffu);
+                        nv[2 * k + 1] = tab_at(tab, off[k] >> 16);
                     }
-                    sum[tn] += s0 + s1;
-                    __builtin_amdgcn_sched_barrier(0);   // keep the table reads of one MFMA tile together
+                    __builtin_amdgcn_sched_barrier(0);
                 }
+                if (b > 0) sum[(b - 1) / (2 * Cfg::TM)] += ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
+#pragma unroll
+                for (int k = 0; k < 8; ++k) pv[k] = nv[k];
+            }
         } else {   // last vocabulary tile: rows past V are clamped duplicates and must not count
 #pragma unroll
             for (int tn = 0; tn < Cfg::TN; ++tn)
@@ -499,27 +511,48 @@ struct EpiDlStore {
         // row = vocabulary column of this lane, 16 bytes = 16 tokens of one (tm, h) group
         uint8_t* dw_base = dw_panel + ((int64_t)(c0 >> 8) * nkt + (r0 >> 7) + (wr >> 1)) * kPanelBytes;
         const uint32_t dw_lane = (uint32_t)((128 * wc + j) * 128 + 64 * (wr & 1) + 16 * h);
+        // Batches of 8 accumulator registers (registers 4g ..+3 of two MFMA tiles of one row block), software-
+        // pipelined by hand: index arithmetic of batch b, its 8 table reads (and the 4 row factors of a new
+        // register group), then products and e5m2 packing of batch b - 1, whose reads have had the arithmetic
+        // of b to return; the four 16-byte stores of a row block follow its last batch.
+        static_assert(Cfg::TN == 4 && Cfg::TM == 2, "batches of two column blocks");
+        constexpr int NB = Cfg::TM * 4 * 2;
+        uint32_t pk[Cfg::TN][4];
+        float pv[8], nv[8];
+        v4f prf, nrf;
 #pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm) {
-            uint32_t pk[Cfg::TN][4];
+        for (int b = 0; b <= NB; ++b) {
+            if (b < NB) {
+                const int tm = b >> 3, g = (b >> 1) & 3, tn0 = 2 * (b & 1);
+                uint32_t off[4];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int lrow = co.wave_row0 + tm * 32 + 8 * g + 4 * h;
-                const v4f rf = *(const v4f*)(rowf_lds + rslot * 256 + lrow);
+                for (int k = 0; k < 4; ++k) {
+                    const v16f& a = acc[tm][tn0 + (k >> 1)];
+                    off[k] = tab_offsets2(pack_logits(a[4 * g + 2 * (k & 1)] * scale, a[4 * g + 2 * (k & 1) + 1] * scale));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if ((b & 1) == 0) nrf = *(const v4f*)(rowf_lds + rslot * 256 + co.wave_row0 + tm * 32 + 8 * g + 4 * h);
 #pragma unroll
-                for (int tn = 0; tn < Cfg::TN; ++tn) {
-                    const v16f& a = acc[tm][tn];
-                    uint32_t o01 = tab_offsets2(pack_logits(a[4 * g] * scale, a[4 * g + 1] * scale));
-                    uint32_t o23 = tab_offsets2(pack_logits(a[4 * g + 2] * scale, a[4 * g + 3] * scale));
-                    pk[tn][g] = f32x4_to_e5m2_sat<SAT>(rf[0] * tab_at(tab, o01 & 0xffffu), rf[1] * tab_at(tab, o01 >> 16),
-                                                       rf[2] * tab_at(tab, o23 & 0xffffu), rf[3] * tab_at(tab, o23 >> 16));
+                for (int k = 0; k < 4; ++k) {
+                    nv[2 * k] = tab_at(tab, off[k] & 0xffffu);
+                    nv[2 * k + 1] = tab_at(tab, off[k] >> 16);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (b > 0) {
+                const int q = b - 1, tm = q >> 3, g = (q >> 1) & 3, tn0 = 2 * (q & 1);
+                pk[tn0][g] = f32x4_to_e5m2_sat<SAT>(prf[0] * pv[0], prf[1] * pv[1], prf[2] * pv[2], prf[3] * pv[3]);
+                pk[tn0 + 1][g] = f32x4_to_e5m2_sat<SAT>(prf[0] * pv[4], prf[1] * pv[5], prf[2] * pv[6], prf[3] * pv[7]);
+                if ((q & 7) == 7) {
+#pragma unroll
+                    for (int tn = 0; tn < Cfg::TN; ++tn)
+                        *(v4i*)(dw_base + (dw_lane + tn * 4096 + tm * 32)) =
+                            (v4i){(int)pk[tn][0], (int)pk[tn][1], (int)pk[tn][2], (int)pk[tn][3]};
                 }
             }
 #pragma unroll
-            for (int tn = 0; tn < Cfg::TN; ++tn)
-                *(v4i*)(dw_base + (dw_lane + tn * 4096 + tm * 32)) =
-                    (v4i){(int)pk[tn][0], (int)pk[tn][1], (int)pk[tn][2], (int)pk[tn][3]};
-            __builtin_amdgcn_sched_barrier(0);
+            for (int k = 0; k < 8; ++k) pv[k] = nv[k];
+            if ((b & 1) == 0) prf = nrf;
         }
     }
 };
