@@ -108,8 +108,17 @@ __device__ __forceinline__ uint32_t quant_one(uint32_t bf16_bits, float s) {
     return FMT == FMT_E4M3 ? f32_to_e4m3_torch(q) : f32_to_e5m2_torch(q);
 }
 
+// Eight values at once.  Common case, taken when no lane of the wave holds a special value: the division
+// is x * r followed by two corrections q <- RN(q + RN(x - q s) r) with r = RN(1 / s).  x * r can be more than
+// one unit in the last place off; after the first correction q is within 2^-46 of the quotient, so the second
+// remainder is exact and its correction gives the correctly rounded quotient (Markstein's theorem: q
+// faithful, r correctly rounded, significand of s not all ones, s and r normal numbers -- `fast_ok` checks
+// the last three and s > 0).  The bf16 rounding and the fp8 casts are the hardware's packed conversions
+// (round to nearest even, subnormals kept).  A quotient that overflows the fp8 format, an infinity or a
+// NaN (the corrected quotient of an infinite x is a NaN, so those are caught too) sends the whole wave
+// through the per-element path, which decides them explicitly.
 template <int FMT>
-__device__ __forceinline__ v2i quant8(v4i in, float s) {
+__device__ __forceinline__ v2i quant8_slow(v4i in, float s) {
     uint32_t w[4] = {(uint32_t)in.x, (uint32_t)in.y, (uint32_t)in.z, (uint32_t)in.w};
     uint32_t c[8];
 #pragma unroll
@@ -121,6 +130,63 @@ __device__ __forceinline__ v2i quant8(v4i in, float s) {
     o.x = (int)(c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24));
     o.y = (int)(c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24));
     return o;
+}
+
+struct QuantScale {
+    float s, r;
+    bool fast_ok;
+    __device__ explicit QuantScale(float scale) : s(scale), r(__fdiv_rn(1.0f, scale)) {
+        const uint32_t sb = __float_as_uint(scale), rb = __float_as_uint(r);
+        const uint32_t se = (sb >> 23) & 0xffu, re = (rb >> 23) & 0xffu;
+        fast_ok = (sb >> 31) == 0 && (sb & 0x7fffffu) != 0x7fffffu && se != 0 && se != 0xff && re != 0 && re != 0xff;
+    }
+};
+
+template <int FMT>
+__device__ __forceinline__ v2i quant8(v4i in, const QuantScale& qs) {
+    const uint32_t w[4] = {(uint32_t)in.x, (uint32_t)in.y, (uint32_t)in.z, (uint32_t)in.w};
+    uint32_t pk[4];      // bf16(x / s), two per word
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float x0 = __uint_as_float(w[i] << 16), x1 = __uint_as_float(w[i] & 0xffff0000u);
+        float q0 = x0 * qs.r, q1 = x1 * qs.r;
+#pragma unroll
+        for (int step = 0; step < 2; ++step) {
+            q0 = __builtin_fmaf(__builtin_fmaf(-q0, qs.s, x0), qs.r, q0);
+            q1 = __builtin_fmaf(__builtin_fmaf(-q1, qs.s, x1), qs.r, q1);
+        }
+        // a zero quotient comes out of the correction as +0: give it the sign of x (s > 0 on this path)
+        pk[i] = cvt_pk_bf16(q0, q1) | (w[i] & 0x80008000u);
+    }
+    // largest magnitude (as bf16 bits) of the eight: at or beyond the first value that does not cast to a finite code?
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    u16x2 m = __builtin_bit_cast(u16x2, pk[0] & 0x7fff7fffu);
+#pragma unroll
+    for (int i = 1; i < 4; ++i) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, pk[i] & 0x7fff7fffu));
+    // e4m3: above 464 (0x43e8) the torch cast gives NaN; e5m2: from 61440 (0x4770) on it gives infinity
+    constexpr unsigned kFirstBad = FMT == FMT_E4M3 ? 0x43e9u : 0x4770u;
+    const bool special = m[0] >= kFirstBad || m[1] >= kFirstBad;
+    if (!qs.fast_ok || __any(special)) return quant8_slow<FMT>(in, qs.s);
+    v2i o;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const float f0 = __uint_as_float(pk[2 * j] << 16), f1 = __uint_as_float(pk[2 * j] & 0xffff0000u);
+        const float f2 = __uint_as_float(pk[2 * j + 1] << 16), f3 = __uint_as_float(pk[2 * j + 1] & 0xffff0000u);
+        int r;
+        if (FMT == FMT_E4M3) {
+            r = __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, __builtin_bit_cast(int, f0), false);
+            r = __builtin_amdgcn_cvt_pk_fp8_f32(f2, f3, r, true);
+        } else {
+            r = __builtin_amdgcn_cvt_pk_bf8_f32(f0, f1, __builtin_bit_cast(int, f0), false);
+            r = __builtin_amdgcn_cvt_pk_bf8_f32(f2, f3, r, true);
+        }
+        o[j] = r;
+    }
+    return o;
+}
+template <int FMT>
+__device__ __forceinline__ v2i quant8(v4i in, float s) {
+    return quant8<FMT>(in, QuantScale(s));
 }
 
 // ---------------------------------------------------------------- wave helpers

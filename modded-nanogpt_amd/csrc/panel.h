@@ -19,60 +19,84 @@ __host__ __device__ inline int64_t panel_offset(int row, int kbyte, int nk /* k-
 
 constexpr int kPanelRaw = -1;    // panel_transpose: the input is fp8 bytes already
 
+// 4 x 4 byte transpose: r[i] holds bytes (columns) 0..3 of row i; afterwards r[j] holds rows 0..3 of column j.
+__device__ __forceinline__ void transpose4x4_bytes(uint32_t (&r)[4]) {
+    // v_perm_b32 D = bytes of {S0, S1} picked by the selector, S1 = bytes 0..3, S0 = bytes 4..7
+    const uint32_t a0 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400);   // r0.b0 r1.b0 r0.b1 r1.b1
+    const uint32_t a1 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602);   // r0.b2 r1.b2 r0.b3 r1.b3
+    const uint32_t b0 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400);
+    const uint32_t b1 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602);
+    r[0] = __builtin_amdgcn_perm(b0, a0, 0x05040100);   // a0.lo16 b0.lo16
+    r[1] = __builtin_amdgcn_perm(b0, a0, 0x07060302);   // a0.hi16 b0.hi16
+    r[2] = __builtin_amdgcn_perm(b1, a1, 0x05040100);
+    r[3] = __builtin_amdgcn_perm(b1, a1, 0x07060302);
+}
+
 // Panel-blocked transpose of a row-major matrix: out row = input column c (c < cols), contraction = input
 // rows [row0, row0 + nrows) padded with zeros to nk * 128, contraction bytes of each k-step permuted by
 // PERM (0 none, 2 dw_pos).  QFMT = kPanelRaw: fp8 input, `ld` in bytes.  QFMT = FMT_E4M3 / FMT_E5M2: bf16
-// input (`ld` in elements) quantised on the way as fp8(bf16(x / scale)).  One workgroup moves a 128 (rows) x
-// 64 (columns) tile.
+// input (`ld` in elements) quantised on the way as fp8(bf16(x / scale)).
+// One workgroup moves a 128 (rows = one k-step) x 128 (columns) tile: 16 KiB of one panel block, contiguous.
+// The tile sits in LDS as fp8 rows of 33 words with the word index XORed by 4 * (row / 16 % 8), which makes
+// the transposing reads below conflict-free.  A thread then owns 4 columns x 16 rows: four 4 x 4 byte
+// blocks, transposed in registers, are the four words of one 16-byte piece of each column's panel row;
+// the 8 threads that share a column group are adjacent lanes, so they write whole 128-byte rows.
 template <int PERM, int QFMT>
 __global__ __launch_bounds__(256) void panel_transpose_kernel(const uint8_t* __restrict__ in, int64_t ld, int row0, int nrows, int cols,
                                                               int nk, float scale, uint8_t* __restrict__ out) {
-    __shared__ __attribute__((aligned(16))) uint8_t tile[128][80];
-    const int kt = blockIdx.x, cg = blockIdx.y, tid = threadIdx.x;
+    constexpr int kStride = 33;
+    __shared__ uint32_t tile[128 * kStride];
+    // neighbouring workgroups take neighbouring column groups of the same rows: together they read whole rows
+    const int cg = blockIdx.x, kt = blockIdx.y, tid = threadIdx.x;
+    auto word_at = [&](int r, int w) -> uint32_t& { return tile[r * kStride + (w ^ (((r >> 4) & 7) << 2))]; };
     if (QFMT == kPanelRaw) {
-        for (int i = tid; i < 512; i += 256) {
-            int r = i >> 2, ch = i & 3;
-            int gr = kt * 128 + r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = tid + 256 * j, r = i >> 3, ch = i & 7;   // 16 input bytes = 16 columns
+            const int gr = kt * 128 + r;
             v4i v = {0, 0, 0, 0};
-            if (gr < nrows && cg * 64 + ch * 16 < cols) v = *(const v4i*)(in + (int64_t)(row0 + gr) * ld + cg * 64 + ch * 16);
-            *(v4i*)&tile[r][ch * 16] = v;
+            if (gr < nrows && cg * 128 + ch * 16 < cols) v = *(const v4i*)(in + (int64_t)(row0 + gr) * ld + cg * 128 + ch * 16);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) word_at(r, ch * 4 + k) = (uint32_t)v[k];
         }
     } else {
-        for (int i = tid; i < 1024; i += 256) {
-            int r = i >> 3, ch = i & 7;
-            int gr = kt * 128 + r;
+        const QuantScale qs(scale);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = tid + 256 * j, r = i >> 4, ch = i & 15;  // 16 input bytes = 8 columns
+            const int gr = kt * 128 + r;
             v2i q = {0, 0};
-            if (gr < nrows && cg * 64 + ch * 8 < cols)
-                q = quant8<QFMT == kPanelRaw ? 0 : QFMT>(*(const v4i*)(in + ((int64_t)(row0 + gr) * ld + cg * 64 + ch * 8) * 2), scale);
-            *(v2i*)&tile[r][ch * 8] = q;
+            if (gr < nrows && cg * 128 + ch * 8 < cols)
+                q = quant8<QFMT == kPanelRaw ? 0 : QFMT>(*(const v4i*)(in + ((int64_t)(row0 + gr) * ld + cg * 128 + ch * 8) * 2), qs);
+            word_at(r, ch * 2) = (uint32_t)q[0];
+            word_at(r, ch * 2 + 1) = (uint32_t)q[1];
         }
     }
     __syncthreads();
-    const int o = tid >> 2, part = tid & 3;
-    const int c = cg * 64 + o;
-    if (c >= cols) return;
-    uint32_t w[8];
+    const int sub = tid & 7, cgp = tid >> 3;      // 16-byte piece of the 128-byte panel row, group of 4 columns
+    // rows whose bytes make up piece `sub`: positions 16 sub ..+15 of the k-step, position 16h + 4g + i of a 32-group
+    // holding row 8g + 4h + i under dw_pos
+    const int rbase = PERM == 2 ? 32 * (sub >> 1) + 4 * (sub & 1) : 16 * sub;
+    uint32_t w[4][4];   // [g][column]
 #pragma unroll
-    for (int d = 0; d < 8; ++d) {
-        uint32_t word = 0;
+    for (int g = 0; g < 4; ++g) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            int p = part * 32 + d * 4 + b;
-            int t = PERM == 2 ? dw_pos_inv(p) : p;
-            word |= (uint32_t)tile[t][o] << (8 * b);
-        }
-        w[d] = word;
+        for (int i = 0; i < 4; ++i) w[g][i] = word_at(rbase + (PERM == 2 ? 8 : 4) * g + i, cgp);
+        transpose4x4_bytes(w[g]);
     }
-    uint8_t* dst = out + panel_offset(c, kt * 128, nk) + part * 32;
-    *(v4i*)dst = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-    *(v4i*)(dst + 16) = (v4i){(int)w[4], (int)w[5], (int)w[6], (int)w[7]};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int col = cg * 128 + cgp * 4 + c;
+        if (col < cols)
+            *(v4i*)(out + panel_offset(col, kt * 128, nk) + sub * 16) = (v4i){(int)w[0][c], (int)w[1][c], (int)w[2][c], (int)w[3][c]};
+    }
 }
 
 template <int PERM, int QFMT = kPanelRaw>
 static int panel_transpose(const void* in, int64_t ld, int row0, int nrows, int cols, int nk, void* out, hipStream_t st,
                            float scale = 1.0f) {
     if (cols % 16 || ld % 16) return fail(NGPT_EALIGN, "panel_transpose: cols=%d ld=%lld", cols, (long long)ld);
-    dim3 grid(nk, (cols + 63) / 64);
+    dim3 grid((cols + 127) / 128, nk);
     panel_transpose_kernel<PERM, QFMT><<<grid, 256, 0, st>>>((const uint8_t*)in, ld, row0, nrows, cols, nk, scale, (uint8_t*)out);
     return check_launch("panel_transpose_kernel");
 }

@@ -9,7 +9,8 @@ __global__ __launch_bounds__(256) void quant_kernel(const v4i* __restrict__ in, 
                                                     int64_t n8, float s) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     int64_t stride = (int64_t)gridDim.x * 256;
-    for (; i < n8; i += stride) out[i] = quant8<FMT>(in[i], s);
+    const QuantScale qs(s);
+    for (; i < n8; i += stride) out[i] = quant8<FMT>(in[i], qs);
 }
 
 // 64 x 64 tile: quantise, write the row-major bytes, and write the transposed bytes via LDS.
@@ -21,6 +22,7 @@ __global__ __launch_bounds__(256) void tile_transpose_kernel(const uint8_t* __re
     __shared__ uint8_t tile[64][64 + 4];   // [col][row]
     const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
     const int t = threadIdx.x;
+    const QuantScale qs(s);
     // phase 1: each thread handles 8 consecutive columns of one row; 8 threads per row, 32 rows per pass
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
@@ -30,7 +32,7 @@ __global__ __launch_bounds__(256) void tile_transpose_kernel(const uint8_t* __re
         if (r < rows && c < cols) {
             if (IN_BYTES == 2) {
                 v4i v = *(const v4i*)(in + ((int64_t)r * cols + c) * 2);
-                q = quant8<FMT>(v, s);
+                q = quant8<FMT>(v, qs);
                 if (out) *(v2i*)(out + (int64_t)r * cols + c) = q;
             } else {
                 q = *(const v2i*)(in + (int64_t)r * cols + c);
