@@ -76,6 +76,22 @@ def test_quant_scaled_bit_exact(amd, oracle, s, dt):
     assert torch.equal(u8(tr_only), u8(ref.T.contiguous()))
 
 
+@pytest.mark.parametrize("s", [0.99999994, 1.9999999, -0.5, 3.0e-5, 7.0e3, 1.0e-39, 2.0e38])
+@pytest.mark.parametrize("dt", [E4M3, E5M2])
+def test_quant_awkward_scales_all_patterns(amd, dt, s):
+    """Scales for which the quantiser must leave its reciprocal-multiply path (significand all ones, negative,
+    subnormal, reciprocal subnormal) or whose quotients overflow / underflow for most inputs: every bf16
+    pattern against torch's own division and casts."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(torch.bfloat16)
+    ref = x.div(s).to(dt)
+    got = amd.quant_fp8(dev(x), s, dt).cpu()
+    r, g = u8(ref).numpy(), u8(got).numpy()
+    nan = np.isnan(ref.float().numpy())
+    assert np.array_equal(g[~nan], r[~nan])
+    assert np.all(np.isnan(got.float().numpy()[nan]))
+
+
 def test_transpose_copy_bytes(amd):
     g = torch.Generator().manual_seed(22)
     for (R, C) in [(64, 64), (16, 48), (208, 1040), (768, 1024)]:
