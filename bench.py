@@ -112,6 +112,22 @@ def secondary(args, amd, oracle) -> int:
         desc = ("config 4 (one layer): " if bwd else "config 2: ") + "norm + quantise + FP8 c_fc with ReLU^2 + bf16 c_proj" + \
                (", forward+backward" if bwd else ", forward") + ", M=49152 D=768 H=3072"
         tokens = Mm
+    elif wl == "ce_logits":
+        # the logits-in-HBM compatibility op: one pass over bf16 logits in, e5m2 gradient out (HBM-bound)
+        Mm, Vv = 49152, 50304
+        logits = torch.empty(Mm, Vv, dtype=torch.bfloat16, device=dev)
+        for r in range(0, Mm, 8192):   # N(0, 4) in slices, to keep the fp32 temporaries small
+            logits[r:r + 8192] = (torch.randn(8192, Vv, device=dev) * 2).bfloat16()
+        targets = torch.randint(0, 50257, (Mm,), generator=g).to(dev)
+        mtp = torch.ones(1, device=dev)
+        ptg = torch.full((Mm,), -1, dtype=torch.int64, device=dev)
+        pw = torch.zeros(1, device=dev)
+        losses = torch.empty(Mm, dtype=torch.float32, device=dev)
+        grad = torch.empty(Mm, Vv, dtype=torch.float8_e5m2, device=dev)
+        step = lambda: torch.ops.nanogpt.ce_fwd_bwd(logits, targets, mtp, ptg, pw, losses, grad, Mm, 1, 23.0, 5.0, 7.5,
+                                                    0.75 / 448, 1.0)
+        hbm_bytes = Mm * Vv * 3 + Mm * 12
+        flops, desc, tokens = 0.0, "nanogpt::ce_fwd_bwd on materialised logits, M=49152 V=50304 (bf16 in, e5m2 gradient out)", Mm
     else:
         print(f"bench.py: unknown workload {wl}", file=sys.stderr)
         return 2
@@ -129,6 +145,17 @@ def secondary(args, amd, oracle) -> int:
     ms = dt / args.steps * 1e3
     tflops = flops / (ms * 1e-3) / 1e12
     peak = PEAK_FP8_TFLOPS
+    if wl == "ce_logits":
+        gbs = hbm_bytes / (ms * 1e-3) / 1e9
+        print(json.dumps({
+            "metric": "tokens/s (secondary workload of the FP8 path)", "value": tokens / (ms * 1e-3), "unit": "tokens/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16 in, fp32 arithmetic, e5m2 out", "data": "synthetic",
+            "config": {"workload": desc}, "event_ms_per_step": e0.elapsed_time(e1) / args.steps,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None,
+                         "note": "algorithmic bytes M*V*(2+1) + M*12 per pass / its duration"},
+        }))
+        return 0
     print(json.dumps({
         "metric": "tokens/s (secondary workload of the FP8 path)", "value": tokens / (ms * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
@@ -143,7 +170,7 @@ def secondary(args, amd, oracle) -> int:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="lmhead_ce",
-                    help="lmhead_ce (default, the headline configuration 3) | mm_cfg1 | mm_lmhead | mlp_fwd | mlp_fwd_bwd")
+                    help="lmhead_ce (default, the headline configuration 3) | mm_cfg1 | mm_lmhead | mlp_fwd | mlp_fwd_bwd | ce_logits")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)

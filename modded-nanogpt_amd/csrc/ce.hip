@@ -216,6 +216,144 @@ __global__ __launch_bounds__(ROW_THREADS) void ce_rows_kernel(
     }
 }
 
+// Rows of up to MAXC * 8 * ROWREG_THREADS columns: a thread keeps its 16-byte pieces of the row in
+// registers -- as table offsets, which both sweeps use -- so the logits are read from memory once, and the
+// pieces of the next row are loaded while this one is processed.  The thread that owns a target column
+// hands the raw logit to the candidate's thread through LDS and patches the exact gradient code into its
+// own 8 output bytes before storing them, so every byte of the gradient is written once.
+constexpr int ROWREG_THREADS = 1024;
+
+template <int MAXC>
+__global__ __launch_bounds__(ROWREG_THREADS) void ce_rows_reg_kernel(
+    const uint16_t* __restrict__ logits, CandArgs ca, float* __restrict__ losses, uint8_t* __restrict__ grad,
+    const float* __restrict__ gtabE, const float* __restrict__ gtabD, Softcap sc, float coef) {
+    __shared__ float tabE[TAB_ENTRIES];
+    __shared__ float tabD[TAB_ENTRIES];
+    __shared__ float red[16];
+    __shared__ uint32_t tl[MAX_CAND];      // raw bf16 bits of the logit at each candidate's target column
+    __shared__ uint32_t fix[MAX_CAND];     // exact e5m2 code for that column
+    __shared__ float loss_term[MAX_CAND];
+    load_table(tabE, gtabE);
+    load_table(tabD, gtabD);
+    const int V = ca.V, n8 = V / 8, tid = threadIdx.x, ncand = ca.n_predict + 1;
+    auto load_row = [&](int row, v4i (&w)[MAXC]) {
+        const uint16_t* lrow = logits + (int64_t)row * V;
+#pragma unroll
+        for (int s_ = 0; s_ < MAXC; ++s_) {
+            const int i = tid + s_ * ROWREG_THREADS;
+            w[s_] = (i < n8) ? *(const v4i*)(lrow + i * 8) : (v4i){0, 0, 0, 0};
+        }
+    };
+    v4i cur[MAXC], nxt[MAXC];
+    int row = blockIdx.x;
+    if (row < ca.M) load_row(row, cur);
+    __syncthreads();
+    for (; row < ca.M; row += gridDim.x) {
+        const int next_row = row + gridDim.x;
+        if (next_row < ca.M) load_row(next_row, nxt);
+        // candidate target columns: the owner publishes the raw logit
+        int my_cand_slot[MAX_CAND], my_cand_pos[MAX_CAND];
+#pragma unroll
+        for (int c = 0; c < MAX_CAND; ++c) {
+            my_cand_slot[c] = -1;
+            my_cand_pos[c] = 0;
+            if (c < ncand) {
+                const int64_t t = cand_target(ca, row, c);
+                if (t >= 0 && t < V) {
+                    const int i8 = (int)(t >> 3);
+                    if ((i8 % ROWREG_THREADS) == tid) {
+                        my_cand_slot[c] = i8 / ROWREG_THREADS;
+                        my_cand_pos[c] = (int)(t & 7);
+                        uint32_t word = 0;
+#pragma unroll
+                        for (int s_ = 0; s_ < MAXC; ++s_)
+#pragma unroll
+                            for (int k = 0; k < 4; ++k)
+                                if (s_ == my_cand_slot[c] && k == (my_cand_pos[c] >> 1)) word = (uint32_t)cur[s_][k];
+                        tl[c] = (my_cand_pos[c] & 1) ? (word >> 16) : (word & 0xffffu);
+                    }
+                }
+            }
+        }
+        // sweep 1: table offsets (kept) and the sum of exponentials
+        float sum = 0.0f;
+#pragma unroll
+        for (int s_ = 0; s_ < MAXC; ++s_) {
+            const bool live = tid + s_ * ROWREG_THREADS < n8;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t off = tab_offsets2((uint32_t)cur[s_][k]);
+                cur[s_][k] = (int)off;
+                if (live) sum += tab_at(tabE, off & 0xffffu) + tab_at(tabE, off >> 16);
+            }
+        }
+        const float S = block_sum(sum, red);      // (its barriers also publish tl[])
+        const float lse = sc.A + logf(S);
+        const float s_w = row_weight_sum(ca, row);
+        const float p_scale = expf(sc.A - lse);
+        const float rowf = coef * (s_w * p_scale);
+        if (tid < ncand) {
+            const int c = tid;
+            const int64_t t = cand_target(ca, row, c);
+            float term = 0.0f;
+            uint32_t code = 0;
+            if (t >= 0 && t < V) {
+                const float sg = softcap_sigma(bf16_bits_to_f32(tl[c]), sc);
+                term = cand_weight(ca, c) * (lse - sc.A * sg);
+                const float p = softcap_E(sg, sc) * p_scale;
+                float term2 = 0.0f;
+                for (int k = 0; k < ncand; ++k)
+                    if (cand_target(ca, row, k) == t) term2 += cand_weight(ca, k);   // every prediction that lands on this column
+                const float gx = coef * (s_w * p - term2) * sg * (1.0f - sg);
+                code = f32x2_to_e5m2_sat(gx, gx) & 0xffu;
+            }
+            loss_term[c] = term;
+            fix[c] = code;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float total = 0.0f;
+            for (int c = 0; c < ncand; ++c) total += loss_term[c];
+            losses[row] = total;
+        }
+        // sweep 2: gradient codes, the exact ones patched in by their owners
+        const bool big = !(fabsf(rowf) <= 4.0f * 57344.0f);
+        uint8_t* grow = grad + (int64_t)row * V;
+#pragma unroll
+        for (int s_ = 0; s_ < MAXC; ++s_) {
+            const int i = tid + s_ * ROWREG_THREADS;
+            if (i < n8) {
+                float g[8];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t off = (uint32_t)cur[s_][k];
+                    g[2 * k] = rowf * tab_at(tabD, off & 0xffffu);
+                    g[2 * k + 1] = rowf * tab_at(tabD, off >> 16);
+                }
+                uint32_t o[2];
+                if (big) {
+                    o[0] = f32x4_to_e5m2_sat<true>(g[0], g[1], g[2], g[3]);
+                    o[1] = f32x4_to_e5m2_sat<true>(g[4], g[5], g[6], g[7]);
+                } else {
+                    o[0] = f32x4_to_e5m2_sat<false>(g[0], g[1], g[2], g[3]);
+                    o[1] = f32x4_to_e5m2_sat<false>(g[4], g[5], g[6], g[7]);
+                }
+#pragma unroll
+                for (int c = 0; c < MAX_CAND; ++c)
+                    if (my_cand_slot[c] == s_) {
+                        const int sh = 8 * (my_cand_pos[c] & 3);
+                        uint32_t& word = o[my_cand_pos[c] >> 2];
+                        word = (word & ~(0xffu << sh)) | (fix[c] << sh);
+                    }
+                *(v2i*)(grow + i * 8) = (v2i){(int)o[0], (int)o[1]};
+            }
+        }
+#pragma unroll
+        for (int s_ = 0; s_ < MAXC; ++s_) cur[s_] = nxt[s_];
+        __syncthreads();     // tl / fix / loss_term / red are reused by the next row
+    }
+}
+
 // =====================================================================================================
 // Fused forward.  GEMM orientation: rows = vocabulary (A = w_f8 [V, K]), columns = tokens
 // (B = x_f8 [M, K]), so one lane owns one token per MFMA tile column and sums exponentials in
@@ -687,8 +825,18 @@ extern "C" int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, 
     float* tabD = tabE + TAB_ENTRIES;
     ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
     CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, n_rows, n_cols};
-    int grid = num_cus() * 2;
+    int grid = num_cus();
     if (grid <= 0) return fail(NGPT_EINVAL, "no HIP device");
+    if (n_cols <= 8 * 8 * ROWREG_THREADS) {    // a row fits the registers of one workgroup
+        if (grid > n_rows) grid = n_rows;
+        const float coef = make_coef(A, C, grad_s, grad_scale);
+        if (n_cols <= 4 * 8 * ROWREG_THREADS)
+            ce_rows_reg_kernel<4><<<grid, ROWREG_THREADS, 0, st>>>((const uint16_t*)logits_bf16, ca, losses, (uint8_t*)grad_e5m2, tabE, tabD, sc, coef);
+        else
+            ce_rows_reg_kernel<8><<<grid, ROWREG_THREADS, 0, st>>>((const uint16_t*)logits_bf16, ca, losses, (uint8_t*)grad_e5m2, tabE, tabD, sc, coef);
+        return check_launch("ce_rows_reg_kernel");
+    }
+    grid *= 2;
     if (grid > n_rows) grid = n_rows;
     ce_rows_kernel<<<grid, ROW_THREADS, 0, st>>>((const uint16_t*)logits_bf16, ca, losses, (uint8_t*)grad_e5m2,
                                                  tabE, tabD, sc, make_coef(A, C, grad_s, grad_scale));
