@@ -253,7 +253,9 @@ def _codes_close(got, ref, frac=1e-3):
     assert ((g - r).abs()[diff] <= 1).all()
 
 
-@pytest.mark.parametrize("M,V,n_predict,prefix", [(64, 1024, 1, False), (96, 50304, 1, False), (80, 2048, 3, True)])
+@pytest.mark.parametrize("M,V,n_predict,prefix", [(64, 1024, 1, False), (96, 50304, 1, False), (80, 2048, 3, True),
+                                                   (300, 40000, 2, True),     # more rows than workgroups, 4 + 4 register pieces
+                                                   (12, 66048, 1, False)])    # rows too long for the register-resident kernel
 def test_ce_fwd_bwd_on_logits(amd, oracle, M, V, n_predict, prefix):
     g = torch.Generator().manual_seed(M + V)
     logits = (torch.randn(M, V, generator=g) * 4).bfloat16()
