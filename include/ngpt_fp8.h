@@ -155,6 +155,11 @@ int64_t ngpt_mlp_input_quant_workspace_bytes(void);
 int ngpt_mlp_input_quant(const void* x_bf16, int rows, int dim, const float* up_scale, void* normed_bf16,
                          void* x_f8, float* dequant, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Backward of the norm inside ngpt_mlp_input_quant: dx = d/dx [ F.rms_norm(x, (dim,)) ] . g for bf16 x, g
+ * [rows, dim], fp32 arithmetic, one rounding to bf16 (the reference leaves this to autograd through
+ * `norm`, train_gpt.py:952-953 and 1643).  dim % 8 == 0, dim <= 2048. */
+int ngpt_rmsnorm_bwd(const void* x_bf16, const void* g_bf16, int rows, int dim, void* dx_bf16, void* stream);
+
 /* Up-projection part of GPT.quantize_mlp_fp8, train_gpt.py:1419-1422: per layer l of w [layers, per_layer] bf16,
  *   scales[l] = bf16(max(amax(|w_l|), 1e-12) / 448)   (written as fp32)
  *   w_f8[l]   = e4m3(bf16(w_l / scales[l]))

@@ -36,6 +36,7 @@ SIGNATURES = {
     "ngpt_quant_transpose_down": (_I, [_P, _I, _I, _I, _L, _P, _P, _P, _P, _P]),
     "ngpt_mlp_input_quant_workspace_bytes": (_L, []),
     "ngpt_mlp_input_quant": (_I, [_P, _I, _I, _P, _P, _P, _P, _P, _L, _P]),
+    "ngpt_rmsnorm_bwd": (_I, [_P, _P, _I, _I, _P, _P]),
     "ngpt_quant_up_weights_workspace_bytes": (_L, [_I]),
     "ngpt_quant_up_weights": (_I, [_P, _I, _L, _P, _P, _P, _L, _P]),
     "ngpt_transpose_add": (_I, [_P, _I, _I, _P, _I, _P]),

@@ -9,23 +9,23 @@ namespace ngpt {
 // layout (a lane owns one column and scattered rows: 1-byte or 4-byte pieces per row), so the
 // wave parks a strip in its private LDS scratch and writes it back out in 16-byte pieces.
 
-// Strip = 32 rows x WTN columns of bytes, stored row-major in global memory (leading dim ld).
-// `codes[tn][v]` holds the byte for accumulator element (tn, v) of one tm.
+// Strip = 32 rows x WTN columns of bytes in the wave's LDS scratch, rows padded where the scratch allows it
+// (fewer bank conflicts on the 16-byte reads).
 template <class Cfg>
-__device__ __forceinline__ void store_strip_rowmajor_u8(
-    const uint32_t (&codes)[Cfg::TN][16], uint8_t* scratch, int lane,
-    uint8_t* out, int64_t ld, int grow0 /* global row of strip row 0 */, int gcol0, int R, int C) {
-    // padded rows where the wave's scratch allows it (fewer bank conflicts on the 16-byte reads)
-    constexpr int STRIDE = (32 * (Cfg::WTN + 16) <= Cfg::WAVE_SCRATCH) ? Cfg::WTN + 16 : Cfg::WTN;
+struct StripU8 {
+    static constexpr int STRIDE = (32 * (Cfg::WTN + 16) <= Cfg::WAVE_SCRATCH) ? Cfg::WTN + 16 : Cfg::WTN;
     static_assert(32 * STRIDE <= Cfg::WAVE_SCRATCH, "strip does not fit the wave's LDS scratch");
-    const int h = lane >> 5, j = lane & 31;
-#pragma unroll
-    for (int tn = 0; tn < Cfg::TN; ++tn)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            int rl = 8 * (v >> 2) + 4 * h + (v & 3);
-            scratch[rl * STRIDE + tn * 32 + j] = (uint8_t)codes[tn][v];
-        }
+    // byte of accumulator element (tn, v) of the strip's tm
+    static __device__ __forceinline__ void put(uint8_t* scratch, int lane, int tn, int v, uint32_t code) {
+        const int rl = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        scratch[rl * STRIDE + tn * 32 + (lane & 31)] = (uint8_t)code;
+    }
+};
+// The strip, complete in LDS, to global memory: row-major with leading dimension ld, 16 bytes per lane.
+template <class Cfg>
+__device__ __forceinline__ void strip_flush_rowmajor_u8(uint8_t* scratch, int lane, uint8_t* out, int64_t ld,
+                                                        int grow0 /* global row of strip row 0 */, int gcol0, int R, int C) {
+    constexpr int STRIDE = StripU8<Cfg>::STRIDE;
     __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the wave's own LDS writes have landed
     constexpr int CH_PER_ROW = Cfg::WTN / 16;
 #pragma unroll
@@ -37,6 +37,19 @@ __device__ __forceinline__ void store_strip_rowmajor_u8(
         if (gr < R && gc + 16 <= C) *(v4i*)(out + (int64_t)gr * ld + gc) = val;
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
+}
+
+// Strip = 32 rows x WTN columns of bytes, stored row-major in global memory (leading dim ld).
+// `codes[tn][v]` holds the byte for accumulator element (tn, v) of one tm.
+template <class Cfg>
+__device__ __forceinline__ void store_strip_rowmajor_u8(
+    const uint32_t (&codes)[Cfg::TN][16], uint8_t* scratch, int lane,
+    uint8_t* out, int64_t ld, int grow0 /* global row of strip row 0 */, int gcol0, int R, int C) {
+#pragma unroll
+    for (int tn = 0; tn < Cfg::TN; ++tn)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) StripU8<Cfg>::put(scratch, lane, tn, v, codes[tn][v]);
+    strip_flush_rowmajor_u8<Cfg>(scratch, lane, out, ld, grow0, gcol0, R, C);
 }
 
 // Strip = 32 columns x WTM rows, stored transposed: out[col][row], leading dim ld.
@@ -285,19 +298,20 @@ using EpiDiscardAblate = EpiDiscardT<true>;    // honours GemmOperands::ablate, 
 
 // post = bf16(max(bf16(acc * *dequant), 0)^2); optionally post_f8 = e4m3(min(post / act_scale, 448))
 // and a per-workgroup running max of post written to partial_amax[bid].
-struct EpiRelu2 {
+template <bool EMIT>      // EMIT: also the e4m3 copy of post and the per-workgroup maxima
+struct EpiRelu2T {
     uint16_t* post;
     int64_t ld;
     const float* dequant;        // 1-element device tensor
-    uint8_t* post_f8;            // nullable
+    uint8_t* post_f8;            // EMIT only
     int64_t ld_f8;
-    const float* act_scale;      // 1-element device tensor, required with post_f8
-    float* partial_amax;         // nullable; n_partials entries
+    const float* act_scale;      // 1-element device tensor, EMIT only
+    float* partial_amax;         // EMIT only; n_partials entries
     int n_partials;
     int R, C;
     float scale, inv_act, amax;
     static constexpr int EXTRA_LDS = 0;
-    static constexpr bool NEEDS_SCRATCH = true;
+    static constexpr bool NEEDS_SCRATCH = EMIT;     // the e4m3 strip is staged through the free operand slot
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     template <class Cfg>
     __device__ void job_begin(int) {}
@@ -306,39 +320,48 @@ struct EpiRelu2 {
     __device__ void partial(bool) {}
     __device__ void begin(int, int, uint8_t*) {
         scale = *dequant;
-        inv_act = post_f8 ? 1.0f / *act_scale : 0.0f;
+        inv_act = EMIT ? 1.0f / *act_scale : 0.0f;
         amax = 0.0f;
     }
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t* scratch, int lane) {
+        // address = wave-uniform pointer + ONE per-lane 32-bit offset, as in EpiStoreBf16
+        uint16_t* origin = post + ((int64_t)r0 * ld + c0);
+        const uint32_t lane_off = (uint32_t)co.row_base * (uint32_t)ld + (uint32_t)co.col_base;
+        const int rlim = R - r0 - co.row_base, clim = C - c0 - co.col_base;
+        const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
 #pragma unroll
         for (int tm = 0; tm < Cfg::TM; ++tm) {
-            uint32_t codes[Cfg::TN][16];
 #pragma unroll
             for (int tn = 0; tn < Cfg::TN; ++tn) {
-                int c = c0 + co.col(tn);
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    int r = r0 + co.row(tm, v);
-                    float pre = round_to_bf16(acc[tm][tn][v] * scale);
-                    pre = fmaxf(pre, 0.0f);
-                    float p = round_to_bf16(pre * pre);
-                    bool ok = (r < R && c < C);
-                    if (ok) post[(int64_t)r * ld + c] = (uint16_t)(__float_as_uint(p) >> 16);
-                    if (post_f8) {
-                        codes[tn][v] = f32_to_e4m3_sat(fminf(p * inv_act, 448.0f));
-                        amax = ok ? fmaxf(amax, p) : amax;
+                for (int v = 0; v < 16; v += 2) {
+                    const int dr = co.dr(tm, v), dc = tn * 32;
+                    // c = bf16(acc * dequant); post = bf16(max(c, 0)^2): both roundings by the packed converter
+                    const uint32_t pre = cvt_pk_bf16(acc[tm][tn][v] * scale, acc[tm][tn][v + 1] * scale);
+                    const float c0f = fmaxf(__uint_as_float(pre << 16), 0.0f), c1f = fmaxf(__uint_as_float(pre & 0xffff0000u), 0.0f);
+                    const uint32_t pk = cvt_pk_bf16(c0f * c0f, c1f * c1f);
+                    uint16_t* pu = origin + ((int64_t)dr * ld + dc);
+                    const bool ok0 = full || (dr < rlim && dc < clim), ok1 = full || (dr + 1 < rlim && dc < clim);
+                    if (ok0) pu[lane_off] = (uint16_t)pk;
+                    if (ok1) pu[lane_off + (uint32_t)ld] = (uint16_t)(pk >> 16);
+                    if (EMIT) {
+                        const float p0 = __uint_as_float(pk << 16), p1 = __uint_as_float(pk & 0xffff0000u);
+                        StripU8<Cfg>::put(scratch, lane, tn, v, f32_to_e4m3_sat(fminf(p0 * inv_act, 448.0f)));
+                        StripU8<Cfg>::put(scratch, lane, tn, v + 1, f32_to_e4m3_sat(fminf(p1 * inv_act, 448.0f)));
+                        amax = ok0 ? fmaxf(amax, p0) : amax;
+                        amax = ok1 ? fmaxf(amax, p1) : amax;
                     }
                 }
+                if (!EMIT) __builtin_amdgcn_sched_barrier(0);
             }
-            if (post_f8)
-                store_strip_rowmajor_u8<Cfg>(codes, scratch, lane, post_f8, ld_f8,
-                                             r0 + co.wave_row0 + tm * 32, c0 + co.wave_col0, R, C);
+            if constexpr (EMIT)
+                strip_flush_rowmajor_u8<Cfg>(scratch, lane, post_f8, ld_f8, r0 + co.wave_row0 + tm * 32, c0 + co.wave_col0, R, C);
         }
     }
     __device__ void end(uint8_t* smem, int bid, int G) {
-        if (!partial_amax) return;
+        if (!EMIT || !partial_amax) return;
         float m = wave_max(amax);
         float* red = (float*)smem;
         int wave = threadIdx.x >> 6;

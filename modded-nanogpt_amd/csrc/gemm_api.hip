@@ -347,17 +347,25 @@ extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float
     if (int e = check_gemm_dims("ngpt_fc_relu2_fwd", M, N, K, K, K)) return e;
     if (N % 16) return fail(NGPT_EALIGN, "ngpt_fc_relu2_fwd: N=%d must be a multiple of 16", N);
     GemmOperands g{(const uint8_t*)x_f8, (const uint8_t*)w_f8, K, K, M, N, K, 1, 0};
-    EpiRelu2 epi{};
-    epi.post = (uint16_t*)post_bf16;
-    epi.ld = N;
-    epi.dequant = dequant;
-    epi.post_f8 = (uint8_t*)post_f8;
-    epi.ld_f8 = N;
-    epi.act_scale = act_scale;
-    epi.partial_amax = post_f8 ? partial_amax : nullptr;
-    epi.n_partials = n_partials;
-    epi.R = M;
-    epi.C = N;
-    int max_grid = post_f8 ? n_partials : 0;   // one partial-amax slot per persistent workgroup
-    return launch_gemm<MainCfg>(g, FMT_E4M3, FMT_E4M3, epi, (hipStream_t)stream, max_grid);
+    auto fill = [&](auto& epi) {
+        epi.post = (uint16_t*)post_bf16;
+        epi.ld = N;
+        epi.dequant = dequant;
+        epi.post_f8 = (uint8_t*)post_f8;
+        epi.ld_f8 = N;
+        epi.act_scale = act_scale;
+        epi.partial_amax = post_f8 ? partial_amax : nullptr;
+        epi.n_partials = n_partials;
+        epi.R = M;
+        epi.C = N;
+    };
+    if (post_f8) {
+        EpiRelu2T<true> epi{};
+        fill(epi);
+        // one partial-amax slot per persistent workgroup
+        return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(g, epi, (hipStream_t)stream, n_partials);
+    }
+    EpiRelu2T<false> epi{};
+    fill(epi);
+    return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(g, epi, (hipStream_t)stream, 0);
 }

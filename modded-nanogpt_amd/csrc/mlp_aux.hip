@@ -286,6 +286,68 @@ extern "C" int ngpt_mlp_input_quant(const void* x_bf16, int rows, int dim, const
     return check_launch("amax_quant_kernel");
 }
 
+// Backward of y = x * rsqrt(mean(x^2) + eps) (F.rms_norm on bf16 input, eps = fp32 machine epsilon):
+// dx = r * g - x * r^3 * mean(g * x), r = rsqrt(mean(x^2) + eps), in fp32, rounded to bf16 once.
+// One wave per row, the row's x and g stay in registers between the reduction and the output.
+__global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ g, int rows,
+                                                          int dim, uint16_t* __restrict__ dx) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int chunks = dim / 8;              // 16-byte chunks per row
+    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+        const v4i* xr = (const v4i*)(x + (int64_t)row * dim);
+        const v4i* gr = (const v4i*)(g + (int64_t)row * dim);
+        v4i bx[4], bg[4];                    // up to 4 chunks per lane: dim <= 2048
+        float ss = 0.0f, sg = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int ch = lane + 64 * c;
+            if (ch < chunks) {
+                bx[c] = xr[ch];
+                bg[c] = gr[ch];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t ux = (uint32_t)bx[c][i], ug = (uint32_t)bg[c][i];
+                    const float x0 = bf16_bits_to_f32(ux & 0xffffu), x1 = bf16_bits_to_f32(ux >> 16);
+                    const float g0 = bf16_bits_to_f32(ug & 0xffffu), g1 = bf16_bits_to_f32(ug >> 16);
+                    ss += x0 * x0 + x1 * x1;
+                    sg += g0 * x0 + g1 * x1;
+                }
+            }
+        }
+        ss = wave_sum(ss);
+        sg = wave_sum(sg);
+        const float r = __fdiv_rn(1.0f, __fsqrt_rn(ss / (float)dim + 1.1920928955078125e-07f));
+        const float k = r * r * r * (sg / (float)dim);
+        v4i* out = (v4i*)(dx + (int64_t)row * dim);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int ch = lane + 64 * c;
+            if (ch < chunks) {
+                v4i o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t ux = (uint32_t)bx[c][i], ug = (uint32_t)bg[c][i];
+                    const float d0 = r * bf16_bits_to_f32(ug & 0xffffu) - k * bf16_bits_to_f32(ux & 0xffffu);
+                    const float d1 = r * bf16_bits_to_f32(ug >> 16) - k * bf16_bits_to_f32(ux >> 16);
+                    o[i] = (int)cvt_pk_bf16(d0, d1);
+                }
+                out[ch] = o;
+            }
+        }
+    }
+}
+
+extern "C" int ngpt_rmsnorm_bwd(const void* x_bf16, const void* g_bf16, int rows, int dim, void* dx_bf16, void* stream) {
+    if (!x_bf16 || !g_bf16 || !dx_bf16) return fail(NGPT_EINVAL, "ngpt_rmsnorm_bwd: null pointer");
+    if (rows <= 0 || dim <= 0) return fail(NGPT_EINVAL, "ngpt_rmsnorm_bwd: empty problem");
+    if (dim % 8 || dim > 2048) return fail(NGPT_EALIGN, "ngpt_rmsnorm_bwd: dim=%d must be a multiple of 8 and <= 2048", dim);
+    int blocks = (rows + 3) / 4;
+    const int cap = num_cus() * 16;
+    if (blocks > cap) blocks = cap;
+    rmsnorm_bwd_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x_bf16, (const uint16_t*)g_bf16, rows, dim, (uint16_t*)dx_bf16);
+    return check_launch("rmsnorm_bwd_kernel");
+}
+
 constexpr int kLayerPartials = 64;
 extern "C" int64_t ngpt_quant_up_weights_workspace_bytes(int layers) { return (int64_t)layers * kLayerPartials * sizeof(float); }
 

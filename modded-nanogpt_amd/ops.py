@@ -384,8 +384,26 @@ def _(x, up_scale):
             torch.empty(1, dtype=torch.float32, device=x.device))
 
 
+@torch.library.custom_op("nanogpt::rms_norm_backward", mutates_args=())
+def rms_norm_backward(g: Tensor, x: Tensor) -> Tensor:
+    """dx of y = F.rms_norm(x, (D,)) for the incoming gradient g: bf16 in and out, fp32 arithmetic."""
+    _gpu(g, x)
+    assert x.dtype == torch.bfloat16 and g.dtype == torch.bfloat16 and x.shape == g.shape
+    x, g = x.contiguous(), g.contiguous()
+    dim = x.shape[-1]
+    dx = torch.empty_like(x)
+    _lib.check(_lib.load().ngpt_rmsnorm_bwd(_p(x), _p(g), x.numel() // dim, dim, _p(dx), _stream(x)), "ngpt_rmsnorm_bwd")
+    return dx
+
+
+@rms_norm_backward.register_fake
+def _(g, x):
+    return torch.empty_like(x)
+
+
 def _mlp_input_quant_setup(ctx, inputs, output):
     ctx.save_for_backward(inputs[0])
+    ctx.set_materialize_grads(False)     # no zero tensors for the fp8 copy and the scale, which carry no gradient
 
 
 def _mlp_input_quant_backward(ctx, d_normed, d_x_f8, d_dequant):
@@ -393,11 +411,7 @@ def _mlp_input_quant_backward(ctx, d_normed, d_x_f8, d_dequant):
     (x,) = ctx.saved_tensors
     if d_normed is None:
         return None, None
-    with torch.enable_grad():
-        xr = x.detach().requires_grad_(True)
-        y = torch.nn.functional.rms_norm(xr, (xr.size(-1),))
-    (dx,) = torch.autograd.grad(y, xr, d_normed)
-    return dx, None
+    return torch.ops.nanogpt.rms_norm_backward(d_normed, x), None
 
 
 mlp_input_quant.register_autograd(_mlp_input_quant_backward, setup_context=_mlp_input_quant_setup)

@@ -456,14 +456,18 @@ def test_mlp_input_quant(amd, oracle, rows, dim):
     assert torch.equal(dequant.cpu(), ref_dq)
 
 
-def test_mlp_input_quant_grad(amd):
-    x = torch.randn(256, 768).bfloat16()
+@pytest.mark.parametrize("shape", [(256, 768), (1001, 1024), (2, 37, 2048), (5, 64)])
+def test_mlp_input_quant_grad(amd, shape):
+    """Gradient through the norm (own kernel) against autograd of F.rms_norm on the CPU."""
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g) * 3).bfloat16()
     xd = dev(x).requires_grad_(True)
     normed, _, _ = torch.ops.nanogpt.mlp_input_quant(xd, torch.ones(1, device="cuda"))
-    gy = torch.randn(256, 768).bfloat16()
+    gy = torch.randn(*shape, generator=g).bfloat16()
     normed.backward(dev(gy))
     xr = x.clone().requires_grad_(True)
-    torch.nn.functional.rms_norm(xr, (768,)).backward(gy)
+    torch.nn.functional.rms_norm(xr, (shape[-1],)).backward(gy)
+    assert xd.grad.dtype == torch.bfloat16 and xd.grad.shape == x.shape
     torch.testing.assert_close(xd.grad.cpu().float(), xr.grad.float(), rtol=2e-2, atol=1e-3)
 
 
