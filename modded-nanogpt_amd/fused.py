@@ -97,6 +97,22 @@ def linear_relu_square(a, b, aux=None, a_f8=None, b_f8=None, dequant_scale_ptr=N
     return ops.fc_relu2_bwd_dpre(a.contiguous(), b.contiguous(), aux.contiguous())
 
 
+def _tokens_contraction(a: Tensor, b: Tensor) -> Tensor:
+    """a.T @ b for a [M, P], b [M, Q] with the tokens M as contraction (the weight gradients of the MLP,
+    triton_kernels.py:722, 727).  A [P, Q] result is only a few dozen tiles for the library's GEMM, which
+    leaves most of the 256 compute units idle (451 us for 49152 x 3072 x 768); cut into 16 slices of the
+    contraction, the same library runs a batch of 16 such GEMMs in 251 us.  The slices' bf16 results are
+    summed in fp32 (measured: same error against an fp32 product as the single GEMM)."""
+    M = a.shape[0]
+    slices = 16
+    while slices > 1 and (M % slices or M // slices < 2048):
+        slices //= 2
+    if slices == 1:
+        return a.T @ b
+    parts = torch.bmm(a.view(slices, M // slices, a.shape[1]).transpose(1, 2), b.view(slices, M // slices, b.shape[1]))
+    return parts.sum(0, dtype=torch.float32).to(a.dtype)
+
+
 class FusedLinearReLUSquareFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, W1, W2, W1_f8=None, dequant_scale=None, x_f8=None, W2_f8=None, W2_scale=None,
@@ -137,9 +153,9 @@ class FusedLinearReLUSquareFunction(torch.autograd.Function):
         x, W1, W2, post = ctx.saved_tensors
         x_flat = x.view((-1, x.shape[-1]))
         g = grad_output.reshape((-1, grad_output.shape[-1]))
-        dW2 = post.T @ g
+        dW2 = _tokens_contraction(post, g)
         dpre = linear_relu_square(g, W2, aux=post)
-        dW1 = dpre.T @ x_flat
+        dW1 = _tokens_contraction(dpre, x_flat)
         dx = dpre @ W1
         return dx.view(x.shape), dW1, dW2, None, None, None, None, None, None, None
 

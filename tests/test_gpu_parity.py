@@ -423,6 +423,19 @@ def test_mlp_forward_with_fp8_down_projection(amd, oracle):
     assert float(partial.max()) > 0
 
 
+@pytest.mark.parametrize("M", [1000, 4096, 32768, 49152])
+def test_tokens_contraction_slices(amd, M):
+    """The weight-gradient GEMMs of the MLP backward (contraction over tokens) in slices against an fp32 product."""
+    from modded_nanogpt_amd.fused import _tokens_contraction
+    g = torch.Generator().manual_seed(M)
+    a = torch.randn(M, 96, generator=g).bfloat16().cuda()
+    b = torch.randn(M, 160, generator=g).bfloat16().cuda()
+    got = _tokens_contraction(a, b)
+    ref = a.float().T @ b.float()
+    assert got.shape == (96, 160) and got.dtype == torch.bfloat16
+    assert_close_gemm(got, ref.cpu())
+
+
 @pytest.mark.parametrize("M,D,H", [(256, 64, 256), (1000, 768, 3072), (2048, 1024, 4096)])
 def test_dpre_bf16_kernel(amd, oracle, M, D, H):
     """bf16 MFMA GEMM with the 2*c*sqrt(post) epilogue, incl. a token count that is not a tile multiple."""
