@@ -112,6 +112,29 @@ def secondary(args, amd, oracle) -> int:
         desc = ("config 4 (one layer): " if bwd else "config 2: ") + "norm + quantise + FP8 c_fc with ReLU^2 + bf16 c_proj" + \
                (", forward+backward" if bwd else ", forward") + ", M=49152 D=768 H=3072"
         tokens = Mm
+    elif wl == "cfg5":
+        # medium-track shapes: FP8 lm_head + softcapped CE forward+backward and one FP8 MLP layer forward+backward per step
+        Mm, D, H, Vv = 65536, 1024, 4096, 50304
+        xh = torch.randn(Mm, D, generator=g).bfloat16().to(dev).requires_grad_(True)
+        wh = (torch.randn(Vv, D, generator=g) / math.sqrt(D)).bfloat16().to(dev).requires_grad_(True)
+        tg = torch.randint(0, 50257, (Mm,), generator=g).to(dev)
+        xr = (torch.randn(Mm, D, generator=g) * 2).bfloat16().to(dev).requires_grad_(True)
+        w_fc = (torch.randn(H, D, generator=g) / math.sqrt(D)).bfloat16().to(dev).requires_grad_(True)
+        w_pt = (torch.randn(D, H, generator=g) / math.sqrt(H)).bfloat16().T.contiguous().to(dev).requires_grad_(True)
+        dy = (torch.randn(1, Mm, D, generator=g) * 1e-3).bfloat16().to(dev)
+        w_f8, scales = torch.ops.nanogpt.quant_up_weights(w_fc.detach()[None])
+
+        def step():
+            xh.grad = wh.grad = xr.grad = w_fc.grad = w_pt.grad = None
+            losses = amd.FusedSoftcappedCrossEntropy.apply(xh, tg, None, None, None, wh, 100 / 448, 1.6 / 448, 0.75 / 448, 1.0,
+                                                           23.0, 5.0, 7.5, "out_in")
+            losses.sum().backward()
+            normed, x_f8, dequant = torch.ops.nanogpt.mlp_input_quant(xr, scales[0:1])
+            out = amd.ReLUSqrdMLP(normed[None], w_fc, w_pt, w_f8[0], dequant, x_f8[None])
+            out.backward(dy)
+            return out
+        flops = 6.0 * Mm * D * Vv + 12.0 * Mm * D * H
+        desc, tokens = "config 5: lm_head + softcapped CE forward+backward and one FP8 MLP layer forward+backward, M=65536 D=1024 H=4096 V=50304", Mm
     elif wl == "ce_logits":
         # the logits-in-HBM compatibility op: one pass over bf16 logits in, e5m2 gradient out (HBM-bound)
         Mm, Vv = 49152, 50304
@@ -170,7 +193,7 @@ def secondary(args, amd, oracle) -> int:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="lmhead_ce",
-                    help="lmhead_ce (default, the headline configuration 3) | mm_cfg1 | mm_lmhead | mlp_fwd | mlp_fwd_bwd | ce_logits")
+                    help="lmhead_ce (default, the headline configuration 3) | mm_cfg1 | mm_lmhead | mlp_fwd | mlp_fwd_bwd | ce_logits | cfg5")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
