@@ -217,14 +217,15 @@ __global__ __launch_bounds__(ROW_THREADS) void ce_rows_kernel(
 }
 
 // Rows of up to MAXC * 8 * ROWREG_THREADS columns: a thread keeps its 16-byte pieces of the row in
-// registers -- as table offsets, which both sweeps use -- so the logits are read from memory once, and the
-// pieces of the next row are loaded while this one is processed.  The thread that owns a target column
-// hands the raw logit to the candidate's thread through LDS and patches the exact gradient code into its
-// own 8 output bytes before storing them, so every byte of the gradient is written once.
-constexpr int ROWREG_THREADS = 1024;
+// registers -- as table offsets, which both sweeps use -- so the logits are read from memory once.  Two
+// workgroups share a compute unit (at most 128 registers per thread): while one reduces, decides the
+// target columns and meets at its barriers, the other streams.  The thread that owns a target column hands
+// the raw logit to the candidate's thread through LDS and patches the exact gradient code into its own 8
+// output bytes before storing them, so every byte of the gradient is written once.
+constexpr int ROWREG_THREADS = 512;
 
 template <int MAXC>
-__global__ __launch_bounds__(ROWREG_THREADS) void ce_rows_reg_kernel(
+__global__ __launch_bounds__(ROWREG_THREADS, 4) void ce_rows_reg_kernel(
     const uint16_t* __restrict__ logits, CandArgs ca, float* __restrict__ losses, uint8_t* __restrict__ grad,
     const float* __restrict__ gtabE, const float* __restrict__ gtabD, Softcap sc, float coef) {
     __shared__ float tabE[TAB_ENTRIES];
@@ -244,13 +245,12 @@ __global__ __launch_bounds__(ROWREG_THREADS) void ce_rows_reg_kernel(
             w[s_] = (i < n8) ? *(const v4i*)(lrow + i * 8) : (v4i){0, 0, 0, 0};
         }
     };
-    v4i cur[MAXC], nxt[MAXC];
+    v4i cur[MAXC];
     int row = blockIdx.x;
     if (row < ca.M) load_row(row, cur);
     __syncthreads();
     for (; row < ca.M; row += gridDim.x) {
         const int next_row = row + gridDim.x;
-        if (next_row < ca.M) load_row(next_row, nxt);
         // candidate target columns: the owner publishes the raw logit
         int my_cand_slot[MAX_CAND], my_cand_pos[MAX_CAND];
 #pragma unroll
@@ -348,8 +348,7 @@ __global__ __launch_bounds__(ROWREG_THREADS) void ce_rows_reg_kernel(
                 *(v2i*)(grow + i * 8) = (v2i){(int)o[0], (int)o[1]};
             }
         }
-#pragma unroll
-        for (int s_ = 0; s_ < MAXC; ++s_) cur[s_] = nxt[s_];
+        if (next_row < ca.M) load_row(next_row, cur);
         __syncthreads();     // tl / fix / loss_term / red are reused by the next row
     }
 }
@@ -827,13 +826,16 @@ extern "C" int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, 
     CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, n_rows, n_cols};
     int grid = num_cus();
     if (grid <= 0) return fail(NGPT_EINVAL, "no HIP device");
-    if (n_cols <= 8 * 8 * ROWREG_THREADS) {    // a row fits the registers of one workgroup
-        if (grid > n_rows) grid = n_rows;
+    if (n_cols <= 16 * 8 * ROWREG_THREADS) {    // a row fits the registers of one workgroup
         const float coef = make_coef(A, C, grad_s, grad_scale);
-        if (n_cols <= 4 * 8 * ROWREG_THREADS)
-            ce_rows_reg_kernel<4><<<grid, ROWREG_THREADS, 0, st>>>((const uint16_t*)logits_bf16, ca, losses, (uint8_t*)grad_e5m2, tabE, tabD, sc, coef);
-        else
-            ce_rows_reg_kernel<8><<<grid, ROWREG_THREADS, 0, st>>>((const uint16_t*)logits_bf16, ca, losses, (uint8_t*)grad_e5m2, tabE, tabD, sc, coef);
+        grid *= 2;
+        if (grid > n_rows) grid = n_rows;
+        auto launch = [&](auto kernel) {
+            kernel<<<grid, ROWREG_THREADS, 0, st>>>((const uint16_t*)logits_bf16, ca, losses, (uint8_t*)grad_e5m2, tabE, tabD, sc, coef);
+        };
+        if (n_cols <= 4 * 8 * ROWREG_THREADS) launch(ce_rows_reg_kernel<4>);
+        else if (n_cols <= 8 * 8 * ROWREG_THREADS) launch(ce_rows_reg_kernel<8>);
+        else launch(ce_rows_reg_kernel<16>);
         return check_launch("ce_rows_reg_kernel");
     }
     grid *= 2;
