@@ -176,56 +176,83 @@ struct EpiDpre {
     uint16_t* out;          // dpre [C = tokens, R = hidden], row stride ld
     const uint16_t* post;   // same shape
     int64_t ld;
-    int R, C;               // R % 4 == 0
-    static constexpr int EXTRA_LDS = 0;
+    int R, C;               // R % 8 == 0
+    static constexpr int EXTRA_LDS = 32768;    // 4 KiB per wave
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
+    static constexpr int TILE_STORES = 16;
+    uint8_t* stage;
+    bool stored_all;
+    __device__ bool all_stores_issued() const { return stored_all; }
     __device__ void partial(bool) {}
-    __device__ void begin(int, int, uint8_t*) {}
+    __device__ void begin(int, int, uint8_t* extra) {
+        stage = extra + (threadIdx.x >> 6) * 4096;
+        stored_all = false;
+    }
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
     __device__ void job_begin(int) {}
     template <class Cfg>
     __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+    // A lane owns one token and four consecutive hidden units per register group, i.e. 8-byte pieces scattered
+    // over 32 rows of post / dpre per memory instruction: issued like that, the address unit spends one cycle
+    // per cache line and the epilogue takes longer than the GEMM.  Instead every 32-token x 64-hidden block
+    // (4 KiB) goes through the wave's LDS region: read from post as whole 128-byte lines (16 bytes per lane),
+    // picked up and replaced piece by piece, and written to dpre as whole lines again.  16-byte chunks are
+    // XOR-swizzled by the row.  (LDS operations of one wave execute in order, so no waits are needed between
+    // the steps; the square root is the hardware's v_sqrt_f32, 1 ulp: its result is multiplied and rounded to
+    // bf16, and the reference's kernel uses an approximate square root too, triton_kernels.py:475.)
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
-                         uint8_t*, int) {
-        const int64_t tile_off = (int64_t)c0 * ld + r0;
-        uint16_t* origin = out + tile_off;
-        const uint16_t* porigin = post + tile_off;
-        const uint32_t lane_off = (uint32_t)co.col_base * (uint32_t)ld + (uint32_t)co.row_base;
-        const int rlim = R - r0 - co.row_base, clim = C - c0 - co.col_base;
+                         uint8_t*, int lane) {
+        static_assert(Cfg::TM == 2 && Cfg::TN == 4 && Cfg::NWAVES * 4096 <= EXTRA_LDS, "64 x 128 wave tiles, 4 KiB of staging each");
+        const int h = lane >> 5, j = lane & 31;
         const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
-        v2i pp[Cfg::TM][Cfg::TN][4];
+        stored_all = full;
+        const int rd_row = lane >> 3, rd_chunk = lane & 7;
+        const int n = r0 + co.wave_row0 + rd_chunk * 8;          // this lane's 8 hidden units in the line-wise steps
+        v4i line[Cfg::TN][4];
+        auto load_block = [&](int tn) {
 #pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < Cfg::TN; ++tn)
-#pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    const int dr = tm * 32 + 8 * a, dc = tn * 32;
-                    const bool ok = full || (dr < rlim && dc < clim);
-                    pp[tm][tn][a] = ok ? *(const v2i*)(porigin + ((int64_t)dc * ld + dr) + lane_off) : (v2i){0, 0};
-                }
-#pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < Cfg::TN; ++tn) {
-#pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    const int dr = tm * 32 + 8 * a, dc = tn * 32;
-                    const bool ok = full || (dr < rlim && dc < clim);
-                    const uint32_t p01 = (uint32_t)pp[tm][tn][a].x, p23 = (uint32_t)pp[tm][tn][a].y;
-                    const v16f& c = acc[tm][tn];
-                    uint32_t c01 = cvt_pk_bf16(c[4 * a], c[4 * a + 1]), c23 = cvt_pk_bf16(c[4 * a + 2], c[4 * a + 3]);   // bf16(acc)
-                    float d0 = 2.0f * bf16_bits_to_f32(c01 & 0xffffu) * __fsqrt_rn(bf16_bits_to_f32(p01 & 0xffffu));
-                    float d1 = 2.0f * bf16_bits_to_f32(c01 >> 16) * __fsqrt_rn(bf16_bits_to_f32(p01 >> 16));
-                    float d2 = 2.0f * bf16_bits_to_f32(c23 & 0xffffu) * __fsqrt_rn(bf16_bits_to_f32(p23 & 0xffffu));
-                    float d3 = 2.0f * bf16_bits_to_f32(c23 >> 16) * __fsqrt_rn(bf16_bits_to_f32(p23 >> 16));
-                    if (ok) *(v2i*)(origin + ((int64_t)dc * ld + dr) + lane_off) = (v2i){(int)cvt_pk_bf16(d0, d1), (int)cvt_pk_bf16(d2, d3)};
-                }
-                __builtin_amdgcn_sched_barrier(0);
+            for (int k = 0; k < 4; ++k) {
+                const int m = c0 + co.wave_col0 + tn * 32 + 8 * k + rd_row;
+                line[tn][k] = (full || (m < C && n < R)) ? *(const v4i*)(post + (int64_t)m * ld + n) : (v4i){0, 0, 0, 0};
             }
+        };
+        load_block(0);
+        load_block(1);
+#pragma unroll
+        for (int tn = 0; tn < Cfg::TN; ++tn) {
+            if (tn + 2 < Cfg::TN) load_block(tn + 2);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int row = 8 * k + rd_row;
+                *(v4i*)(stage + row * 128 + ((rd_chunk ^ (row & 7)) << 4)) = line[tn][k];
+            }
+#pragma unroll
+            for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    uint8_t* at = stage + j * 128 + (((tm * 4 + g) ^ (j & 7)) << 4) + 8 * h;
+                    const v2i p = *(const v2i*)at;
+                    const uint32_t p01 = (uint32_t)p.x, p23 = (uint32_t)p.y;
+                    const v16f& c = acc[tm][tn];
+                    const uint32_t c01 = cvt_pk_bf16(c[4 * g], c[4 * g + 1]), c23 = cvt_pk_bf16(c[4 * g + 2], c[4 * g + 3]);   // bf16(acc)
+                    const float d0 = 2.0f * bf16_bits_to_f32(c01 & 0xffffu) * __builtin_amdgcn_sqrtf(bf16_bits_to_f32(p01 & 0xffffu));
+                    const float d1 = 2.0f * bf16_bits_to_f32(c01 >> 16) * __builtin_amdgcn_sqrtf(bf16_bits_to_f32(p01 >> 16));
+                    const float d2 = 2.0f * bf16_bits_to_f32(c23 & 0xffffu) * __builtin_amdgcn_sqrtf(bf16_bits_to_f32(p23 & 0xffffu));
+                    const float d3 = 2.0f * bf16_bits_to_f32(c23 >> 16) * __builtin_amdgcn_sqrtf(bf16_bits_to_f32(p23 >> 16));
+                    *(v2i*)at = (v2i){(int)cvt_pk_bf16(d0, d1), (int)cvt_pk_bf16(d2, d3)};
+                }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int row = 8 * k + rd_row;
+                const v4i v = *(const v4i*)(stage + row * 128 + ((rd_chunk ^ (row & 7)) << 4));
+                const int m = c0 + co.wave_col0 + tn * 32 + row;
+                if (full || (m < C && n < R)) *(v4i*)(out + (int64_t)m * ld + n) = v;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 };
 

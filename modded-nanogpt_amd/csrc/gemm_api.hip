@@ -329,7 +329,7 @@ extern "C" int ngpt_fc_relu2_bwd_dpre(const void* dy_bf16, const void* w2_bf16, 
                                       void* dpre_bf16, void* stream) {
     if (!dy_bf16 || !w2_bf16 || !post_bf16 || !dpre_bf16) return fail(NGPT_EINVAL, "ngpt_fc_relu2_bwd_dpre: null pointer");
     if (M <= 0 || H <= 0 || D <= 0) return fail(NGPT_EINVAL, "ngpt_fc_relu2_bwd_dpre: empty problem M=%d H=%d D=%d", M, H, D);
-    if (D % 64 || H % 4) return fail(NGPT_EALIGN, "ngpt_fc_relu2_bwd_dpre: need D %% 64 == 0 and H %% 4 == 0 (D=%d H=%d)", D, H);
+    if (D % 64 || H % 8) return fail(NGPT_EALIGN, "ngpt_fc_relu2_bwd_dpre: need D %% 64 == 0 and H %% 8 == 0 (D=%d H=%d)", D, H);
     // bf16 operands: the loader works in bytes, so the contraction length and row strides are 2 * D.
     // Transposed product (tile rows = hidden units, tile columns = tokens), see EpiDpre.
     GemmOperands g{(const uint8_t*)w2_bf16, (const uint8_t*)dy_bf16, 2 * (int64_t)D, 2 * (int64_t)D, H, M, 2 * D, 1, 0};

@@ -528,6 +528,13 @@ struct EpiTileStores : std::integral_constant<int, 0> {};
 template <class E>
 struct EpiTileStores<E, std::void_t<decltype(E::TILE_STORES)>> : std::integral_constant<int, E::TILE_STORES> {};
 
+// An epilogue whose number of stores depends on the tile (masked edges) has `bool all_stores_issued() const`:
+// the relaxed wait after its tile is taken only if it returns true.
+template <class E, class = void>
+struct EpiReportsStores : std::false_type {};
+template <class E>
+struct EpiReportsStores<E, std::void_t<decltype(std::declval<const E&>().all_stores_issued())>> : std::true_type {};
+
 // Epilogues with `static constexpr bool HAS_TILE_BEGIN = true` get tile_begin<Cfg>(r0, c0) before the
 // k-loop of every job; LDS it fills (also through direct-to-LDS loads) is visible in tile().
 template <class E, class = void>
@@ -629,7 +636,8 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         // relaxed wait: only behind an epilogue that stored (not the first job), with a later k-step of
         // the same job to wait for tile_begin's load, and only if that epilogue's refill was not deferred
         constexpr bool kNeverDefers = !Epi::NEEDS_SCRATCH && !Epi::JOB_END_NEEDS_SCRATCH;
-        const bool relax = kNeverDefers && EpiTileStores<Epi>::value > 0 && !first_job && kt1 - kt0 >= 2;
+        bool relax = kNeverDefers && EpiTileStores<Epi>::value > 0 && !first_job && kt1 - kt0 >= 2;
+        if constexpr (EpiReportsStores<Epi>::value) relax = relax && epi.all_stores_issued();
         if (relax) kstep(std::true_type{}, std::true_type{}, kt0 + 1 == kt1);
         else kstep(std::true_type{}, std::false_type{}, kt0 + 1 == kt1);
         first_job = false;
