@@ -323,6 +323,73 @@ struct EpiStoreF32 {
 using EpiDiscard = EpiDiscardT<false>;
 using EpiDiscardAblate = EpiDiscardT<true>;    // honours GemmOperands::ablate, at the price of its branches
 
+// post = bf16(max(bf16(acc * dequant), 0)^2) for a GEMM that runs TRANSPOSED (tile rows = hidden units, tile
+// columns = tokens, post [tokens, hidden] row-major): a lane's four consecutive accumulator registers are
+// four consecutive hidden units of one token.  Every 32-token x 64-hidden block (4 KiB) is collected in the
+// wave's LDS region and written as whole 128-byte lines, 16 bytes per lane (see EpiDpre).  R % 8 == 0.
+struct EpiRelu2Lines {
+    uint16_t* post;
+    int64_t ld;
+    const float* dequant;        // 1-element device tensor
+    int R, C;                    // R = hidden units (tile rows), C = tokens (tile columns)
+    static constexpr int EXTRA_LDS = 32768;
+    static constexpr bool NEEDS_SCRATCH = false;
+    static constexpr bool JOB_END_NEEDS_SCRATCH = false;
+    static constexpr int TILE_STORES = 16;
+    float scale;
+    uint8_t* stage;
+    bool stored_all;
+    __device__ bool all_stores_issued() const { return stored_all; }
+    __device__ void partial(bool) {}
+    __device__ void begin(int, int, uint8_t* extra) {
+        scale = *dequant;
+        stage = extra + (threadIdx.x >> 6) * 4096;
+        stored_all = false;
+    }
+    __device__ void end(uint8_t*, int, int) {}
+    template <class Cfg>
+    __device__ void job_begin(int) {}
+    template <class Cfg>
+    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co, uint8_t*, int lane) {
+        static_assert(Cfg::TM == 2 && Cfg::TN == 4 && Cfg::NWAVES * 4096 <= EXTRA_LDS, "64 x 128 wave tiles, 4 KiB of staging each");
+        const int h = lane >> 5, j = lane & 31;
+        const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
+        stored_all = full;
+        const int rd_row = lane >> 3, rd_chunk = lane & 7;
+        const int n = r0 + co.wave_row0 + rd_chunk * 8;
+        // address = wave-uniform pointer (tile origin + the block's and line group's fixed position) + ONE per-lane offset
+        uint16_t* origin = post + ((int64_t)c0 * ld + r0);
+        const uint32_t lane_off = (uint32_t)(co.wave_col0 + rd_row) * (uint32_t)ld + (uint32_t)(co.wave_row0 + rd_chunk * 8);
+        auto relu2 = [&](float a0, float a1) {
+            const uint32_t pre = cvt_pk_bf16(a0 * scale, a1 * scale);
+            const float c0f = fmaxf(__uint_as_float(pre << 16), 0.0f), c1f = fmaxf(__uint_as_float(pre & 0xffff0000u), 0.0f);
+            return (int)cvt_pk_bf16(c0f * c0f, c1f * c1f);
+        };
+#pragma unroll
+        for (int tn = 0; tn < Cfg::TN; ++tn) {
+#pragma unroll
+            for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const v16f& a = acc[tm][tn];
+                    *(v2i*)(stage + j * 128 + (((tm * 4 + g) ^ (j & 7)) << 4) + 8 * h) =
+                        (v2i){relu2(a[4 * g], a[4 * g + 1]), relu2(a[4 * g + 2], a[4 * g + 3])};
+                    if (g & 1) __builtin_amdgcn_sched_barrier(0);   // keep the arithmetic next to its LDS write (registers)
+                }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int row = 8 * k + rd_row;
+                const v4i v = *(const v4i*)(stage + row * 128 + ((rd_chunk ^ (row & 7)) << 4));
+                const int m = c0 + co.wave_col0 + tn * 32 + row;
+                if (full || (m < C && n < R)) *(v4i*)(origin + (int64_t)(tn * 32 + 8 * k) * ld + lane_off) = v;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+};
+
 // post = bf16(max(bf16(acc * *dequant), 0)^2); optionally post_f8 = e4m3(min(post / act_scale, 448))
 // and a per-workgroup running max of post written to partial_amax[bid].
 template <bool EMIT>      // EMIT: also the e4m3 copy of post and the per-workgroup maxima

@@ -365,6 +365,12 @@ extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float
         // one partial-amax slot per persistent workgroup
         return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(g, epi, (hipStream_t)stream, n_partials);
     }
+    if (N % 8 == 0) {
+        // without the e4m3 copy: transposed product (tile rows = hidden units, tile columns = tokens), whole-line stores
+        GemmOperands gt{(const uint8_t*)w_f8, (const uint8_t*)x_f8, K, K, N, M, K, 1, 0};
+        EpiRelu2Lines epi{(uint16_t*)post_bf16, N, dequant, N, M};
+        return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(gt, epi, (hipStream_t)stream, 0);
+    }
     EpiRelu2T<false> epi{};
     fill(epi);
     return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(g, epi, (hipStream_t)stream, 0);
