@@ -140,7 +140,7 @@ class FusedLinearReLUSquareFunction(torch.autograd.Function):
             # 1-element device tensors; their product is taken on the device, no host sync.
             w2_dh = W2_f8.T
             assert w2_dh.is_contiguous()
-            x3 = ops.gemm_fp8_tn(post_f8, w2_dh, 1.0, out_dtype=torch.float32)
+            x3 = ops.gemm_fp8_tn_op(post_f8, w2_dh, 1.0, True)
             x3 = (x3 * (activation_scale * W2_scale)).to(torch.bfloat16)
         else:
             x3 = post @ W2

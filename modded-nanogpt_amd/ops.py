@@ -479,3 +479,16 @@ def gemm_fp8_tn(a: Tensor, b: Tensor, scale: float, out_dtype=torch.bfloat16, ou
                                             R, Cn, K, scale, _p(out), out.stride(0), kind, _stream(a)),
                "ngpt_gemm_fp8_tn")
     return out
+
+
+@torch.library.custom_op("nanogpt::gemm_fp8_tn", mutates_args=())
+def gemm_fp8_tn_op(a: Tensor, b: Tensor, scale: float, out_f32: bool) -> Tensor:
+    """`gemm_fp8_tn` as a registered operator, for callers that run under `torch.compile(fullgraph=True)`
+    (the FP8 down projection inside `FusedLinearReLUSquareFunction`, reference triton_kernels.py:706-713)."""
+    return gemm_fp8_tn(a, b, scale, out_dtype=torch.float32 if out_f32 else torch.bfloat16)
+
+
+@gemm_fp8_tn_op.register_fake
+def _(a, b, scale, out_f32):
+    assert a.ndim == 2 and b.ndim == 2 and a.shape[1] == b.shape[1]
+    return a.new_empty((a.shape[0], b.shape[0]), dtype=torch.float32 if out_f32 else torch.bfloat16)

@@ -492,3 +492,48 @@ def test_quant_up_weights(amd, oracle, L, H, D):
     ref_f8, ref_s = oracle.quantize_up_weights(w)
     assert torch.equal(scales.cpu(), ref_s)
     assert torch.equal(w_f8.cpu().view(torch.uint8), ref_f8.view(torch.uint8))
+
+
+def test_path_traces_under_torch_compile_fullgraph(amd, oracle):
+    """The reference runs its model under torch.compile(dynamic=False, fullgraph=True) (train_gpt.py:2260):
+    dynamo, fake tensors and AOT autograd must get through every operator of the path without a graph
+    break, forward and backward, and give what eager calls of the same kernels give."""
+    M, D, H, V = 512, 256, 1024, 1024
+    g = torch.Generator().manual_seed(71)
+    x0 = dev(torch.randn(M, D, generator=g).bfloat16())
+    w_fc = dev((torch.randn(H, D, generator=g) / math.sqrt(D)).bfloat16())
+    w_proj_t = dev((torch.randn(H, D, generator=g) / math.sqrt(H)).bfloat16())
+    w_head = dev((torch.randn(D, V, generator=g) / math.sqrt(D)).bfloat16())      # (in, out) as at the reference's HEAD
+    w_mm = dev((torch.randn(D, D, generator=g) / math.sqrt(D)).bfloat16())
+    targets = dev(torch.randint(0, V, (M,), generator=g))
+    w_f8, up_scales = torch.ops.nanogpt.quant_up_weights(w_fc[None].contiguous())
+    w2_scale = (w_proj_t.float().abs().max() / 448).reshape(1)
+    w2_f8_dh = (w_proj_t.float() / w2_scale).T.contiguous().to(E4M3)               # [D, H]
+    act_scale = torch.full((1,), 0.02, device="cuda")
+    x_s, w_s, grad_s = 100 / 448, 1.6 / 448, 0.75 / 448
+
+    def step(x, w_mm, w_fc, w_proj_t, w_head, partial, fp8_down):
+        h = torch.ops.nanogpt.mm(x, w_mm, x_s=1.0, w_s=1 / 32, grad_s=grad_s)[0]
+        normed, x_f8, dequant = torch.ops.nanogpt.mlp_input_quant(h, up_scales[0:1])
+        if fp8_down:
+            h = h + amd.ReLUSqrdMLP(normed, w_fc, w_proj_t, w_f8[0], dequant, x_f8, w2_f8_dh.T, w2_scale, act_scale, partial)
+        else:
+            h = h + amd.ReLUSqrdMLP(normed, w_fc, w_proj_t, w_f8[0], dequant, x_f8)
+        losses = amd.FusedSoftcappedCrossEntropy.apply(h, targets, None, None, None, w_head, x_s, w_s, grad_s, 1.0)
+        return losses.sum()
+
+    for fp8_down in (False, True):
+        results = []
+        for fn in (step, torch.compile(step, fullgraph=True, dynamic=False, backend="aot_eager")):
+            leaves = [t.clone().requires_grad_(True) for t in (x0, w_mm, w_fc, w_proj_t, w_head)]
+            partial = torch.zeros(256, device="cuda")
+            loss = fn(*leaves, partial, fp8_down)
+            loss.backward()
+            results.append((loss.detach(), [t.grad for t in leaves], partial))
+        (l0, g0, p0), (l1, g1, p1) = results
+        assert torch.isfinite(l0) and torch.equal(l0, l1)
+        for a, b in zip(g0, g1):
+            assert a is not None and b is not None and a.dtype == b.dtype and a.shape == b.shape
+            # same kernels, same order; only the fp32 atomics of the split tiles may reorder
+            assert rel_err(b.float(), a.float()) <= 1e-5
+        assert torch.equal(p0, p1) and (float(p0.max()) > 0) == fp8_down
