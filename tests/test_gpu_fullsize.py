@@ -137,6 +137,56 @@ def test_config2_mlp_forward_full_size(amd, oracle):
     assert _rel(out.cpu()[0, rows], out_ref) <= GEMM_TOL
 
 
+def test_config4_mlp_backward_full_size(amd, oracle):
+    """FP8 MLP forward + bf16 backward at M = 49152 (one layer of benchmark configuration 4).  dpre and dx are
+    row-local: a row sample against the oracle.  The weight gradients contract over all tokens: against an
+    fp32 product of the kernel's own post / dpre on the GPU (the plain reference for a floating-point
+    contraction), and as the sum of the gradients of the two token halves (additivity, which also
+    exercises the sliced contraction at a second size)."""
+    g = torch.Generator().manual_seed(4)
+    M, D, H = 49152, 768, 3072
+    d = "cuda"
+    x_raw = torch.randn(M, D, generator=g).bfloat16()
+    w_fc = (torch.randn(H, D, generator=g) / math.sqrt(D)).bfloat16()
+    w_proj_t = (torch.randn(D, H, generator=g) / math.sqrt(H)).bfloat16().T.contiguous()
+    dy = (torch.randn(M, D, generator=g) * 1e-3).bfloat16()
+    w_f8, scales = torch.ops.nanogpt.quant_up_weights(w_fc[None].to(d))
+    normed_all, x_f8_all, dequant = torch.ops.nanogpt.mlp_input_quant(x_raw.to(d), scales[0:1])
+
+    def run(rows):   # forward + backward on a slice of the tokens, same quantised input as the whole
+        normed = normed_all[rows].detach().clone().requires_grad_(True)
+        x_f8 = x_f8_all[rows].contiguous()
+        w1 = w_fc.to(d).requires_grad_(True)
+        w2 = w_proj_t.to(d).requires_grad_(True)
+        out = amd.ReLUSqrdMLP(normed[None], w1, w2, w_f8[0], dequant, x_f8[None])
+        out.backward(dy[rows].to(d)[None])
+        post = torch.ops.nanogpt.fc_relu2_fwd(x_f8, w_f8[0], dequant)
+        return normed, post, normed.grad, w1.grad, w2.grad
+
+    everything = slice(0, M)
+    normed, post, dx, dw1, dw2 = run(everything)
+    dyd = dy.to(d)
+    dpre = torch.ops.nanogpt.fc_relu2_bwd_dpre(dyd, w_proj_t.to(d), post)
+    torch.cuda.synchronize()
+    # row-local parts on a sample of rows
+    rows = torch.cat([torch.arange(0, M, 1531), torch.arange(M - 16, M)]).unique()
+    dpre_ref = oracle.fc_relu2_bwd_dpre(dy[rows], w_proj_t, post.cpu()[rows])
+    assert _rel(dpre.cpu()[rows], dpre_ref) <= GEMM_TOL
+    dx_ref = (dpre_ref.float() @ w_fc.float()).bfloat16()
+    assert _rel(dx.cpu()[rows], dx_ref) <= GEMM_TOL
+    # weight gradients against an fp32 contraction of the same operands
+    dw2_ref = post.float().T @ dyd.float()
+    dw1_ref = dpre.float().T @ normed.detach().float()
+    assert dw1.shape == (H, D) and dw2.shape == (H, D)
+    assert _rel(dw2, dw2_ref) <= GEMM_TOL and _rel(dw1, dw1_ref) <= GEMM_TOL
+    # additivity over the token halves (each half's bf16 result carries its own rounding)
+    del dw1_ref, dw2_ref
+    _, _, _, dw1_a, dw2_a = run(slice(0, M // 2))
+    _, _, _, dw1_b, dw2_b = run(slice(M // 2, M))
+    assert _rel(dw2_a.float() + dw2_b.float(), dw2.float()) <= GEMM_TOL
+    assert _rel(dw1_a.float() + dw1_b.float(), dw1.float()) <= GEMM_TOL
+
+
 @pytest.mark.parametrize("layout", ["out_in", "in_out"])
 def test_mm_forward_backward_lm_head_shape(amd, oracle, layout):
     """nanogpt::mm / mm_t forward + backward at an lm_head-sized problem (N = 50304): row / column subsets
