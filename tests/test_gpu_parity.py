@@ -166,6 +166,28 @@ def test_mm_backward_and_autograd(amd, oracle, M, N, K):
     assert_close_gemm(wg.grad, dw_ref)
 
 
+@pytest.mark.parametrize("rem", [1, 70, 100, 200])
+def test_mm_backward_remainder_tiles_split_along_the_contraction(amd, rem):
+    """dx of mm_backward with 256 + rem output tiles on a 256-workgroup grid: the remainder tiles are cut
+    into 4, 3, 2 or 1 jobs along the contraction and meet in fp32; dW here is 16 tiles cut 16 ways.
+    Reference: the fp32 product of the same fp8 operands on the GPU."""
+    M, N, K = 256 * (256 + rem), 4096, 256
+    x_s, w_s, grad_s = 100 / 448, 1.6 / 448, 0.75 / 448
+    gen = torch.Generator(device="cuda").manual_seed(100 + rem)
+    x_f8 = torch.randn(M, K, device="cuda", generator=gen).mul_(4).to(E4M3)
+    w_f8 = torch.randn(N, K, device="cuda", generator=gen).mul_(4).to(E4M3)
+    go = torch.randn(M, N, device="cuda", generator=gen).mul_(1e-3).bfloat16()
+    dx, dw = torch.ops.nanogpt.mm_backward(go, x_f8, w_f8, x_s, w_s, grad_s)
+    g_f8 = amd.quant_fp8(go, grad_s, E5M2).float()
+    dx_ref = (g_f8 @ w_f8.float()) * (grad_s * w_s)
+    dw_ref = (g_f8.T @ x_f8.float()) * (x_s * grad_s)
+    assert rel_err(dx.float(), dx_ref) <= 5e-3          # bf16 output
+    assert rel_err(dw.float(), dw_ref) <= 1e-4          # fp32 output, fp32 partial sums
+    # no tile left out or written twice: the row blocks of dx compare equally well everywhere
+    blocks = (dx.float() - dx_ref).view(-1, 256, K).norm(dim=(1, 2)) / dx_ref.view(-1, 256, K).norm(dim=(1, 2))
+    assert float(blocks.max()) <= 5e-3
+
+
 def test_mm_t_matches_mm(amd, oracle):
     x, w, _, _ = oracle.make_cfg1(seed=5, M=512, N=640, K=256)
     x_s, w_s, grad_s = 100 / 448, 1.6 / 448, 0.75 / 448
