@@ -112,6 +112,26 @@ def secondary(args, amd, oracle) -> int:
         desc = ("config 4 (one layer): " if bwd else "config 2: ") + "norm + quantise + FP8 c_fc with ReLU^2 + bf16 c_proj" + \
                (", forward+backward" if bwd else ", forward") + ", M=49152 D=768 H=3072"
         tokens = Mm
+    elif wl == "mlp_cfg4":
+        # configuration 4 as worded: twelve layers with their own weights, forward+backward, back to back on one stream
+        Mm, D, H, L = 49152, 768, 3072, 12
+        xr = (torch.randn(Mm, D, generator=g) * 2).bfloat16().to(dev).requires_grad_(True)
+        w_fc = [(torch.randn(H, D, generator=g) / math.sqrt(D)).bfloat16().to(dev).requires_grad_(True) for _ in range(L)]
+        w_pt = [(torch.randn(D, H, generator=g) / math.sqrt(H)).bfloat16().T.contiguous().to(dev).requires_grad_(True) for _ in range(L)]
+        dy = (torch.randn(1, Mm, D, generator=g) * 1e-3).bfloat16().to(dev)
+        w_f8, scales = torch.ops.nanogpt.quant_up_weights(torch.stack([w.detach() for w in w_fc]))
+
+        def step():
+            xr.grad = None
+            for l in range(L):
+                w_fc[l].grad = w_pt[l].grad = None
+                normed, x_f8, dequant = torch.ops.nanogpt.mlp_input_quant(xr, scales[l:l + 1])
+                out = amd.ReLUSqrdMLP(normed[None], w_fc[l], w_pt[l], w_f8[l], dequant, x_f8[None])
+                out.backward(dy)
+            return out
+        flops = 12.0 * Mm * D * H * L
+        desc = "config 4: 12 layers (own weights) of norm + quantise + FP8 c_fc with ReLU^2 + bf16 c_proj, forward+backward, M=49152 D=768 H=3072"
+        tokens = Mm
     elif wl == "cfg5":
         # medium-track shapes: FP8 lm_head + softcapped CE forward+backward and one FP8 MLP layer forward+backward per step
         Mm, D, H, Vv = 65536, 1024, 4096, 50304
@@ -193,7 +213,7 @@ def secondary(args, amd, oracle) -> int:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="lmhead_ce",
-                    help="lmhead_ce (default, the headline configuration 3) | mm_cfg1 | mm_lmhead | mlp_fwd | mlp_fwd_bwd | ce_logits | cfg5")
+                    help="lmhead_ce (default, the headline configuration 3) | mm_cfg1 | mm_lmhead | mlp_fwd | mlp_fwd_bwd | mlp_cfg4 | ce_logits | cfg5")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
