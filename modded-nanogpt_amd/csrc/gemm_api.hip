@@ -107,14 +107,18 @@ static BalancePlan plan_balance(int R, int C, int K) {
 
 // Zero (MODE 0) or convert to bf16 (MODE 1) the 256 x 256 tiles number [first, first + gridDim.x) of the
 // walk order, i.e. exactly the tiles that the balanced walk splits.
+constexpr int kRemSlices = 8;
+static_assert(MainCfg::BM % kRemSlices == 0, "row slices of a tile");
 template <int MODE>
 __global__ void rem_tiles_kernel(float* part32, int64_t ld32, uint16_t* out, int64_t ldo, int R, int C, int first) {
     TileOrder order(R, C, MainCfg::BM, MainCfg::BN);
     int tr, tc;
     order.coords(first + blockIdx.x, tr, tc);
-    const int r0 = tr * MainCfg::BM, c0 = tc * MainCfg::BN;
+    // blockIdx.y: which slice of the tile's rows (a few dozen tiles alone would leave most of the chip idle)
+    const int rows = MainCfg::BM / gridDim.y;
+    const int r0 = tr * MainCfg::BM + blockIdx.y * rows, c0 = tc * MainCfg::BN;
     const int cols4 = MainCfg::BN / 4;
-    for (int i = threadIdx.x; i < MainCfg::BM * cols4; i += blockDim.x) {
+    for (int i = threadIdx.x; i < rows * cols4; i += blockDim.x) {
         int r = r0 + i / cols4, c = c0 + (i % cols4) * 4;
         if (r >= R || c >= C) continue;          // C % 4 == 0 is checked by the caller
         float* p = part32 + (int64_t)r * ld32 + c;
@@ -138,11 +142,11 @@ int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb
     BalancePlan p = plan_balance(R, C, K);
     if (p.splits > 1 && !part32) return fail(NGPT_EINVAL, "gemm_balanced_bf16: split tiles need the fp32 scratch matrix");
     ProfileScope prof(g_gemm_slot, st);
-    if (p.splits > 1) rem_tiles_kernel<0><<<p.rem, 256, 0, st>>>(part32, C, nullptr, 0, R, C, p.full);
+    if (p.splits > 1) rem_tiles_kernel<0><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(part32, C, nullptr, 0, R, C, p.full);
     GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full, a_rows_pad};
     EpiStoreBf16 epi{(uint16_t*)out_bf16, ldc, scale, R, C, part32, C, false};
     if (int e = launch_gemm<MainCfg>(g, fa, fb, epi, st)) return e;
-    if (p.splits > 1) rem_tiles_kernel<1><<<p.rem, 256, 0, st>>>(part32, C, (uint16_t*)out_bf16, ldc, R, C, p.full);
+    if (p.splits > 1) rem_tiles_kernel<1><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(part32, C, (uint16_t*)out_bf16, ldc, R, C, p.full);
     return check_launch("gemm_balanced_bf16");
 }
 
@@ -159,7 +163,7 @@ int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb,
         EpiStoreF32<true> epi{out, ldc, scale, R, C, false};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
-    if (p.splits > 1) rem_tiles_kernel<0><<<p.rem, 256, 0, st>>>(out, ldc, nullptr, 0, R, C, p.full);
+    if (p.splits > 1) rem_tiles_kernel<0><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(out, ldc, nullptr, 0, R, C, p.full);
     EpiStoreF32<false> epi{out, ldc, scale, R, C, false};
     return launch_gemm<MainCfg>(g, fa, fb, epi, st);
 }
