@@ -97,6 +97,37 @@ def test_config5_shape(amd, oracle):
     _check_dw_columns(oracle, t, sc, cols, lse, x_f8, w_f8, dw)
 
 
+def test_mtp_and_prefix_targets_at_training_shape(amd, oracle):
+    """Stage-1 shape of the reference's schedule (train_gpt.py:1980-1983): M = 16384 tokens, three predicted
+    tokens per position with weights, prefix targets, (in, out) weight as at HEAD, through the autograd function.
+    Contiguous row blocks against the oracle; inside a block the last two rows look ahead past the block's
+    end, so only the final block (the true end of the batch, where the look-ahead stops) is compared whole."""
+    g = torch.Generator().manual_seed(16)
+    M, K, V = 16384, 768, 50304
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w_kv = (torch.randn(V, K, generator=g) / math.sqrt(K)).bfloat16().T.contiguous()      # (in, out)
+    t = torch.randint(0, 50257, (M,), generator=g)
+    t[5] = -100                                                                            # an ignored position
+    mtp = torch.tensor([1.0, 0.5, 0.25])
+    pt = torch.where(torch.rand(M, generator=g) < 0.3, torch.randint(0, 50257, (M,), generator=g), torch.full((M,), -1))
+    pw = torch.tensor([0.4])
+    x_s, w_s, grad_s, grad_scale = 100 / 448, 1.6 / 448, 0.75 / 448, 2.0
+    d = "cuda"
+    xd, wd = x.to(d).requires_grad_(True), w_kv.to(d).requires_grad_(True)
+    losses = amd.FusedSoftcappedCrossEntropy.apply(xd, t.to(d), mtp.to(d), pt.to(d), pw.to(d), wd, x_s, w_s, grad_s, grad_scale)
+    losses.sum().backward()
+    torch.cuda.synchronize()
+    assert wd.grad.shape == (K, V) and xd.grad.dtype == torch.bfloat16     # (autograd casts the fp32 dW to the leaf's dtype)
+    n_ahead = mtp.numel() - 1
+    for lo, hi in ((0, 96), (8100, 8292), (M - 96, M)):
+        rows = slice(lo, hi)
+        l_ref, ctx = oracle.lm_head_ce_fwd(x[rows], t[rows], mtp, pt[rows], pw, w_kv, x_s, w_s, grad_s, grad_scale)
+        dx_ref, _ = oracle.lm_head_ce_bwd(ctx)
+        keep = (hi - lo) if hi == M else (hi - lo - n_ahead)
+        assert (losses.detach().cpu()[rows][:keep] - l_ref[:keep]).abs().max().item() <= LOSS_TOL
+        assert _rel(xd.grad.cpu()[rows][:keep], dx_ref[:keep]) <= GEMM_TOL
+
+
 def test_two_passes(amd, oracle):
     """More tokens than one pass of the backward holds (65536): dW accumulates over the passes."""
     g = torch.Generator().manual_seed(7)
