@@ -177,7 +177,7 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
         n_rows = x.shape[0]
         dev = x.device
         if mtp_weights is None:
-            mtp_weights = torch.tensor([1.0], device=dev, dtype=torch.float32)
+            mtp_weights = torch.ones(1, device=dev, dtype=torch.float32)   # a fill kernel, not a host copy: legal under graph capture
         mtp_weights = mtp_weights.to(torch.float32).contiguous()
         targets = targets.contiguous()
         if prefix_targets is None:

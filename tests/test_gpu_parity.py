@@ -559,3 +559,51 @@ def test_path_traces_under_torch_compile_fullgraph(amd, oracle):
             # same kernels, same order; only the fp32 atomics of the split tiles may reorder
             assert rel_err(b.float(), a.float()) <= 1e-5
         assert torch.equal(p0, p1) and (float(p0.max()) > 0) == fp8_down
+
+
+def test_path_replays_from_a_hip_graph(amd):
+    """Launch-bound callers capture the step in a HIP graph: the library neither allocates, nor synchronises, nor
+    clears memory through the runtime, so a captured step (mm forward+backward, the MLP function, the fused CE,
+    all through autograd) must replay correctly.  Replayed three times on new inputs, with eager work and
+    synchronisations in between, each replay against the eager result for the same inputs."""
+    M, D, H, V = 512, 256, 1024, 2048
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    rnd = lambda *s, scale=1.0: (torch.randn(*s, device="cuda", generator=gen) * scale).bfloat16()
+    x_in = rnd(M, D)
+    w_mm, w_fc, w_pt, w_head = rnd(D, D, scale=D ** -0.5), rnd(H, D, scale=D ** -0.5), rnd(H, D, scale=H ** -0.5), rnd(D, V, scale=D ** -0.5)
+    targets = torch.randint(0, V, (M,), device="cuda", generator=gen)
+    w_f8, up_scales = torch.ops.nanogpt.quant_up_weights(w_fc[None].contiguous())
+    x_s, w_s, grad_s = 100 / 448, 1.6 / 448, 0.75 / 448
+    leaves = [t.clone().requires_grad_(True) for t in (w_mm, w_fc, w_pt, w_head)]
+
+    def step(x):
+        for t in leaves:
+            t.grad = None
+        x = x.detach().requires_grad_(True)
+        h = torch.ops.nanogpt.mm(x, leaves[0], x_s=1.0, w_s=1 / 32, grad_s=grad_s)[0]
+        normed, x_f8, dequant = torch.ops.nanogpt.mlp_input_quant(h, up_scales[0:1])
+        h = h + amd.ReLUSqrdMLP(normed, leaves[1], leaves[2], w_f8[0], dequant, x_f8)
+        losses = amd.FusedSoftcappedCrossEntropy.apply(h, targets, None, None, None, leaves[3], x_s, w_s, grad_s, 1.0)
+        loss = losses.sum()
+        loss.backward()
+        return [loss.detach().clone(), x.grad.clone()] + [t.grad.clone() for t in leaves]
+
+    side = torch.cuda.Stream()                 # default priority
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(x_in)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step(x_in)
+    for rep in range(3):
+        x_in.copy_(rnd(M, D))
+        want = step(x_in)                      # eager, same buffers as the graph reads
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip(captured, want):
+            assert torch.isfinite(got.float()).all()
+            assert rel_err(got.float(), ref.float()) <= 1e-5, f"replay {rep}"
