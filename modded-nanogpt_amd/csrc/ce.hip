@@ -726,7 +726,7 @@ int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb
 int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
                       float scale, float* out, int64_t ldc, bool accumulate, hipStream_t st);
 
-extern int g_gemm_slot;
+extern thread_local int g_gemm_slot;
 struct GemmSlot {   // books the plain GEMM launches inside a scope under a CE profile slot
     int saved;
     explicit GemmSlot(int s) : saved(g_gemm_slot) { g_gemm_slot = s; }

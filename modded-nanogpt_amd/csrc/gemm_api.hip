@@ -43,10 +43,8 @@ void profile_end(int slot, hipStream_t st) {
     if (!g_prof_pending[slot].empty()) (void)hipEventRecord(g_prof_open[slot], st);
 }
 
-static char g_err[512];
 char* last_error_buf() {
     static thread_local char buf[512];
-    (void)g_err;
     return buf;
 }
 
@@ -76,7 +74,7 @@ static int check_gemm_dims(const char* who, int R, int C, int K, int64_t lda, in
 }
 
 // Which profile slot the next gemm_store launches are booked under (set by the fused CE backward).
-int g_gemm_slot = PROF_GEMM;
+thread_local int g_gemm_slot = PROF_GEMM;   // per host thread: entry points may be called concurrently
 
 // ---------------------------------------------------------------------------------------------
 // Balanced walk.  A persistent grid of G workgroups finishes `tiles` tiles in ceil(tiles / G) rounds,
