@@ -881,10 +881,10 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
     ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
     // a vocabulary split can be empty for a tiny V; its partial sums must read as zero
     fill_f32_kernel<<<(CE_SPLITS * M + 255) / 256, 256, 0, st>>>(part, (int64_t)CE_SPLITS * M, 0.0f);
-    if (int e = ngpt_quant_fp8(x_bf16, x_f8, (int64_t)M * K, x_s, NGPT_FMT_E4M3, stream)) return e;
     if (w_layout == NGPT_W_OUT_IN) {
-        if (int e = ngpt_quant_fp8(w_bf16, w_f8_vk, (int64_t)V * K, w_s, NGPT_FMT_E4M3, stream)) return e;
+        if (int e = quant_e4m3_pair(x_bf16, x_f8, (int64_t)M * K, x_s, w_bf16, w_f8_vk, (int64_t)V * K, w_s, st)) return e;
     } else {
+        if (int e = ngpt_quant_fp8(x_bf16, x_f8, (int64_t)M * K, x_s, NGPT_FMT_E4M3, stream)) return e;
         if (int e = ngpt_quant_fp8_2d(w_bf16, K, V, w_s, NGPT_FMT_E4M3, nullptr, w_f8_vk, stream)) return e;
     }
 

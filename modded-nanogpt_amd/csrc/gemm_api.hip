@@ -178,6 +178,9 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
     ProfileScope prof(g_gemm_slot, st);
     if (out_kind == 0) {
         EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C, nullptr, 0, false};
+        const int tiles = ((R + MainCfg::BM - 1) / MainCfg::BM) * ((C + MainCfg::BN - 1) / MainCfg::BN);
+        if (fa == FMT_E4M3 && fb == FMT_E4M3 && splits == 1 && 2 * tiles <= num_cus())
+            return launch_gemm_fmt<SmallCfg, FMT_E4M3, FMT_E4M3>(g, epi, st, 0);
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
     if (out_kind == 3) {
@@ -267,11 +270,11 @@ extern "C" int ngpt_mm_fwd(const void* x_bf16, const void* w_bf16, int M, int N,
     if (need > 0 && (!workspace || workspace_bytes < need))
         return fail(NGPT_EWORKSPACE, "ngpt_mm_fwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
     hipStream_t st = (hipStream_t)stream;
-    if (int e = ngpt_quant_fp8(x_bf16, x_f8, (int64_t)M * K, x_s, NGPT_FMT_E4M3, stream)) return e;
     const void* w_nk = w_f8;
     if (w_layout == NGPT_W_OUT_IN) {
-        if (int e = ngpt_quant_fp8(w_bf16, w_f8, (int64_t)N * K, w_s, NGPT_FMT_E4M3, stream)) return e;
+        if (int e = quant_e4m3_pair(x_bf16, x_f8, (int64_t)M * K, x_s, w_bf16, w_f8, (int64_t)N * K, w_s, st)) return e;
     } else {
+        if (int e = ngpt_quant_fp8(x_bf16, x_f8, (int64_t)M * K, x_s, NGPT_FMT_E4M3, stream)) return e;
         // w is [K, N]: one pass writes w_f8 [K, N] and the [N, K] copy the GEMM reads
         if (int e = ngpt_quant_fp8_2d(w_bf16, K, N, w_s, NGPT_FMT_E4M3, w_f8, workspace, stream)) return e;
         w_nk = workspace;

@@ -23,6 +23,10 @@ inline int check_launch(const char* what) {
     return NGPT_OK;
 }
 
+// e4m3 copies of two bf16 tensors in one launch (quant.hip).
+int quant_e4m3_pair(const void* in0, void* out0, int64_t n0, float s0, const void* in1, void* out1, int64_t n1, float s1,
+                    hipStream_t st);
+
 // Compute units of the current device (cached per process; one GPU per process by design).
 int num_cus();
 

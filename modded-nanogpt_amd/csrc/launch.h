@@ -7,6 +7,9 @@ namespace ngpt {
 
 // 256 x 256 tile, 8 waves as 4 (rows) x 2 (cols): each wave owns 64 x 128 = 2 x 4 MFMA tiles.
 using MainCfg = TileCfg<256, 256, 4, 2, 128, 2>;
+// Small problems (fewer 256 x 256 tiles than half the compute units): 128 x 128 tiles, 4 waves of 64 x 64, two
+// workgroups per compute unit, so that four times as many workgroups share the work.
+using SmallCfg = TileCfg<128, 128, 2, 2, 128, 2, 2>;
 // (Measured slower on MI355X for the shapes of this path: four 32 KiB stages of 64-byte k-steps, and a
 // 256 x 128 tile with two 4-wave workgroups per CU.  The kernel stays generic over TileCfg.)
 

@@ -13,6 +13,19 @@ __global__ __launch_bounds__(256) void quant_kernel(const v4i* __restrict__ in, 
     for (; i < n8; i += stride) out[i] = quant8<FMT>(in[i], qs);
 }
 
+// Two tensors in one launch (activations and weights ahead of a GEMM): blocks [0, blocks0) take the first.
+__global__ __launch_bounds__(256) void quant_pair_kernel(const v4i* __restrict__ in0, v2i* __restrict__ out0, int64_t n8_0, float s0,
+                                                         const v4i* __restrict__ in1, v2i* __restrict__ out1, int64_t n8_1, float s1,
+                                                         int blocks0) {
+    const bool first = (int)blockIdx.x < blocks0;
+    const v4i* in = first ? in0 : in1;
+    v2i* out = first ? out0 : out1;
+    const int64_t n8 = first ? n8_0 : n8_1;
+    const int b = first ? blockIdx.x : blockIdx.x - blocks0, nb = first ? blocks0 : gridDim.x - blocks0;
+    const QuantScale qs(first ? s0 : s1);
+    for (int64_t i = (int64_t)b * 256 + threadIdx.x; i < n8; i += (int64_t)nb * 256) out[i] = quant8<FMT_E4M3>(in[i], qs);
+}
+
 // 64 x 64 tile: quantise, write the row-major bytes, and write the transposed bytes via LDS.
 // IN_BYTES = 2: bf16 input quantised with scale s.  IN_BYTES = 1: plain byte transpose.
 template <int FMT, int IN_BYTES>
@@ -62,6 +75,24 @@ __global__ __launch_bounds__(256) void tile_transpose_kernel(const uint8_t* __re
 }  // namespace ngpt
 
 using namespace ngpt;
+
+namespace ngpt {
+// e4m3 copies of two bf16 tensors (n0, n1 elements, multiples of 8) in one launch.
+int quant_e4m3_pair(const void* in0, void* out0, int64_t n0, float s0, const void* in1, void* out1, int64_t n1, float s1,
+                    hipStream_t st) {
+    if (n0 % 8 || n1 % 8 || n0 <= 0 || n1 <= 0) return fail(NGPT_EALIGN, "quant_e4m3_pair: sizes %lld, %lld", (long long)n0, (long long)n1);
+    const int64_t cap = (int64_t)num_cus() * 16;
+    // blocks in proportion to the sizes, at least one each
+    int64_t b0 = (n0 / 8 + 255) / 256, b1 = (n1 / 8 + 255) / 256;
+    if (b0 + b1 > cap) {
+        b0 = b0 * cap / (b0 + b1);
+        if (b0 < 1) b0 = 1;
+        b1 = cap - b0 < 1 ? 1 : cap - b0;
+    }
+    quant_pair_kernel<<<(int)(b0 + b1), 256, 0, st>>>((const v4i*)in0, (v2i*)out0, n0 / 8, s0, (const v4i*)in1, (v2i*)out1, n1 / 8, s1, (int)b0);
+    return check_launch("quant_pair_kernel");
+}
+}  // namespace ngpt
 
 extern "C" int ngpt_quant_fp8(const void* in_bf16, void* out_f8, int64_t n, float scale, int fmt, void* stream) {
     if (!in_bf16 || !out_f8 || n < 0) return fail(NGPT_EINVAL, "ngpt_quant_fp8: null pointer or negative size");
