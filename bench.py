@@ -47,7 +47,28 @@ def profile_read(lib):
     return out
 
 
-def cpu_baseline(oracle, x, w, t, sc, budget_s=20.0):
+def make_cfg1(seed: int = 0, M: int = 1024, N: int = 3072, K: int = 768):
+    """Configuration 1: x ~ N(0,1) bf16 [M,K]; W ~ N(0,1/K) bf16 [N,K]; x_s = 1, w_s = 1/32 (drawn on the CPU, fp32 then cast)."""
+    import math
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    return x, w, 1.0, 1.0 / 32
+
+
+def make_cfg3(seed: int = 0, M: int = 49152, K: int = 768, V: int = 50304, n_tok: int = 50257):
+    """Configuration 3: x ~ N(0,1), W ~ N(0,1/K) (out,in), the reference's lm_head scales (train_gpt.py:1225), uniform targets."""
+    import math
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(V, K, generator=g) / math.sqrt(K)).bfloat16()
+    t = torch.randint(0, n_tok, (M,), generator=g, dtype=torch.int64)
+    return x, w, t, dict(x_s=100 / 448, w_s=1.6 / 448, grad_s=0.75 / 448, grad_scale=1.0, A=23.0, B=5.0, C=7.5)
+
+
+def cpu_baseline(x, w, t, sc, budget_s=20.0):
+    # the only place where this script touches the CPU oracle: as the baseline that is timed beside the GPU path
+    from oracle import nanogpt_fp8_oracle as oracle
     """Oracle forward+backward on the first rows of the same inputs; ~budget_s seconds of CPU work."""
     threads = torch.get_num_threads()
     rows_per_chunk = 1024
@@ -77,14 +98,14 @@ def calibrate_copy(dev) -> None:
     del src, dst
 
 
-def secondary(args, amd, oracle) -> int:
+def secondary(args, amd) -> int:
     """Other workloads of the path, same JSON shape; timed with events on the current stream."""
     import math
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(0)
     wl = args.workload
     if wl == "mm_cfg1":
-        x, w, x_s, w_s = oracle.make_cfg1(seed=0)
+        x, w, x_s, w_s = make_cfg1(seed=0)
         xd, wd = x.to(dev), w.to(dev)
         step = lambda: torch.ops.nanogpt.mm(xd, wd, x_s, w_s, 1.0)
         flops, desc, tokens = 2.0 * x.shape[0] * w.shape[0] * x.shape[1], "config 1: nanogpt::mm forward, M=1024 N=3072 K=768", x.shape[0]
@@ -242,14 +263,12 @@ def main() -> int:
 
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     import modded_nanogpt_amd as amd
-    from oracle import nanogpt_fp8_oracle as oracle
-
     lib = amd._lib.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     if args.workload != "lmhead_ce":
-        return secondary(args, amd, oracle)
+        return secondary(args, amd)
     dev = torch.device("cuda:0")
-    x, w, t, sc = oracle.make_cfg3(seed=0)
+    x, w, t, sc = make_cfg3(seed=0)
     xd, wd, td = x.to(dev), w.to(dev), t.to(dev)
     mtp = torch.tensor([1.0], device=dev)
     pt = torch.full((M,), -1, dtype=torch.int64, device=dev)
@@ -321,7 +340,7 @@ def main() -> int:
         "kernels": kernels, "roofline": roofline,
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(oracle, x, w, t, sc)
+        result["cpu_baseline"] = cpu_baseline(x, w, t, sc)
     print(json.dumps(result))
     return 0
 
