@@ -125,6 +125,24 @@ def test_package_never_imports_the_oracle():
             assert "oracle" not in p.read_text(), p
 
 
+def test_bench_uses_the_oracle_only_as_the_cpu_baseline():
+    """In bench.py the oracle may be imported by the cpu_baseline function and nowhere else."""
+    import ast
+    tree = ast.parse((ROOT / "bench.py").read_text())
+    def imports_oracle(node):
+        for n in ast.walk(node):
+            if isinstance(n, ast.ImportFrom) and n.module and n.module.split(".")[0] == "oracle":
+                return True
+            if isinstance(n, ast.Import) and any(a.name.split(".")[0] == "oracle" for a in n.names):
+                return True
+        return False
+    for node in tree.body:
+        if isinstance(node, ast.FunctionDef) and node.name == "cpu_baseline":
+            assert imports_oracle(node)
+        else:
+            assert not imports_oracle(node), getattr(node, "name", node)
+
+
 def test_shipped_gemm_kernels_do_not_spill(amd, tmp_path):
     """The 8-wave GEMM kernels must fit 256 VGPRs without spilling: one scratch reload inside the
     k-loop makes the compiler wait for all outstanding operand loads and serialises them."""
