@@ -212,9 +212,8 @@ __device__ __forceinline__ void global_to_lds16(const void* gptr, void* lds_wave
 }
 
 // Workgroup barrier WITHOUT the implicit "wait for all outstanding memory operations" that
-// __syncthreads() carries: the caller states which waits it needs (wait_vmem_le / wait_lds) so
+// __syncthreads() carries: the caller states which waits it needs (wait_vmem_le) so
 // that operand loads of later pipeline stages can stay in flight across the barrier.
-__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void wg_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 }  // namespace ngpt

@@ -39,49 +39,6 @@ __device__ __forceinline__ void strip_flush_rowmajor_u8(uint8_t* scratch, int la
     __builtin_amdgcn_s_waitcnt(0xc07f);
 }
 
-// Strip = 32 rows x WTN columns of bytes, stored row-major in global memory (leading dim ld).
-// `codes[tn][v]` holds the byte for accumulator element (tn, v) of one tm.
-template <class Cfg>
-__device__ __forceinline__ void store_strip_rowmajor_u8(
-    const uint32_t (&codes)[Cfg::TN][16], uint8_t* scratch, int lane,
-    uint8_t* out, int64_t ld, int grow0 /* global row of strip row 0 */, int gcol0, int R, int C) {
-#pragma unroll
-    for (int tn = 0; tn < Cfg::TN; ++tn)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) StripU8<Cfg>::put(scratch, lane, tn, v, codes[tn][v]);
-    strip_flush_rowmajor_u8<Cfg>(scratch, lane, out, ld, grow0, gcol0, R, C);
-}
-
-// Strip = 32 columns x WTM rows, stored transposed: out[col][row], leading dim ld.
-// `packed[tm][g]` holds four consecutive rows (8g + 4h .. +3 of tm) as one little-endian word.
-template <class Cfg>
-__device__ __forceinline__ void store_strip_transposed_u8(
-    const uint32_t (&packed)[Cfg::TM][4], uint8_t* scratch, int lane,
-    uint8_t* out, int64_t ld, int grow0, int gcol0 /* global col of strip col 0 */, int R, int C) {
-    constexpr int STRIDE = Cfg::WTM + 16;
-    static_assert(32 * STRIDE <= Cfg::WAVE_SCRATCH, "strip does not fit the wave's LDS scratch");
-    const int h = lane >> 5, j = lane & 31;
-#pragma unroll
-    for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-            *(uint32_t*)(scratch + j * STRIDE + tm * 32 + 8 * g + 4 * h) = packed[tm][g];
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    constexpr int CH_PER_ROW = Cfg::WTM / 16;
-    constexpr int PASSES = (32 * CH_PER_ROW + 63) / 64;
-#pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-        int id = p * 64 + lane;
-        int cl = id / CH_PER_ROW, ch = id % CH_PER_ROW;
-        if (cl < 32) {
-            v4i val = *(const v4i*)(scratch + cl * STRIDE + ch * 16);
-            int gc = gcol0 + cl, gr = grow0 + ch * 16;
-            if (gc < C && gr + 16 <= R) *(v4i*)(out + (int64_t)gc * ld + gr) = val;
-        }
-    }
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-}
-
 // acc * scale into an fp32 matrix: plain stores, or fire-and-forget L2 atomics (no read-modify-write
 // through registers) when `atomic`.  Shared by the fp32 output and by partial tiles of a split contraction.
 template <class Cfg>
