@@ -56,12 +56,15 @@ int ngpt_num_cus(void);
 int ngpt_profile_enable(int on);
 int ngpt_profile_read(int slot, double* total_ms, int* launches);
 
-/* Timing aid, no counterpart in the reference.  key 2: ablation bits for timing runs of
- * ngpt_gemm_fp8_tn with out_kind 3 (1 = no operand loads, 2 = no MFMAs, 4 = no k-loop barrier; results
- * are then meaningless); key 4: split-K factor used by ngpt_gemm_fp8_tn with out_kind 2; key 7: 1 =
- * accept operand row strides below K (overlapping rows keep the operands cache resident in timing runs).
- * Other keys are reserved. */
+#ifdef NGPT_BENCH_BUILD
+/* Timing aid, no counterpart in the reference; exists only in the measurement build of the library
+ * (libngpt_fp8_bench.so, compiled with -DNGPT_BENCH_BUILD), never in libngpt_fp8.so.  key 2: ablation bits
+ * for timing runs of ngpt_gemm_fp8_tn with out_kind 3 (1 = no operand loads, 2 = no MFMAs, 4 = no k-loop
+ * barrier; results are then meaningless); key 4: split-K factor used by ngpt_gemm_fp8_tn with out_kind 2;
+ * key 7: 1 = accept operand row strides below K (overlapping rows keep the operands cache resident in
+ * timing runs).  Process-global and not synchronised: one thread, set before the timed calls. */
 int ngpt_tuning_set(int key, int value);
+#endif
 
 /* ---- quantisers ---------------------------------------------------------------------------
  * out[i] = fp8(bf16_rne(fp32(in[i]) / scale)), round-to-nearest-even, NOT saturating
@@ -81,12 +84,16 @@ int ngpt_quant_fp8_2d(const void* in_bf16, int rows, int cols, float scale, int 
  * the fp8 operands.  rows % 16 == 0, cols % 16 == 0. */
 int ngpt_transpose_u8(const void* in, int rows, int cols, void* out, void* stream);
 
+/* out[c, r] = in[r, c] for elements of 1, 2 or 4 bytes and any shape: `transpose_copy` as the optimizer calls it on
+ * the bf16 tied embedding / lm_head weights (train_gpt.py:808-810; triton_kernels.py:788-841). */
+int ngpt_transpose_copy(const void* src, int rows, int cols, void* dst, int elem_bytes, void* stream);
+
 /* ---- the GEMM building block --------------------------------------------------------------
  * C[r, c] = scale * sum_k A[r, k] * B[c, k]; A [R, K] and B [C, K] are fp8 with the contraction
  * index contiguous (row strides lda / ldb bytes).  What `torch._scaled_mm` does for the
  * reference (call sites train_gpt_medium.py:47,76,85; train_gpt.py:85,117,128;
  * triton_kernels.py:1217,1268,1283).  out_kind: 0 = bf16, 1 = fp32, 2 = fp32 accumulate
- * (C += ...), 3 = discard the result (times the contraction loop alone).  ldc in elements.  K % 128 == 0, lda % 16 == 0, ldb % 16 == 0. */
+ * (C += ...); 3 = discard the result (times the contraction loop alone) in the measurement build only.  ldc in elements.  K % 128 == 0, lda % 16 == 0, ldb % 16 == 0. */
 int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const void* B, int fmt_b, int64_t ldb,
                      int R, int C, int K, float scale, void* out, int64_t ldc, int out_kind,
                      void* stream);
@@ -147,7 +154,7 @@ int ngpt_quant_transpose_down(const void* weights_bf16, int num_layers, int hidd
 /* MLP input producer, train_gpt.py:1643-1647 with norm() = F.rms_norm(x, (dim,)) (:952-953):
  *   normed  = rms_norm(x)                         bf16 [rows, dim]
  *   amax    = max(|normed|) clamped to 1e-12      (bf16 value)
- *   x_f8    = e4m3(bf16(normed * bf16(448 / amax)))
+ *   x_f8    = e4m3(bf16(normed * q)),  q = bf16(bf16(1 / amax) * 448)   (eager: `448.0 / amax` is amax.reciprocal() * 448.0)
  *   dequant = up_scale[0] * amax / 448            1-element fp32 device buffer (no host sync)
  * Two passes over the activations.  up_scale and dequant are device pointers.  dim % 8 == 0, dim <= 2048.
  * workspace: ngpt_mlp_input_quant_workspace_bytes() bytes of device memory. */
@@ -179,6 +186,14 @@ int ngpt_transpose_add(const void* src, int rows, int cols, void* dst, int elem_
  * Writes losses fp32 [n_rows] and grad e5m2 [n_rows, n_cols] (saturating store).
  * n_cols % 8 == 0, 1 <= n_predict <= NGPT_MAX_PREDICT.  The workspace holds two lookup
  * tables over the bf16 logit values. */
+/* Host-only check (no GPU work, callable without a device): can the CE kernels evaluate the softcap
+ * A * sigmoid((l + B) / C) for these constants?  Their lookup tables cover bf16 logits with |l| in [2^-12, 2^8)
+ * exactly and assume that sigma no longer changes outside, and they sum exponentials relative to the cap A.
+ * Returns NGPT_OK (the reference's 23 / 5 / 7.5 and e.g. 30 / 0 / 7.5, the 15 * tanh(x / 15) + 15 form of
+ * train_gpt.py:1683-1684) or NGPT_ERANGE with a message.  The three CE entry points below apply the same
+ * check and return NGPT_ERANGE instead of a silently wrong loss. */
+int ngpt_softcap_supported(float A, float B, float C);
+
 int64_t ngpt_ce_fwd_bwd_workspace_bytes(void);
 int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, const float* mtp_weights,
                     const int64_t* prefix_targets, const float* prefix_weight,
@@ -203,6 +218,21 @@ int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const int64_t* ta
                        int M, int K, int V, float x_s, float w_s, float A, float B, float C,
                        float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
                        int w_layout, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* The same forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): no workspace argument, the library uses a buffer of its own that
+ * is part of its code object (a static device array of about 1.1 MB, held by every GPU the library runs on
+ * until the process ends).  It has no counterpart in the reference.  Arguments and results are those of
+ * ngpt_lmhead_ce_fwd; M may be at most ngpt_lmhead_ce_fwd_static_max_rows() (65536), more is NGPT_ERANGE.
+ * The call allocates and frees nothing.  All calls on one GPU share that GPU's buffer: calls that may overlap
+ * on one GPU (two streams, two host threads) race; issue them on one stream or use ngpt_lmhead_ce_fwd. */
+int ngpt_lmhead_ce_fwd_static_max_rows(void);
+int ngpt_lmhead_ce_fwd_static(const void* x_bf16, const void* w_bf16, const int64_t* targets,
+                              const float* mtp_weights, int n_predict,
+                              const int64_t* prefix_targets, const float* prefix_weight,
+                              int M, int K, int V, float x_s, float w_s, float A, float B, float C,
+                              float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
+                              int w_layout, void* stream);
 
 /* Backward: gradients of sum(losses) * grad_scale (the incoming autograd gradient is ignored,
  * as in triton_kernels.py:1117,1262).  dx [M,K] bf16; dw fp32 in the weight's own layout

@@ -17,6 +17,7 @@ PKG = pathlib.Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libngpt_fp8.so"
+BENCH_LIB_PATH = LIB_DIR / "libngpt_fp8_bench.so"     # + the timing aids behind NGPT_BENCH_BUILD, for measurements only
 SOURCES = ["gemm_api.hip", "quant.hip", "ce.hip", "mlp_aux.hip"]
 
 HIPCC_FLAGS = [
@@ -34,12 +35,14 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (set HIPCC or add /opt/rocm/bin to PATH)")
 
 
-def build(verbose: bool = True) -> pathlib.Path:
-    """Compile every HIP source into one shared library; always recompiles."""
+def build(verbose: bool = True, bench: bool = False) -> pathlib.Path:
+    """Compile every HIP source into one shared library; always recompiles.  `bench`: the measurement build."""
     LIB_DIR.mkdir(exist_ok=True)
     srcs = [str(CSRC / s) for s in SOURCES if (CSRC / s).exists()]
-    tmp = LIB_PATH.with_suffix(".so.tmp")
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(PKG.parent / "include"), "-o", str(tmp), *srcs]
+    out = BENCH_LIB_PATH if bench else LIB_PATH
+    tmp = out.with_suffix(".so.tmp")
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *(["-DNGPT_BENCH_BUILD"] if bench else []), "-I", str(PKG.parent / "include"),
+           "-o", str(tmp), *srcs]
     if verbose:
         print("+", " ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -50,9 +53,10 @@ def build(verbose: bool = True) -> pathlib.Path:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, out)
+    return out
 
 
 if __name__ == "__main__":
     print(build())
+    print(build(bench=True))

@@ -16,6 +16,9 @@
 #include "host_util.h"
 #include "launch.h"
 #include "panel.h"
+#include <atomic>
+#include <cmath>
+#include <cstring>
 
 namespace ngpt {
 
@@ -740,6 +743,54 @@ static Softcap make_softcap(float A, float B, float C) {
     sc.B_div_C = B * sc.inv_C;
     return sc;
 }
+// The tables hold the softcap exactly for |l| in [2^-12, 2^8); outside, a logit takes the entry of the nearest
+// covered value, and the sum of exponentials is taken relative to the cap A without a running maximum.  Both are
+// exact for constants like the reference's (A = 23, B = 5, C = 7.5) and silently wrong for others (a large C
+// leaves sigma unsaturated at |l| = 256, a large A underflows exp(-A)), so every entry point checks its
+// (A, B, C) here, on the host, with the kernel's own fp32 expressions:
+//   * |l| < 2^-12 rounds to the same bf16 sigma as l = 0 (checked at the largest uncovered magnitude, both signs;
+//     sigma is monotone in l);
+//   * l >= 2^8 : bf16 sigma has reached 1 at the last covered value, l = 255;
+//   * l <= -2^8: at l = -255 sigma is below 2^-36 and exp(A sigma - A) equals exp(-A) in fp32, so the summand is
+//     that of sigma = 0, and the gradient there, at most coef * S_w * sigma, lies more than the whole e5m2
+//     range (57344 / 2^-17 < 2^33) below any gradient entry that is itself representable: both the exact value
+//     and the table's round to zero;
+//   * exp(-A) is a normal fp32 number with room to spare, so neither a row's sum nor its products underflow.
+static float host_bf16_round(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    u &= 0xffff0000u;
+    memcpy(&f, &u, 4);
+    return f;
+}
+static float host_bf16_value(uint32_t bits) {
+    bits <<= 16;
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+static float host_sigma(float l, const Softcap& sc) {
+    const float u = l * sc.inv_C + sc.B_div_C;
+    return host_bf16_round(1.0f / (1.0f + expf(-u)));
+}
+static int check_softcap(const char* who, float A, float B, float C) {
+    if (!(A > 0.0f) || !(C > 0.0f) || !std::isfinite(A) || !std::isfinite(B) || !std::isfinite(C))
+        return fail(NGPT_ERANGE, "%s: softcap constants A=%g B=%g C=%g must be finite with A > 0 and C > 0", who, A, B, C);
+    const Softcap sc = make_softcap(A, B, C);
+    const float tiny = host_bf16_value(TAB_LO - 1), last = host_bf16_value(TAB_LO + TAB_N - 1);
+    const float s0 = host_sigma(0.0f, sc);
+    const char* why = nullptr;
+    if (host_sigma(tiny, sc) != s0 || host_sigma(-tiny, sc) != s0) why = "logits below 2^-12 in magnitude do not round to sigma(0)";
+    else if (host_sigma(last, sc) != 1.0f) why = "sigma has not reached 1 in bf16 at logit 255";
+    else if (!(host_sigma(-last, sc) < 0x1p-36f) || expf(A * host_sigma(-last, sc) - A) != expf(-A))
+        why = "sigma has not vanished at logit -255";
+    else if (!(expf(-A) >= 0x1p-100f)) why = "exp(-A) is too small for sums of exponentials relative to the cap";
+    if (why)
+        return fail(NGPT_ERANGE, "%s: softcap A=%g B=%g C=%g is outside what the lookup tables cover (%s)", who, A, B, C, why);
+    return NGPT_OK;
+}
+
 // grad_scale * (1/C * A) * (1/grad_s), in the reference's fp32 order
 static float make_coef(float A, float C, float grad_s, float grad_scale) {
     return grad_scale * (1.0f / C * A) * (1.0f / grad_s);
@@ -757,11 +808,8 @@ template <class Cfg>
 static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwd& epi, hipStream_t st) {
     auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, EpiCEFwd, CEJobIter>;
     constexpr int LDS = Cfg::SMEM_BYTES + EpiCEFwd::EXTRA_LDS;   // dynamic part; the table is static LDS
-    static bool configured = false;
-    if (!configured) {
-        if (int e = allow_lds(kernel, LDS)) return e;
-        configured = true;
-    }
+    static PerDeviceOnce configured;
+    if (int e = configured.run([&] { return allow_lds(kernel, LDS); })) return e;
     int cus = num_cus();
     if (cus < CE_XCDS * CE_SPLITS) return fail(NGPT_EINVAL, "no HIP device (or fewer than %d compute units)", CE_XCDS * CE_SPLITS);
     int tiles_m = (g.C + Cfg::BN - 1) / Cfg::BN;
@@ -780,11 +828,8 @@ template <class Cfg, class Epi>
 static int launch_grid_kernel(const GemmOperands& g, const Epi& epi, hipStream_t st, int slot, const char* what) {
     auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, Epi, GridIter>;
     constexpr int LDS = Cfg::SMEM_BYTES + Epi::EXTRA_LDS;
-    static bool configured = false;
-    if (!configured) {
-        if (int e = allow_lds(kernel, LDS)) return e;
-        configured = true;
-    }
+    static PerDeviceOnce configured;
+    if (int e = configured.run([&] { return allow_lds(kernel, LDS); })) return e;
     const int cus = num_cus();
     if (cus <= 0) return fail(NGPT_EINVAL, "no HIP device");
     int tiles = ((g.R + Cfg::BM - 1) / Cfg::BM) * ((g.C + Cfg::BN - 1) / Cfg::BN);
@@ -807,6 +852,8 @@ static int64_t round256(int64_t n) { return (n + 255) / 256 * 256; }
 using namespace ngpt;
 
 // ------------------------------------------------------------------------------------------------
+extern "C" int ngpt_softcap_supported(float A, float B, float C) { return check_softcap("ngpt_softcap_supported", A, B, C); }
+
 extern "C" int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, const float* mtp_weights,
                                const int64_t* prefix_targets, const float* prefix_weight,
                                float* losses, void* grad_e5m2, int n_rows, int n_cols, int n_predict,
@@ -814,6 +861,7 @@ extern "C" int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, 
                                void* workspace, int64_t workspace_bytes, void* stream) {
     if (!logits_bf16 || !losses || !grad_e5m2) return fail(NGPT_EINVAL, "ngpt_ce_fwd_bwd: null pointer");
     if (int e = check_cand("ngpt_ce_fwd_bwd", targets, mtp_weights, n_predict)) return e;
+    if (int e = check_softcap("ngpt_ce_fwd_bwd", A, B, C)) return e;
     if (n_rows <= 0 || n_cols <= 0) return fail(NGPT_EINVAL, "ngpt_ce_fwd_bwd: empty logits %d x %d", n_rows, n_cols);
     if (n_cols % 8) return fail(NGPT_EALIGN, "ngpt_ce_fwd_bwd: n_cols=%d must be a multiple of 8", n_cols);
     if (!workspace || workspace_bytes < 2 * TAB_BYTES)
@@ -855,22 +903,25 @@ extern "C" int64_t ngpt_lmhead_ce_fwd_workspace_bytes(int M, int K, int V, int w
     return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)CE_SPLITS * M * 4, 256);
 }
 
-extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const int64_t* targets,
-                                  const float* mtp_weights, int n_predict,
-                                  const int64_t* prefix_targets, const float* prefix_weight,
-                                  int M, int K, int V, float x_s, float w_s, float A, float B, float C,
-                                  float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
-                                  int w_layout, void* workspace, int64_t workspace_bytes, void* stream) {
+namespace ngpt {
+// Forward of the fused lm_head + CE on a workspace that the caller (ngpt_lmhead_ce_fwd) or the library itself
+// (ngpt_lmhead_ce_fwd_static) provides; `who` names the entry point in error messages.
+static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w_bf16, const int64_t* targets,
+                              const float* mtp_weights, int n_predict, const int64_t* prefix_targets, const float* prefix_weight,
+                              int M, int K, int V, float x_s, float w_s, float A, float B, float C,
+                              float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
+                              int w_layout, void* workspace, int64_t workspace_bytes, void* stream) {
     if (!x_bf16 || !w_bf16 || !losses || !lse || !saved_sigma || !x_f8 || !w_f8_vk || !workspace)
-        return fail(NGPT_EINVAL, "ngpt_lmhead_ce_fwd: null pointer");
-    if (int e = check_cand("ngpt_lmhead_ce_fwd", targets, mtp_weights, n_predict)) return e;
-    if (M <= 0 || K <= 0 || V <= 0) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_fwd: empty problem M=%d K=%d V=%d", M, K, V);
+        return fail(NGPT_EINVAL, "%s: null pointer", who);
+    if (int e = check_cand(who, targets, mtp_weights, n_predict)) return e;
+    if (int e = check_softcap(who, A, B, C)) return e;
+    if (M <= 0 || K <= 0 || V <= 0) return fail(NGPT_EINVAL, "%s: empty problem M=%d K=%d V=%d", who, M, K, V);
     if (K % 128 || M % 16 || V % 16)
-        return fail(NGPT_EALIGN, "ngpt_lmhead_ce_fwd: need K %% 128 == 0, M %% 16 == 0, V %% 16 == 0 (M=%d K=%d V=%d)", M, K, V);
-    if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_fwd: w_layout=%d", w_layout);
+        return fail(NGPT_EALIGN, "%s: need K %% 128 == 0, M %% 16 == 0, V %% 16 == 0 (M=%d K=%d V=%d)", who, M, K, V);
+    if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "%s: w_layout=%d", who, w_layout);
     int64_t need = ngpt_lmhead_ce_fwd_workspace_bytes(M, K, V, w_layout);
     if (workspace_bytes < need)
-        return fail(NGPT_EWORKSPACE, "ngpt_lmhead_ce_fwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
+        return fail(NGPT_EWORKSPACE, "%s: workspace %lld < %lld bytes", who, (long long)workspace_bytes, (long long)need);
     hipStream_t st = (hipStream_t)stream;
     uint8_t* ws = (uint8_t*)workspace;
     float* tabE = (float*)ws;
@@ -901,6 +952,59 @@ extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const 
     ce_finalize_kernel<<<(M + 255) / 256, 256, 0, st>>>(part, saved_sigma, epi.ca, sc, losses, lse);
     return check_launch("ce_finalize_kernel");
 }
+}  // namespace ngpt
+
+// ---- allocation-free forward -------------------------------------------------------------------
+// The workspace of the forward (two lookup tables and the per-split partial sums of exponentials) for up to
+// kStaticMaxRows tokens, as a file-scope device array: every GPU the library runs on holds its own copy at its own
+// address until the process ends.  In host code the array's name is only a handle: its device address on the
+// current GPU comes from hipGetSymbolAddress, once per device, and that pointer is what kernels are given.
+constexpr int kStaticMaxRows = 65536;
+constexpr int64_t kStaticBytes = (2 * TAB_BYTES + 255) / 256 * 256 + (int64_t)CE_SPLITS * kStaticMaxRows * 4;
+static __device__ __align__(256) uint8_t scratch[kStaticBytes];
+
+static std::atomic<void*> g_static_ptr[kMaxDevices];
+static int static_scratch(void** out) {
+    const int dev = current_device();
+    if (dev < 0 || dev >= kMaxDevices) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_fwd_static: no current HIP device (or its index is above %d)", kMaxDevices - 1);
+    void* p = g_static_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail(e != hipSuccess ? (int)e : NGPT_EINVAL, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+        g_static_ptr[dev].store(p, std::memory_order_release);      // racing first calls store the same address
+    }
+    *out = p;
+    return NGPT_OK;
+}
+
+extern "C" int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const int64_t* targets,
+                                  const float* mtp_weights, int n_predict,
+                                  const int64_t* prefix_targets, const float* prefix_weight,
+                                  int M, int K, int V, float x_s, float w_s, float A, float B, float C,
+                                  float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
+                                  int w_layout, void* workspace, int64_t workspace_bytes, void* stream) {
+    return lmhead_ce_fwd_impl("ngpt_lmhead_ce_fwd", x_bf16, w_bf16, targets, mtp_weights, n_predict, prefix_targets, prefix_weight,
+                              M, K, V, x_s, w_s, A, B, C, losses, lse, saved_sigma, x_f8, w_f8_vk, w_layout,
+                              workspace, workspace_bytes, stream);
+}
+
+extern "C" int ngpt_lmhead_ce_fwd_static_max_rows(void) { return kStaticMaxRows; }
+
+extern "C" int ngpt_lmhead_ce_fwd_static(const void* x_bf16, const void* w_bf16, const int64_t* targets,
+                                         const float* mtp_weights, int n_predict,
+                                         const int64_t* prefix_targets, const float* prefix_weight,
+                                         int M, int K, int V, float x_s, float w_s, float A, float B, float C,
+                                         float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
+                                         int w_layout, void* stream) {
+    if (M > kStaticMaxRows)
+        return fail(NGPT_ERANGE, "ngpt_lmhead_ce_fwd_static: M=%d exceeds the %d rows its built-in workspace holds; "
+                    "use ngpt_lmhead_ce_fwd with a caller-provided workspace", M, kStaticMaxRows);
+    void* ws = nullptr;
+    if (int e = static_scratch(&ws)) return e;
+    return lmhead_ce_fwd_impl("ngpt_lmhead_ce_fwd_static", x_bf16, w_bf16, targets, mtp_weights, n_predict, prefix_targets,
+                              prefix_weight, M, K, V, x_s, w_s, A, B, C, losses, lse, saved_sigma, x_f8, w_f8_vk, w_layout,
+                              ws, kStaticBytes, stream);
+}
 
 // ------------------------------------------------------------------------------------------------
 // backward workspace: tabE | tabD | rowf [M rounded up to 256] | big [same, one int per 256 rows used] | x^T panel [Kp, Mt] | W^T panel [Kp, V] | dlogits panel [Vp, Mt] |
@@ -922,6 +1026,7 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     if (!x_f8 || !w_f8_vk || !lse || !saved_sigma || !dx_bf16 || !dw_f32 || !workspace)
         return fail(NGPT_EINVAL, "ngpt_lmhead_ce_bwd: null pointer");
     if (int e = check_cand("ngpt_lmhead_ce_bwd", targets, mtp_weights, n_predict)) return e;
+    if (int e = check_softcap("ngpt_lmhead_ce_bwd", A, B, C)) return e;
     if (M <= 0 || K <= 0 || V <= 0) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_bwd: empty problem M=%d K=%d V=%d", M, K, V);
     if (K % 128 || M % 128 || V % 128)
         return fail(NGPT_EALIGN, "ngpt_lmhead_ce_bwd: need M, K, V multiples of 128 (M=%d K=%d V=%d)", M, K, V);

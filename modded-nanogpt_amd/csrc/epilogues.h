@@ -213,7 +213,9 @@ struct EpiDpre {
     }
 };
 
-// Mainloop-only timing aid: keeps the accumulators alive but writes (practically) nothing.
+#ifdef NGPT_BENCH_BUILD
+// Mainloop-only timing aid (measurement build of the library only): keeps the accumulators alive but writes
+// (practically) nothing.
 template <bool ABLATE>
 struct EpiDiscardT {
     static constexpr bool ABLATABLE = ABLATE;
@@ -250,6 +252,10 @@ struct EpiDiscardT {
     }
 };
 
+using EpiDiscard = EpiDiscardT<false>;
+using EpiDiscardAblate = EpiDiscardT<true>;    // honours GemmOperands::ablate, at the price of its branches
+#endif  // NGPT_BENCH_BUILD
+
 // out[r, c] (+)= acc * scale in fp32.  The += form (ACCUMULATE, or a job that holds only part of its
 // tile's contraction) uses floating-point atomics on an output the caller has initialised.
 template <bool ACCUMULATE>
@@ -276,9 +282,6 @@ struct EpiStoreF32 {
         else store_tile_f32<Cfg>(acc, out, ld, scale, R, C, r0, c0, co, false);
     }
 };
-
-using EpiDiscard = EpiDiscardT<false>;
-using EpiDiscardAblate = EpiDiscardT<true>;    // honours GemmOperands::ablate, at the price of its branches
 
 // post = bf16(max(bf16(acc * dequant), 0)^2) for a GEMM that runs TRANSPOSED (tile rows = hidden units, tile
 // columns = tokens, post [tokens, hidden] row-major): a lane's four consecutive accumulator registers are

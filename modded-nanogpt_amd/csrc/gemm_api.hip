@@ -4,6 +4,7 @@
 #include "host_util.h"
 #include "launch.h"
 #include "panel.h"
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -48,26 +49,45 @@ char* last_error_buf() {
     return buf;
 }
 
-int num_cus() {
-    static int cached = -1;
-    if (cached < 0) {
-        int dev = 0;
-        hipDeviceProp_t p;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) {
-            (void)hipGetLastError();
-            return 0;
-        }
-        cached = p.multiProcessorCount;
+int current_device() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
     }
-    return cached;
+    return dev;
 }
 
+// Compute units of the CURRENT device; one relaxed atomic per device caches the query (two threads that
+// race on the first call both store the same value).
+int num_cus() {
+    static std::atomic<int> cached[kMaxDevices];
+    const int dev = current_device();
+    if (dev < 0) return 0;
+    if (dev < kMaxDevices) {
+        const int c = cached[dev].load(std::memory_order_relaxed);
+        if (c > 0) return c;
+    }
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    if (dev < kMaxDevices) cached[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
+#ifdef NGPT_BENCH_BUILD
 int g_tuning[8] = {0, 2, 0, 0, 1, 0, 0, 0};
+static bool relaxed_strides() { return g_tuning[7] != 0; }
+#else
+static bool relaxed_strides() { return false; }
+#endif
 
 static int check_gemm_dims(const char* who, int R, int C, int K, int64_t lda, int64_t ldb) {
     if (R <= 0 || C <= 0 || K <= 0) return fail(NGPT_EINVAL, "%s: empty problem R=%d C=%d K=%d", who, R, C, K);
     if (K % 128) return fail(NGPT_EALIGN, "%s: contraction length %d must be a multiple of 128", who, K);
-    if (lda % 16 || ldb % 16 || ((lda < K || ldb < K) && !g_tuning[7]))
+    if (lda % 16 || ldb % 16 || ((lda < K || ldb < K) && !relaxed_strides()))
         return fail(NGPT_EALIGN, "%s: operand row strides (%lld, %lld) must be multiples of 16 and >= K",
                     who, (long long)lda, (long long)ldb);
     return NGPT_OK;
@@ -174,7 +194,12 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
     if (splits < 1) splits = 1;
     if (splits > K / 128) splits = K / 128;
     if (splits > 1 && out_kind != 2) return fail(NGPT_EINVAL, "gemm_fp8_tn: split-K needs the accumulating fp32 output");
-    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, splits, g_tuning[2]};
+#ifdef NGPT_BENCH_BUILD
+    const int ablate = g_tuning[2];
+#else
+    const int ablate = 0;
+#endif
+    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, splits, ablate};
     ProfileScope prof(g_gemm_slot, st);
     if (out_kind == 0) {
         EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C, nullptr, 0, false};
@@ -184,12 +209,16 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
     if (out_kind == 3) {
+#ifdef NGPT_BENCH_BUILD
         if (g.ablate) {
             EpiDiscardAblate epi{(float*)out, 0, 0};
             return launch_gemm<MainCfg>(g, fa, fb, epi, st);
         }
         EpiDiscard epi{(float*)out, 0, 0};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
+#else
+        return fail(NGPT_EINVAL, "gemm_fp8_tn: out_kind 3 (discard) exists in the measurement build of the library only");
+#endif
     }
     if (out_kind == 2) {
         EpiStoreF32<true> epi{(float*)out, ldc, scale, R, C, false};
@@ -207,11 +236,13 @@ extern "C" int ngpt_abi_version(void) { return 1; }
 extern "C" const char* ngpt_last_error(void) { return last_error_buf(); }
 extern "C" int ngpt_num_cus(void) { return num_cus(); }
 
+#ifdef NGPT_BENCH_BUILD
 extern "C" int ngpt_tuning_set(int key, int value) {
     if (key < 0 || key >= 8) return fail(NGPT_EINVAL, "ngpt_tuning_set: key=%d", key);
     g_tuning[key] = value;
     return NGPT_OK;
 }
+#endif
 
 extern "C" int ngpt_profile_enable(int on) {
     std::lock_guard<std::mutex> lk(g_prof_mu);
@@ -249,7 +280,12 @@ extern "C" int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const voi
     if ((fmt_a | fmt_b) & ~1) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: fmt_a=%d fmt_b=%d", fmt_a, fmt_b);
     if (out_kind < 0 || out_kind > 3) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: out_kind=%d", out_kind);
     if (ldc < C) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: ldc=%lld < C=%d", (long long)ldc, C);
-    return gemm_store(A, fmt_a, lda, B, fmt_b, ldb, R, C, K, scale, out, ldc, out_kind, (hipStream_t)stream, g_tuning[4]);
+#ifdef NGPT_BENCH_BUILD
+    const int splits = g_tuning[4];
+#else
+    const int splits = 1;
+#endif
+    return gemm_store(A, fmt_a, lda, B, fmt_b, ldb, R, C, K, scale, out, ldc, out_kind, (hipStream_t)stream, splits);
 }
 
 // ------------------------------------------------------------------------------------------ mm forward

@@ -48,7 +48,7 @@ struct GemmOperands {
     int64_t lda, ldb;   // ignored for a blocked operand
     int R, C, K;        // K % 128 == 0
     int splits;         // split-K: the contraction of a split tile is cut into this many jobs (>= 1); needs an accumulating epilogue if > 1
-    int ablate;         // timing aid: bit 0 = issue no operand loads after the first, bit 1 = no MFMA work, bit 2 = no k-loop barrier
+    int ablate;         // timing aid, measurement build only (no epilogue of the default build honours it): bit 0 = issue no operand loads after the first, bit 1 = no MFMA work, bit 2 = no k-loop barrier
     int layout;         // kBlockedA | kBlockedB | kRowsPermuted
     int full_tiles;     // the first full_tiles tiles (in walk order) are never split; 0 = `splits` applies to every tile
     int a_rows_pad;     // transposed A only: R rounded up to 256

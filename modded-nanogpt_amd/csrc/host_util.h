@@ -27,7 +27,9 @@ inline int check_launch(const char* what) {
 int quant_e4m3_pair(const void* in0, void* out0, int64_t n0, float s0, const void* in1, void* out1, int64_t n1, float s1,
                     hipStream_t st);
 
-// Compute units of the current device (cached per process; one GPU per process by design).
+// Index of the current HIP device (-1 if there is none) and its number of compute units (cached per device).
+constexpr int kMaxDevices = 64;
+int current_device();
 int num_cus();
 
 // Allow a kernel to use `bytes` of dynamic LDS (needed above 64 KiB); cached per kernel.

@@ -2,6 +2,7 @@
 #pragma once
 #include "gemm_tn.h"
 #include "host_util.h"
+#include <atomic>
 
 namespace ngpt {
 
@@ -13,20 +14,33 @@ using SmallCfg = TileCfg<128, 128, 2, 2, 128, 2, 2>;
 // (Measured slower on MI355X for the shapes of this path: four 32 KiB stages of 64-byte k-steps, and a
 // 256 x 128 tile with two 4-wave workgroups per CU.  The kernel stays generic over TileCfg.)
 
-// Tuning keys: [2] ablation bits (timing aid, honoured by the discarding epilogue only),
+#ifdef NGPT_BENCH_BUILD
+// Measurement build only.  Tuning keys: [2] ablation bits (honoured by the discarding epilogue only),
 // [4] split-K factor of ngpt_gemm_fp8_tn,
-// [7] 1 = accept operand row strides below K (timing aid: overlapping rows keep the operands cache resident)
+// [7] 1 = accept operand row strides below K (overlapping rows keep the operands cache resident)
 extern int g_tuning[8];
+#endif
+
+// hipFuncSetAttribute applies to the device that is current when it is called: one flag per kernel
+// instantiation and device.  Racing first calls both set the attribute, which is harmless.
+struct PerDeviceOnce {
+    std::atomic<bool> done[kMaxDevices];
+    template <class F>
+    int run(F&& f) {
+        const int dev = current_device();
+        if (dev >= 0 && dev < kMaxDevices && done[dev].load(std::memory_order_acquire)) return NGPT_OK;
+        if (int e = f()) return e;
+        if (dev >= 0 && dev < kMaxDevices) done[dev].store(true, std::memory_order_release);
+        return NGPT_OK;
+    }
+};
 
 template <class Cfg, int FA, int FB, class Epi>
 int launch_gemm_fmt(const GemmOperands& g, const Epi& epi, hipStream_t st, int max_grid) {
     auto kernel = gemm_tn_kernel<Cfg, FA, FB, Epi, GridIter>;
     constexpr int LDS = Cfg::SMEM_BYTES + Epi::EXTRA_LDS;
-    static bool configured = false;
-    if (!configured) {
-        if (int e = allow_lds(kernel, LDS)) return e;
-        configured = true;
-    }
+    static PerDeviceOnce configured;
+    if (int e = configured.run([&] { return allow_lds(kernel, LDS); })) return e;
     int tiles = ((g.R + Cfg::BM - 1) / Cfg::BM) * ((g.C + Cfg::BN - 1) / Cfg::BN) * (g.splits < 1 ? 1 : g.splits);
     int cus = num_cus();
     if (cus <= 0) return fail(NGPT_EINVAL, "no HIP device");

@@ -94,6 +94,25 @@ __global__ __launch_bounds__(256) void transpose_add_kernel(const T* __restrict_
     }
 }
 
+// dst [cols, rows] = src [rows, cols]^T for 2- and 4-byte elements, 64 x 64 tiles through LDS (the 1-byte
+// case has its own kernel with 16-byte accesses, tile_transpose_kernel).
+template <class T>
+__global__ __launch_bounds__(256) void transpose_copy_kernel(const T* __restrict__ src, int rows, int cols, T* __restrict__ dst) {
+    __shared__ T tile[64][64 + (sizeof(T) == 2 ? 2 : 1)];
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int rl = i >> 6, cl = i & 63;
+        const int r = r0 + rl, c = c0 + cl;
+        if (r < rows && c < cols) tile[rl][cl] = src[(int64_t)r * cols + c];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int cl = i >> 6, rl = i & 63;       // dst row = source column
+        const int r = r0 + rl, c = c0 + cl;
+        if (r < rows && c < cols) dst[(int64_t)c * rows + r] = tile[rl][cl];
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // MLP input producer: rms-norm, per-tensor amax and dynamic e4m3 quantisation (two passes over the
 // activations instead of the two reductions plus two element-wise passes of the eager formulation).
@@ -159,15 +178,17 @@ __device__ __forceinline__ float block_max_of(const float* __restrict__ v, int n
     return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
 }
 
-// Pass 2.  amax = max(partials) clamped to bf16(1e-12); x_f8 = e4m3(bf16(normed * bf16(448 / amax)))
-// (every bf16 operation of the eager expression rounds); dequant[0] = up_scale * amax / 448 in fp32.
+// Pass 2.  amax = max(partials) clamped to bf16(1e-12); x_f8 = e4m3(bf16(normed * q)) with
+// q = bf16(bf16(1 / amax) * 448): every bf16 operation of the eager expression rounds, and eager evaluates
+// `448.0 / amax` (Python float over a bf16 tensor) as amax.reciprocal() * 448.0, not as one division -- the two
+// differ in the last bf16 digit for about a quarter of all amax values.  dequant[0] = up_scale * amax / 448 in fp32.
 __global__ __launch_bounds__(256) void amax_quant_kernel(const v4i* __restrict__ normed, int64_t n8, const float* __restrict__ partial,
                                                          int npartial, const float* __restrict__ up_scale,
                                                          v2i* __restrict__ x_f8, float* __restrict__ dequant) {
     __shared__ float red[4];
     float amax = fmaxf(block_max_of(partial, npartial, red), round_to_bf16(1.0e-12f));
     if (blockIdx.x == 0 && threadIdx.x == 0) dequant[0] = __fdiv_rn(up_scale[0] * amax, 448.0f);
-    const float q = round_to_bf16(__fdiv_rn(448.0f, amax));
+    const float q = round_to_bf16(round_to_bf16(__fdiv_rn(1.0f, amax)) * 448.0f);
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
         v4i v = normed[i];
         const uint32_t u[4] = {(uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w};
@@ -261,6 +282,21 @@ extern "C" int ngpt_transpose_add(const void* src, int rows, int cols, void* dst
     else
         return fail(NGPT_EINVAL, "ngpt_transpose_add: elem_bytes=%d (2 = bf16, 4 = fp32)", elem_bytes);
     return check_launch("transpose_add_kernel");
+}
+
+extern "C" int ngpt_transpose_copy(const void* src, int rows, int cols, void* dst, int elem_bytes, void* stream) {
+    if (!src || !dst || rows <= 0 || cols <= 0) return fail(NGPT_EINVAL, "ngpt_transpose_copy: null pointer or empty matrix");
+    if (elem_bytes == 1 && rows % 16 == 0 && cols % 16 == 0) return ngpt_transpose_u8(src, rows, cols, dst, stream);
+    dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+    if (elem_bytes == 1)
+        transpose_copy_kernel<uint8_t><<<grid, 256, 0, (hipStream_t)stream>>>((const uint8_t*)src, rows, cols, (uint8_t*)dst);
+    else if (elem_bytes == 2)
+        transpose_copy_kernel<uint16_t><<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)src, rows, cols, (uint16_t*)dst);
+    else if (elem_bytes == 4)
+        transpose_copy_kernel<uint32_t><<<grid, 256, 0, (hipStream_t)stream>>>((const uint32_t*)src, rows, cols, (uint32_t*)dst);
+    else
+        return fail(NGPT_EINVAL, "ngpt_transpose_copy: elem_bytes=%d (1, 2 or 4)", elem_bytes);
+    return check_launch("transpose_copy_kernel");
 }
 
 extern "C" int64_t ngpt_mlp_input_quant_workspace_bytes(void) { return kNormPartials * (int64_t)sizeof(float); }

@@ -18,14 +18,15 @@ E4M3 = torch.float8_e4m3fn
 
 
 def transpose_copy(src: Tensor, dst: Tensor) -> None:
-    """dst (N, M) = src (M, N).T for 1-byte element types -- reference triton_kernels.py:819-841."""
+    """dst (N, M) = src (M, N).T for any element type of 1, 2 or 4 bytes -- reference triton_kernels.py:819-841
+    (called on the fp8 operands and, by the optimizer, on the bf16 tied weights, train_gpt.py:808-810)."""
     assert src.ndim == 2 and dst.ndim == 2
     M, N = src.shape
     assert dst.shape == (N, M), f"Expected dst shape ({N}, {M}), got {dst.shape}"
-    assert src.is_contiguous() and dst.is_contiguous() and src.element_size() == 1 and dst.element_size() == 1
+    assert src.is_contiguous() and dst.is_contiguous() and src.dtype == dst.dtype and src.element_size() in (1, 2, 4)
     ops._gpu(src, dst)
-    _lib.check(_lib.load().ngpt_transpose_u8(src.data_ptr(), M, N, dst.data_ptr(), ops._stream(src)),
-               "ngpt_transpose_u8")
+    _lib.check(_lib.load().ngpt_transpose_copy(src.data_ptr(), M, N, dst.data_ptr(), src.element_size(),
+                                               ops._stream(src)), "ngpt_transpose_copy")
 
 
 def transpose_add(src: Tensor, dst: Tensor) -> None:

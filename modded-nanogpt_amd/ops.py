@@ -85,7 +85,8 @@ def mm_backward_op(g: Tensor, x_f8: Tensor, w_f8: Tensor, x_s: float, w_s: float
     dx = torch.empty((M, K), dtype=torch.bfloat16, device=g.device)
     dw_kn = torch.empty((K, N), dtype=torch.float32, device=g.device)
     ws = _workspace(lib.ngpt_mm_bwd_workspace_bytes(M, N, K, _lib.W_OUT_IN), g.device)
-    _lib.check(lib.ngpt_mm_bwd(_p(g), _p(x_f8.contiguous()), _p(w_f8.contiguous()), M, N, K, x_s, w_s, grad_s,
+    x_f8, w_f8 = x_f8.contiguous(), w_f8.contiguous()     # bound to names: the copies outlive the launch
+    _lib.check(lib.ngpt_mm_bwd(_p(g), _p(x_f8), _p(w_f8), M, N, K, x_s, w_s, grad_s,
                                _p(dx), _p(dw_kn), _lib.W_OUT_IN, _p(ws), ws.numel(), _stream(g)), "ngpt_mm_bwd")
     return dx, dw_kn.T
 
@@ -155,7 +156,8 @@ def mm_t_backward_op(g: Tensor, x_f8: Tensor, w_f8: Tensor, x_s: float, w_s: flo
     dx = torch.empty((M, K), dtype=torch.bfloat16, device=g.device)
     dw = torch.empty((K, N), dtype=torch.float32, device=g.device)
     ws = _workspace(lib.ngpt_mm_bwd_workspace_bytes(M, N, K, _lib.W_IN_OUT), g.device)
-    _lib.check(lib.ngpt_mm_bwd(_p(g), _p(x_f8.contiguous()), _p(w_f8.contiguous()), M, N, K, x_s, w_s, grad_s,
+    x_f8, w_f8 = x_f8.contiguous(), w_f8.contiguous()     # bound to names: the copies outlive the launch
+    _lib.check(lib.ngpt_mm_bwd(_p(g), _p(x_f8), _p(w_f8), M, N, K, x_s, w_s, grad_s,
                                _p(dx), _p(dw), _lib.W_IN_OUT, _p(ws), ws.numel(), _stream(g)), "ngpt_mm_bwd")
     return dx, dw
 
@@ -359,7 +361,7 @@ def _(dy, w2, post):
 
 @torch.library.custom_op("nanogpt::mlp_input_quant", mutates_args=())
 def mlp_input_quant(x: Tensor, up_scale: Tensor) -> tuple[Tensor, Tensor, Tensor]:
-    """(normed, x_f8, dequant) = (rms_norm(x), e4m3(normed * (448 / amax(|normed|))), up_scale * amax / 448) for
+    """(normed, x_f8, dequant) = (rms_norm(x), e4m3(normed * (448.0 / amax(|normed|))), up_scale * amax / 448) for
     bf16 x [..., D]; dequant is a 1-element fp32 device tensor (what the reference keeps in
     `_mlp_dequant_scale_buf`).  Nothing synchronises with the host."""
     _gpu(x, up_scale)

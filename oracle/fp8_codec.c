@@ -17,6 +17,10 @@
  *     fp8(bf16_rne(fp32(x) / fp32(s))) -- the division is IEEE fp32 and its
  *     result is rounded to bf16 before the fp8 cast.
  *
+ *   - the two per-tensor quantisers of the FP8 MLP with every rounding of the eager
+ *     expressions written out (train_gpt.py:1645-1647 and :1419-1422); they pin the
+ *     torch formulations in nanogpt_fp8_oracle.py (tests/test_oracle_math.py).
+ *
  * Pinned by tests/test_oracle_fp8.py: closed-form decode of all 256 codes of
  * each format, encode(decode(c)) == c, monotonicity, tie-to-even at every
  * midpoint between adjacent codes, the overflow thresholds, and agreement
@@ -164,4 +168,49 @@ void ngpt_oracle_gemm_tn_codes(const uint8_t* A, const uint8_t* B, double* C,
             }
             C[(int64_t)m * N + n] = acc * scale;
         }
+}
+
+static float bf16_round(float f) { return ngpt_oracle_bf16_to_f32(ngpt_oracle_f32_to_bf16(f)); }
+
+/* max |v| over n bf16 values, clamped below by bf16(1e-12): `t.abs().max().clamp(min=1e-12)` on a bf16 tensor. */
+static float bf16_amax_clamped(const uint16_t* v, int64_t n) {
+    float m = 0.0f;
+    for (int64_t i = 0; i < n; ++i) {
+        float a = fabsf(ngpt_oracle_bf16_to_f32(v[i]));
+        if (a > m) m = a;
+    }
+    float lo = bf16_round(1.0e-12f);
+    return m < lo ? lo : m;
+}
+
+/*
+ * MLP input quantiser, train_gpt.py:1645-1647, every bf16 operation of the eager expressions rounding:
+ *   amax    = normed.abs().max().clamp(min=1e-12)                    bf16
+ *   q       = 448.0 / amax = bf16(bf16(1 / amax) * 448)             (float / Tensor is reciprocal() * float)
+ *   x_f8    = e4m3fn(bf16(normed * q))
+ *   dequant = (up_scale * amax) / 448                                fp32, in-place mul_ then div_
+ */
+void ngpt_oracle_mlp_input_quant(const uint16_t* normed, int64_t n, float up_scale, uint8_t* x_f8, float* dequant) {
+    float amax = bf16_amax_clamped(normed, n);
+    float q = bf16_round(bf16_round(1.0f / amax) * 448.0f);
+    for (int64_t i = 0; i < n; ++i)
+        x_f8[i] = ngpt_oracle_f32_to_e4m3fn(bf16_round(ngpt_oracle_bf16_to_f32(normed[i]) * q));
+    float d = up_scale * amax;
+    *dequant = d / 448.0f;
+}
+
+/*
+ * Up-projection weight quantiser, train_gpt.py:1419-1422, per layer l of w [layers, per_layer] bf16:
+ *   scale[l] = bf16(amax_l / 448)  with amax_l = max |w_l| clamped below by bf16(1e-12)   (bf16 tensor / float)
+ *   w_f8[l]  = e4m3fn(bf16(w_l / scale[l]))                                                 (bf16 tensor / bf16 tensor)
+ * scales are returned as fp32 (`up_scales.float()`).
+ */
+void ngpt_oracle_quant_up_weights(const uint16_t* w, int layers, int64_t per_layer, uint8_t* w_f8, float* scales) {
+    for (int l = 0; l < layers; ++l) {
+        const uint16_t* wl = w + (int64_t)l * per_layer;
+        float scale = bf16_round(bf16_amax_clamped(wl, per_layer) / 448.0f);
+        scales[l] = scale;
+        for (int64_t i = 0; i < per_layer; ++i)
+            w_f8[(int64_t)l * per_layer + i] = ngpt_oracle_f32_to_e4m3fn(bf16_round(ngpt_oracle_bf16_to_f32(wl[i]) / scale));
+    }
 }

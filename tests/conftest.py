@@ -34,7 +34,8 @@ def fp8_tables(golden_dir):
 def oracle_c():
     """ctypes handle on the C part of the oracle (built on demand; CPU only)."""
     so = ROOT / "oracle" / "libngpt_oracle.so"
-    if not so.exists():
+    src = ROOT / "oracle" / "fp8_codec.c"
+    if not so.exists() or (src.exists() and src.stat().st_mtime > so.stat().st_mtime):
         subprocess.check_call(["make", "-C", str(ROOT / "oracle")])
     lib = ctypes.CDLL(str(so))
     u8, u16, f32 = ctypes.c_uint8, ctypes.c_uint16, ctypes.c_float
@@ -56,6 +57,10 @@ def oracle_c():
     lib.ngpt_oracle_encode_f32.argtypes = [vp, vp, ctypes.c_int64, ctypes.c_int]
     lib.ngpt_oracle_gemm_tn_codes.restype = None
     lib.ngpt_oracle_gemm_tn_codes.argtypes = [vp, vp, vp] + [ctypes.c_int] * 5 + [ctypes.c_double]
+    lib.ngpt_oracle_mlp_input_quant.restype = None
+    lib.ngpt_oracle_mlp_input_quant.argtypes = [vp, ctypes.c_int64, f32, vp, vp]
+    lib.ngpt_oracle_quant_up_weights.restype = None
+    lib.ngpt_oracle_quant_up_weights.argtypes = [vp, ctypes.c_int, ctypes.c_int64, vp, vp]
     return lib
 
 

@@ -22,8 +22,13 @@ def amd():
     return modded_nanogpt_amd
 
 
-def declared_symbols():
+def declared_symbols(bench_only=False):
     text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    bench = "".join(re.findall(r"#ifdef NGPT_BENCH_BUILD(.*?)#endif", text, flags=re.S))
+    if bench_only:
+        text = bench
+    else:
+        text = re.sub(r"#ifdef NGPT_BENCH_BUILD.*?#endif", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(ngpt_[a-z0-9_]+)\s*\(", text)))
 
 
@@ -35,6 +40,39 @@ def test_header_symbols_are_exported_and_bound(amd):
         assert hasattr(lib, n), f"{n} declared in include/ngpt_fp8.h but not exported"
     assert sorted(amd._lib.SIGNATURES) == names, "ctypes table and header disagree"
     assert amd._lib.load().ngpt_abi_version() == 1
+
+
+def test_timing_aids_are_in_the_measurement_build_only(amd):
+    """ngpt_tuning_set and the discarding epilogue flip process-global state and give meaningless results: the shipped
+    library must not export them; the measurement build (same sources, -DNGPT_BENCH_BUILD) has them on top."""
+    aids = declared_symbols(bench_only=True)
+    assert aids == sorted(amd._lib.BENCH_SIGNATURES) and "ngpt_tuning_set" in aids
+    lib = ctypes.CDLL(str(amd._lib.LIB_PATH))
+    for n in aids:
+        assert not hasattr(lib, n), f"{n} must not be exported by the default library"
+    # out_kind 3 (discard) is refused by the default build before anything is enqueued
+    assert amd._lib.load().ngpt_gemm_fp8_tn(1, 0, 128, 1, 0, 128, 4, 4, 128, 1.0, 1, 4, 3, None) == -1
+    if not amd._lib.BENCH_LIB_PATH.exists():
+        from modded_nanogpt_amd.build import build
+        build(verbose=False, bench=True)
+    bench = ctypes.CDLL(str(amd._lib.BENCH_LIB_PATH))
+    for n in aids + declared_symbols():
+        assert hasattr(bench, n), n
+
+
+def test_softcap_guard_is_host_only(amd):
+    """The CE kernels' lookup tables assume that sigma no longer changes beyond |logit| = 256 and sum exponentials
+    relative to the cap: constants that break this are refused (never a silently wrong loss), without a GPU."""
+    lib = amd._lib.load()
+    assert lib.ngpt_softcap_supported(23.0, 5.0, 7.5) == 0            # the reference's constants
+    assert lib.ngpt_softcap_supported(30.0, 0.0, 7.5) == 0            # 15 * tanh(x / 15) + 15
+    assert lib.ngpt_softcap_supported(23.0, 5.0, 1000.0) == -4        # sigma far from saturated at |l| = 256
+    assert b"outside what the lookup tables cover" in lib.ngpt_last_error()
+    assert lib.ngpt_softcap_supported(200.0, 5.0, 7.5) == -4          # exp(-A) underflows
+    assert lib.ngpt_softcap_supported(23.0, 5.0, 0.0) == -4 and lib.ngpt_softcap_supported(float("nan"), 5.0, 7.5) == -4
+    assert lib.ngpt_softcap_supported(23.0, -300.0, 7.5) == -4        # shifted so far that sigma(255) has not reached 1
+    # the entry points apply the same check before they enqueue anything
+    assert lib.ngpt_ce_fwd_bwd(1, 1, 1, None, None, 1, 1, 4, 64, 1, 23.0, 5.0, 1000.0, 1.0, 1.0, 1, 1 << 20, None) == -4
 
 
 def test_argument_errors_do_not_need_a_gpu(amd):

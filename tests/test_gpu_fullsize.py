@@ -168,14 +168,15 @@ def test_config2_mlp_forward_full_size(amd, oracle):
     assert _rel(out.cpu()[0, rows], out_ref) <= GEMM_TOL
 
 
-def test_config4_mlp_backward_full_size(amd, oracle):
-    """FP8 MLP forward + bf16 backward at M = 49152 (one layer of benchmark configuration 4).  dpre and dx are
+@pytest.mark.parametrize("M,D,H", [(49152, 768, 3072), (65536, 1024, 4096)])
+def test_config4_mlp_backward_full_size(amd, oracle, M, D, H):
+    """FP8 MLP forward + bf16 backward at M = 49152 (one layer of benchmark configuration 4) and at the medium-track
+    shape M = 65536, D = 1024, H = 4096 (the MLP half of configuration 5).  dpre and dx are
     row-local: a row sample against the oracle.  The weight gradients contract over all tokens: against an
     fp32 product of the kernel's own post / dpre on the GPU (the plain reference for a floating-point
     contraction), and as the sum of the gradients of the two token halves (additivity, which also
     exercises the sliced contraction at a second size)."""
     g = torch.Generator().manual_seed(4)
-    M, D, H = 49152, 768, 3072
     d = "cuda"
     x_raw = torch.randn(M, D, generator=g).bfloat16()
     w_fc = (torch.randn(H, D, generator=g) / math.sqrt(D)).bfloat16()
@@ -199,8 +200,10 @@ def test_config4_mlp_backward_full_size(amd, oracle):
     dyd = dy.to(d)
     dpre = torch.ops.nanogpt.fc_relu2_bwd_dpre(dyd, w_proj_t.to(d), post)
     torch.cuda.synchronize()
-    # row-local parts on a sample of rows
+    # row-local parts on a sample of rows: the forward's post against the oracle's on the same fp8 operands, then the backward
     rows = torch.cat([torch.arange(0, M, 1531), torch.arange(M - 16, M)]).unique()
+    post_ref = oracle.fc_relu2_fwd(x_f8_all.cpu()[rows], w_f8.cpu()[0], dequant.cpu())
+    assert _rel(post.cpu()[rows], post_ref) <= GEMM_TOL
     dpre_ref = oracle.fc_relu2_bwd_dpre(dy[rows], w_proj_t, post.cpu()[rows])
     assert _rel(dpre.cpu()[rows], dpre_ref) <= GEMM_TOL
     dx_ref = (dpre_ref.float() @ w_fc.float()).bfloat16()
@@ -216,6 +219,39 @@ def test_config4_mlp_backward_full_size(amd, oracle):
     _, _, _, dw1_b, dw2_b = run(slice(M // 2, M))
     assert _rel(dw2_a.float() + dw2_b.float(), dw2.float()) <= GEMM_TOL
     assert _rel(dw1_a.float() + dw1_b.float(), dw1.float()) <= GEMM_TOL
+
+
+def test_config4_twelve_layers_back_to_back(amd):
+    """Benchmark configuration 4 as worded: twelve layers with their own weights, forward + backward, enqueued back
+    to back on one stream without a synchronisation in between.  Every layer's outputs and gradients must be what
+    the same layer gives when it runs alone (split tiles meet through fp32 atomics, whose order is free)."""
+    g = torch.Generator().manual_seed(12)
+    M, D, H, L = 49152, 768, 3072, 12
+    d = "cuda"
+    x_raw = (torch.randn(M, D, generator=g) * 2).bfloat16().to(d)
+    dy = (torch.randn(1, M, D, generator=g) * 1e-3).bfloat16().to(d)
+    w_fc = [(torch.randn(H, D, generator=g) / math.sqrt(D)).bfloat16().to(d) for _ in range(L)]
+    w_pt = [(torch.randn(D, H, generator=g) / math.sqrt(H)).bfloat16().T.contiguous().to(d) for _ in range(L)]
+    w_f8, scales = torch.ops.nanogpt.quant_up_weights(torch.stack(w_fc))
+
+    def layer(l):
+        x = x_raw.clone().requires_grad_(True)
+        w1, w2 = w_fc[l].clone().requires_grad_(True), w_pt[l].clone().requires_grad_(True)
+        normed, x_f8, dequant = torch.ops.nanogpt.mlp_input_quant(x, scales[l:l + 1])
+        out = amd.ReLUSqrdMLP(normed[None], w1, w2, w_f8[l], dequant, x_f8[None])
+        out.backward(dy)
+        return [out.detach(), x.grad, w1.grad, w2.grad]
+
+    together = [layer(l) for l in range(L)]          # nothing synchronises between the layers
+    torch.cuda.synchronize()
+    for l in (0, 5, 11):
+        alone = layer(l)
+        torch.cuda.synchronize()
+        for got, ref in zip(together[l], alone):
+            assert torch.isfinite(got.float()).all()
+            assert _rel(got, ref) <= 1e-5, f"layer {l}"
+    # layers differ from each other (own weights): a result that leaked from a neighbour would not pass the check above
+    assert _rel(together[0][2], together[11][2]) > 0.5
 
 
 @pytest.mark.parametrize("layout", ["out_in", "in_out"])

@@ -253,3 +253,68 @@ def test_down_projection_requantiser_oracle(oracle):
     p = torch.tensor([[0.0, 3.0, 1.0], [0.0, 0.0, 0.0]])
     s = oracle.reduce_mlp_activation_scales(p, headroom=1.8)
     assert torch.allclose(s, torch.tensor([3.0 * 1.8 / 448, 1e-12 * 1.8 / 448]))
+
+
+def test_ce_grad_columns_is_a_column_slice_of_ce_fwd_bwd(oracle):
+    """ce_grad_columns (the checker of the full-size dW tests) must store exactly the codes ce_fwd_bwd stores
+    in those columns -- target columns included -- given the rows' log-sum-exp."""
+    for seed, scale, grad_s, grad_scale in ((14, 4.0, 0.75 / 448, 1.0), (15, 1.0, 2.0 ** -14, 3.0)):
+        logits, targets = _ce_inputs(M=64, V=512, seed=seed, scale=scale)
+        M, V = logits.shape
+        targets[3], targets[9] = -1, V + 5                      # invalid targets contribute nothing
+        losses, dl, lse = oracle.ce_fwd_bwd(logits, targets, torch.tensor([1.0]), torch.full((M,), -1), torch.zeros(1),
+                                            M, 1, 23.0, 5.0, 7.5, grad_s, grad_scale)
+        g = torch.Generator().manual_seed(seed)
+        cols = torch.unique(torch.cat([torch.randperm(V, generator=g)[:96], targets[(targets >= 0) & (targets < V)][:40]]))
+        hits = int((targets.unsqueeze(1) == cols.unsqueeze(0)).sum())
+        assert hits >= 40                                        # the subset does contain target columns
+        sub = oracle.ce_grad_columns(logits[:, cols].contiguous(), cols, lse, targets, 23.0, 5.0, 7.5, grad_s, grad_scale)
+        assert sub.dtype == torch.float8_e5m2
+        assert torch.equal(sub.view(torch.uint8), dl[:, cols].contiguous().view(torch.uint8))
+        # a dropped one-hot term would change exactly the target entries
+        wrong = oracle.ce_grad_columns(logits[:, cols].contiguous(), cols, lse, torch.full_like(targets, -1), 23.0, 5.0, 7.5,
+                                       grad_s, grad_scale)
+        assert int((wrong.view(torch.uint8) != sub.view(torch.uint8)).sum()) >= hits // 2
+
+
+def _bf16_bits(t):
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def test_mlp_quantisers_round_where_eager_rounds(oracle, oracle_c):
+    """mlp_input_quant and quantize_up_weights are torch expressions; the scalar C restatement writes every rounding
+    out (448.0 / amax is reciprocal() * 448 in eager, each bf16 operation rounds).  They must agree bit for bit, and
+    the inputs are chosen so that the plausible mistakes (one division, no intermediate rounding) do change codes."""
+    import ctypes
+    differs_single_div = differs_no_round = 0
+    for seed in range(12):
+        g = torch.Generator().manual_seed(100 + seed)
+        normed = oracle.rms_norm((torch.randn(64, 96, generator=g) * (1 + seed)).bfloat16())
+        if seed == 11:
+            normed = torch.zeros(8, 16).bfloat16()               # amax clamps to bf16(1e-12)
+        up_scale = torch.tensor([0.0123 * (seed + 1)])
+        x_f8, dequant = oracle.mlp_input_quant(normed, up_scale)
+        n = normed.numel()
+        out = np.empty(n, dtype=np.uint8)
+        dq = ctypes.c_float(0)
+        oracle_c.ngpt_oracle_mlp_input_quant(_bf16_bits(normed).ctypes.data, n, float(up_scale), out.ctypes.data, ctypes.byref(dq))
+        assert np.array_equal(out, x_f8.view(torch.uint8).numpy().ravel()), seed
+        assert dq.value == float(dequant), seed
+        # the two mistakes this guards against
+        amax = normed.float().abs().max().clamp(min=1e-12)
+        one_div = (normed.float() * (448.0 / amax).bfloat16().float()).bfloat16().to(torch.float8_e4m3fn)
+        no_round = (normed.float() * (448.0 / amax)).to(torch.float8_e4m3fn)
+        differs_single_div += int(not torch.equal(one_div.view(torch.uint8), x_f8.view(torch.uint8)))
+        differs_no_round += int(not torch.equal(no_round.view(torch.uint8), x_f8.view(torch.uint8)))
+    assert differs_single_div >= 1 and differs_no_round >= 1
+
+    g = torch.Generator().manual_seed(200)
+    w = (torch.randn(5, 48, 64, generator=g) * torch.tensor([0.02, 0.5, 3.0, 1e-3, 0.0]).view(5, 1, 1)).bfloat16()
+    w_f8, scales = oracle.quantize_up_weights(w)
+    out = np.empty(w.numel(), dtype=np.uint8)
+    sc = np.empty(5, dtype=np.float32)
+    oracle_c.ngpt_oracle_quant_up_weights(_bf16_bits(w).ctypes.data, 5, 48 * 64, out.ctypes.data, sc.ctypes.data)
+    assert np.array_equal(out, w_f8.view(torch.uint8).numpy().ravel())
+    assert np.array_equal(sc, scales.numpy())
+    no_round = (w.float() / (w.float().reshape(5, -1).abs().amax(1).clamp(min=1e-12) / 448).view(5, 1, 1)).to(torch.float8_e4m3fn)
+    assert not torch.equal(no_round.view(torch.uint8), w_f8.view(torch.uint8))
