@@ -128,6 +128,11 @@ int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, 
                       void* post_bf16, void* post_f8, const float* act_scale,
                       float* partial_amax, int n_partials, void* stream);
 
+/* The same kernel on bf16 operands (FORWARD without USE_FP8, the reference's DISABLE_FP8 path, launched at
+ * triton_kernels.py:716-718): post [M,N] = bf16(max(bf16(x . w^T), 0)^2) for x [M,K], w [N,K] bf16.
+ * K % 64 == 0, N % 8 == 0. */
+int ngpt_linear_relu2_bf16(const void* x_bf16, const void* w_bf16, int M, int N, int K, void* post_bf16, void* stream);
+
 /* ---- MLP backward through ReLU^2 ----------------------------------------------------------
  * linear_relu_square_kernel with FORWARD = False, triton_kernels.py:472-476, 493-496, called at :726.
  * dy [M, D] bf16, w2 [H, D] bf16, post [M, H] bf16 ->
@@ -135,6 +140,22 @@ int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, 
  * product fused into the epilogue.  D % 64 == 0. */
 int ngpt_fc_relu2_bwd_dpre(const void* dy_bf16, const void* w2_bf16, const void* post_bf16, int M, int H, int D,
                            void* dpre_bf16, void* stream);
+
+/* ---- the plain bf16 products of the MLP ----------------------------------------------------
+ * out[r, c] = bf16(sum_k A(r, k) * B(c, k)), fp32 accumulation, one rounding.  Each operand is a row-major bf16
+ * matrix in one of two layouts: NGPT_K_CONTIGUOUS = stored [rows, K] (contraction contiguous, leading dimension
+ * >= K), NGPT_K_ROWS = stored [K, rows] (the contraction index is the row, leading dimension >= rows), read
+ * through transposing LDS loads without a transposed copy.  Leading dimensions in elements.  Replaces the four
+ * cuBLAS products of FusedLinearReLUSquareFunction, triton_kernels.py:715 (`post @ W2`: A = post K_CONTIGUOUS,
+ * B = W2 K_ROWS), :723 (`post.T @ grad_output`: both K_ROWS, contraction over the tokens), :727 (`dpre.T @ x`)
+ * and :728 (`dpre @ W1`).  Few output tiles with a long contraction are cut along it and meet in fp32.
+ * K % 64 == 0, R % 8 == 0, C % 8 == 0.  workspace: ngpt_gemm_bf16_workspace_bytes(R, C, K) bytes. */
+#define NGPT_K_CONTIGUOUS  0
+#define NGPT_K_ROWS        1
+int64_t ngpt_gemm_bf16_workspace_bytes(int R, int C, int K);
+int ngpt_gemm_bf16(const void* A, int a_layout, int64_t lda, const void* B, int b_layout, int64_t ldb,
+                   int R, int C, int K, void* out_bf16, int64_t ldc, void* workspace, int64_t workspace_bytes,
+                   void* stream);
 
 /* ---- delayed-scaling bookkeeping of the FP8 down projection, tied-embedding gradient add -----
  * scales[l] = max(max_i partial_amax[l * partial_stride + i], 1e-12) * headroom / 448:

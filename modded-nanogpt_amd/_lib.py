@@ -15,6 +15,7 @@ BENCH_SIGNATURES = {
 
 E4M3, E5M2 = 0, 1
 W_OUT_IN, W_IN_OUT = 0, 1
+K_CONTIGUOUS, K_ROWS = 0, 1
 MAX_PREDICT = 4
 
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
@@ -36,7 +37,10 @@ SIGNATURES = {
     "ngpt_mm_bwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
     "ngpt_mm_bwd": (_I, [_P, _P, _P, _I, _I, _I, _F, _F, _F, _P, _P, _I, _P, _L, _P]),
     "ngpt_fc_relu2_fwd": (_I, [_P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _P]),
+    "ngpt_linear_relu2_bf16": (_I, [_P, _P, _I, _I, _I, _P, _P]),
     "ngpt_fc_relu2_bwd_dpre": (_I, [_P, _P, _P, _I, _I, _I, _P, _P]),
+    "ngpt_gemm_bf16_workspace_bytes": (_L, [_I, _I, _I]),
+    "ngpt_gemm_bf16": (_I, [_P, _I, _L, _P, _I, _L, _I, _I, _I, _P, _L, _P, _L, _P]),
     "ngpt_reduce_scales": (_I, [_P, _L, _I, _I, _F, _P, _P]),
     "ngpt_quant_transpose_down": (_I, [_P, _I, _I, _I, _L, _P, _P, _P, _P, _P]),
     "ngpt_mlp_input_quant_workspace_bytes": (_L, []),

@@ -290,7 +290,7 @@ struct EpiStoreF32 {
 struct EpiRelu2Lines {
     uint16_t* post;
     int64_t ld;
-    const float* dequant;        // 1-element device tensor
+    const float* dequant;        // 1-element device tensor, or null for a scale of one (bf16 operands)
     int R, C;                    // R = hidden units (tile rows), C = tokens (tile columns)
     static constexpr int EXTRA_LDS = 32768;
     static constexpr bool NEEDS_SCRATCH = false;
@@ -302,7 +302,7 @@ struct EpiRelu2Lines {
     __device__ bool all_stores_issued() const { return stored_all; }
     __device__ void partial(bool) {}
     __device__ void begin(int, int, uint8_t* extra) {
-        scale = *dequant;
+        scale = dequant ? *dequant : 1.0f;
         stage = extra + (threadIdx.x >> 6) * 4096;
         stored_all = false;
     }

@@ -378,6 +378,46 @@ extern "C" int ngpt_fc_relu2_bwd_dpre(const void* dy_bf16, const void* w2_bf16, 
     return launch_gemm_fmt<MainCfg, FMT_BF16, FMT_BF16>(g, epi, (hipStream_t)stream, 0);
 }
 
+// ------------------------------------------------------------------------------------------ plain bf16 GEMM
+// The four bf16 products of FusedLinearReLUSquareFunction besides dpre (triton_kernels.py:715, 723, 727, 728).
+extern "C" int64_t ngpt_gemm_bf16_workspace_bytes(int R, int C, int K) {
+    (void)K;
+    return align_up((int64_t)R * C * 4, 256);
+}
+
+extern "C" int ngpt_gemm_bf16(const void* A, int a_layout, int64_t lda, const void* B, int b_layout, int64_t ldb,
+                              int R, int C, int K, void* out_bf16, int64_t ldc, void* workspace, int64_t workspace_bytes,
+                              void* stream) {
+    if (!A || !B || !out_bf16 || !workspace) return fail(NGPT_EINVAL, "ngpt_gemm_bf16: null pointer");
+    if (R <= 0 || C <= 0 || K <= 0) return fail(NGPT_EINVAL, "ngpt_gemm_bf16: empty problem R=%d C=%d K=%d", R, C, K);
+    if ((a_layout | b_layout) & ~1) return fail(NGPT_EINVAL, "ngpt_gemm_bf16: a_layout=%d b_layout=%d", a_layout, b_layout);
+    if (K % 64 || R % 8 || C % 8)
+        return fail(NGPT_EALIGN, "ngpt_gemm_bf16: need K %% 64 == 0, R %% 8 == 0, C %% 8 == 0 (R=%d C=%d K=%d)", R, C, K);
+    const int64_t min_lda = a_layout == NGPT_K_CONTIGUOUS ? K : R, min_ldb = b_layout == NGPT_K_CONTIGUOUS ? K : C;
+    if (lda % 8 || ldb % 8 || lda < min_lda || ldb < min_ldb || ldc < C || ldc % 4)
+        return fail(NGPT_EALIGN, "ngpt_gemm_bf16: leading dimensions lda=%lld ldb=%lld ldc=%lld", (long long)lda, (long long)ldb, (long long)ldc);
+    if (workspace_bytes < ngpt_gemm_bf16_workspace_bytes(R, C, K))
+        return fail(NGPT_EWORKSPACE, "ngpt_gemm_bf16: workspace %lld < %lld bytes", (long long)workspace_bytes,
+                    (long long)ngpt_gemm_bf16_workspace_bytes(R, C, K));
+    // the loader works in bytes: contraction length and row strides are 2 x the element counts
+    const int fa = a_layout == NGPT_K_CONTIGUOUS ? FMT_BF16 : (FMT_BF16 | FMT_TRANSPOSED);
+    const int fb = b_layout == NGPT_K_CONTIGUOUS ? FMT_BF16 : (FMT_BF16 | FMT_TRANSPOSED);
+    return gemm_balanced_bf16(A, fa, 2 * lda, B, fb, 2 * ldb, 0, R, C, 2 * K, 1.0f, out_bf16, ldc, (float*)workspace, 0,
+                              (hipStream_t)stream);
+}
+
+// post [M, N] = bf16(max(bf16(x . w^T), 0)^2) on bf16 operands: linear_relu_square_kernel FORWARD without USE_FP8
+// (triton_kernels.py:402-499 as launched at :716-718 when no fp8 copies are passed).  Same transposed product and
+// whole-line stores as the FP8 c_fc.
+extern "C" int ngpt_linear_relu2_bf16(const void* x_bf16, const void* w_bf16, int M, int N, int K, void* post_bf16, void* stream) {
+    if (!x_bf16 || !w_bf16 || !post_bf16) return fail(NGPT_EINVAL, "ngpt_linear_relu2_bf16: null pointer");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(NGPT_EINVAL, "ngpt_linear_relu2_bf16: empty problem M=%d N=%d K=%d", M, N, K);
+    if (K % 64 || N % 8) return fail(NGPT_EALIGN, "ngpt_linear_relu2_bf16: need K %% 64 == 0 and N %% 8 == 0 (N=%d K=%d)", N, K);
+    GemmOperands gt{(const uint8_t*)w_bf16, (const uint8_t*)x_bf16, 2 * (int64_t)K, 2 * (int64_t)K, N, M, 2 * K, 1, 0};
+    EpiRelu2Lines epi{(uint16_t*)post_bf16, N, nullptr, N, M};
+    return launch_gemm_fmt<MainCfg, FMT_BF16, FMT_BF16>(gt, epi, (hipStream_t)stream, 0);
+}
+
 // ------------------------------------------------------------------------------------------ fc + relu^2
 extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, int M, int N, int K,
                                  void* post_bf16, void* post_f8, const float* act_scale,

@@ -39,6 +39,10 @@ namespace ngpt {
 // k-step of a tile then reads two contiguous 16 KiB pieces (128 contraction rows x 128 output rows each).
 // kRowsPermuted: the 128-byte rows of a transposed A panel hold the output rows of every 32-group in dw_pos
 // order (panel.h); the epilogue's row arithmetic undoes it (AccCoords::perm).
+// Transposed bf16 operand (FMT_BF16 | FMT_TRANSPOSED, either operand): the pointer is a row-major matrix with the
+// CONTRACTION index as its rows (row stride lda / ldb BYTES) and this operand's output rows / columns contiguous,
+// i.e. C = A^T . B style products without a transposed copy.  One k-step = 64 contraction rows x 256 bf16 = 32 KiB;
+// the contraction length must be a multiple of 64 rows, R / C multiples of 8.
 constexpr int kBlockedA = 1, kBlockedB = 2, kRowsPermuted = 4;
 constexpr int kPanelRows = 256, kPanelBytes = kPanelRows * 128;
 
@@ -128,10 +132,22 @@ __device__ __forceinline__ void wait_vmem_le() {
 template <class Cfg>
 struct LaneOffsets {
     uint32_t a_off[Cfg::A_LOADS], b_off[Cfg::B_LOADS];   // byte offset of this lane's chunk from the tile's first row
-    __device__ void init(const GemmOperands& g, int wave, int lane, int r0, int c0, bool a_transposed) {
+    // Transposed bf16 slab: LDS row = contraction row (64 per k-step) of 512 bytes = 32 chunks; one wave-level load
+    // covers two rows.  The chunk stored at position p of row m is global chunk p ^ (4 * (m & 3)): with it the 32
+    // lanes that a transposing read serves together hit 32 distinct 8-byte bank pairs (see frag offsets below).
+    // `lim` = columns of this operand left from the tile's origin (a multiple of 8): chunks past it are clamped.
+    static __device__ uint32_t tr16_off(int load, int wave, int lane, int64_t ld, int lim) {
+        const int m = 2 * (wave + load * Cfg::NWAVES) + (lane >> 5);
+        int chunk = (lane & 31) ^ (4 * (m & 3));
+        chunk = min(chunk, lim / 8 - 1);
+        return (uint32_t)((int64_t)m * ld + chunk * 16);
+    }
+    __device__ void init(const GemmOperands& g, int wave, int lane, int r0, int c0, bool a_transposed, bool a_tr16 = false,
+                         bool b_tr16 = false) {
         int lrow = lane / Cfg::CPR, lchunk = lane % Cfg::CPR;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i) {
+            if (a_tr16) { a_off[i] = tr16_off(i, wave, lane, g.lda, g.R - r0); continue; }
             if (a_transposed) {
                 // 1 KiB piece `c32` of the k-step's 32: half (token block) c32 / 16, contraction rows 8 * (c32 % 16) ..+7;
                 // the 16-byte chunk q of contraction row r lands at chunk position q ^ (r & 7)
@@ -148,6 +164,7 @@ struct LaneOffsets {
         }
 #pragma unroll
         for (int i = 0; i < Cfg::B_LOADS; ++i) {
+            if (b_tr16) { b_off[i] = tr16_off(i, wave, lane, g.ldb, g.C - c0); continue; }
             int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
             int q = lchunk ^ Cfg::swz(R);
             if (g.layout & kBlockedB) { b_off[i] = (uint32_t)(R * 128 + q * 16); continue; }
@@ -170,7 +187,12 @@ struct TileMainloop {
     int a_kt;                // transposed A: index of the next k-step to load; a_next then is the tile's base
     int64_t a_pair_stride;   // transposed A: bytes between the panel rows of two consecutive 256-blocks of the contraction
     int wave, lane, wr, wc;
-    static constexpr bool ATR = (AFMT & FMT_TRANSPOSED) != 0;
+    static constexpr bool BF16 = (AFMT & 3) == FMT_BF16;
+    static constexpr bool ATR = (AFMT & FMT_TRANSPOSED) != 0 && !BF16;      // fp8 A given as the panel of its transpose
+    static constexpr bool ATR16 = (AFMT & FMT_TRANSPOSED) != 0 && BF16;     // bf16 operands with the contraction as rows
+    static constexpr bool BTR16 = (BFMT & FMT_TRANSPOSED) != 0 && BF16;
+    static_assert(!(BFMT & FMT_TRANSPOSED) || BF16, "a transposed B operand exists for bf16 only");
+    static_assert(!(ATR16 || BTR16) || (Cfg::BM == 256 && Cfg::BN == 256 && Cfg::BK == 128), "transposed bf16 slabs are 64 x 256");
 
     __device__ void init() {
         int tid = threadIdx.x;
@@ -182,11 +204,12 @@ struct TileMainloop {
         wc = wave % Cfg::WAVES_N;
         // first 16-byte chunk of this lane's operand fragment: fp8 MFMAs (32x32x64) take 32 bytes per
         // lane (chunks 2h, 2h+1), the bf16 MFMA (32x32x16) takes 16 bytes (chunk h)
-        int q0 = (AFMT == FMT_BF16) ? (lane >> 5) : (lane >> 5) * 2;
+        int q0 = BF16 ? (lane >> 5) : (lane >> 5) * 2;
 #pragma unroll
         for (int t = 0; t < Cfg::TM; ++t) {
             int row = wr * Cfg::WTM + t * 32 + (lane & 31);
             frag_a[t] = row * Cfg::BK + ((q0 ^ Cfg::swz(row)) << 4);
+            if (ATR16) frag_a[t] = tr16_frag(wr * Cfg::WTM + t * 32);
             if (ATR) {
                 // Source address of this lane for the transposing read (ds_read_b64_tr_b8: inside each block
                 // of 16 lanes, lane i receives byte i % 8 of the 8-byte rows of lanes 2j + i / 8, j = 0..7).
@@ -204,7 +227,21 @@ struct TileMainloop {
         for (int t = 0; t < Cfg::TN; ++t) {
             int row = wc * Cfg::WTN + t * 32 + (lane & 31);
             frag_b[t] = Cfg::A_BYTES + row * Cfg::BK + ((q0 ^ Cfg::swz(row)) << 4);
+            if (BTR16) frag_b[t] = Cfg::A_BYTES + tr16_frag(wc * Cfg::WTN + t * 32);
         }
+    }
+    // Source address of this lane for the transposing 16-bit read (ds_read_b64_tr_b16: inside each block of 16
+    // lanes, lane i receives element i % 4 of the 4-element rows of lanes 4j + i / 4, j = 0..3).  Lane s of a
+    // block supplies contraction row s / 4 and output rows 4 * (s % 4) ..+3, so lane i ends up with 4 consecutive
+    // contraction elements of output row i.  Blocks 0, 1 serve rows 0..15, 16..31 of the MFMA tile for the first 8
+    // of a sub-step's 16 contraction rows (two reads, 4 rows = 2 KiB apart), blocks 2, 3 the same for the second 8:
+    // a lane half holds its 8 contraction elements in natural order, as a row-major operand's 16-byte chunk does.
+    // `row0`: first output row of the MFMA tile inside the workgroup tile.
+    __device__ int tr16_frag(int row0) const {
+        const int s = lane & 15, blk = lane >> 4;
+        const int m = 8 * (blk >> 1) + (s >> 2);                      // contraction row inside the sub-step; m & 3 == s >> 2
+        const int byte = 2 * (row0 + 16 * (blk & 1) + 4 * (s & 3));   // inside the 512-byte row
+        return m * 512 + ((((byte >> 4) ^ (4 * (s >> 2))) << 4) | (byte & 15));
     }
 
     // Point the loads at tile (r0, c0).  Rows past the end are clamped to the last row: they are
@@ -223,7 +260,15 @@ struct TileMainloop {
             a_pair_stride = (int64_t)(g.a_rows_pad >> 7) * kPanelBytes;
             a_kt = kt;
         }
-        lo.init(g, wave, lane, r0, c0, ATR);
+        if (ATR16) {   // 64 contraction rows per k-step, the tile's rows start 2 * r0 bytes into each
+            a_step = (int)(64 * g.lda);
+            a_next = g.A + 2 * (int64_t)r0 + (int64_t)kt * a_step;
+        }
+        if (BTR16) {
+            b_step = (int)(64 * g.ldb);
+            b_next = g.B + 2 * (int64_t)c0 + (int64_t)kt * b_step;
+        }
+        lo.init(g, wave, lane, r0, c0, ATR, ATR16, BTR16);
     }
 
     // Loads the next k-step of the current tile into LDS slot `stage` and moves on to the one after: the A
@@ -296,6 +341,48 @@ struct TileMainloop {
         }
     }
 
+    // bf16 fragments (16 bytes per lane and MFMA tile) of contraction sub-step KS (16 elements) as inline assembly:
+    // a transposed operand takes two transposing 8-byte reads 4 contraction rows (2 KiB) apart, a row-major one
+    // one 16-byte read of chunk (2 KS + lane half) of its swizzled 128-byte row.
+    template <int OFF>
+    static __device__ __forceinline__ v2i read_tr16(uint32_t lds_addr) {
+        v2i r;
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(lds_addr), "n"(OFF));
+        return r;
+    }
+    static __device__ __forceinline__ v4i read_b128(uint32_t lds_addr) {
+        v4i r;
+        asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(lds_addr));
+        return r;
+    }
+    template <int KS>
+    __device__ __forceinline__ void read_frags16(uint32_t sbase, v4i (&fa)[Cfg::TM], v4i (&fb)[Cfg::TN]) const {
+        static_assert(Cfg::BK == 128 && 3 * 8192 + 2048 < 65536, "16-bit immediate offsets of the transposing reads");
+#pragma unroll
+        for (int t = 0; t < Cfg::TM; ++t) {
+            if constexpr (ATR16) {
+                const v2i lo = read_tr16<KS * 8192>(sbase + (uint32_t)frag_a[t]), hi = read_tr16<KS * 8192 + 2048>(sbase + (uint32_t)frag_a[t]);
+                fa[t] = (v4i){lo.x, lo.y, hi.x, hi.y};
+            } else {
+                fa[t] = read_b128(sbase + (uint32_t)(frag_a[t] ^ (KS * 32)));
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < Cfg::TN; ++t) {
+            if constexpr (BTR16) {
+                const v2i lo = read_tr16<KS * 8192>(sbase + (uint32_t)frag_b[t]), hi = read_tr16<KS * 8192 + 2048>(sbase + (uint32_t)frag_b[t]);
+                fb[t] = (v4i){lo.x, lo.y, hi.x, hi.y};
+            } else {
+                fb[t] = read_b128(sbase + (uint32_t)(frag_b[t] ^ (KS * 32)));
+            }
+        }
+    }
+    // All LDS reads issued so far have returned; ties the fragments to that point.
+    static __device__ __forceinline__ void frag16_fence(v4i (&fa)[Cfg::TM], v4i (&fb)[Cfg::TN]) {
+        static_assert(Cfg::TM == 2 && Cfg::TN == 4, "fragment count of the fence");
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
+    }
+
     // One k-step of MFMAs on the operands in LDS slot `stage`, software-pipelined by hand.
     //  * Fragment reads run one MFMA group (TM MFMAs that share a B fragment) ahead of their use, and
     //    scheduling barriers keep the compiler from hoisting all reads to the top, which would leave
@@ -318,6 +405,37 @@ struct TileMainloop {
             // no fragment hand-over between k-steps
             constexpr int KS = Cfg::BK / 32;
             issue_loads_b(smem);
+            if constexpr (ATR16 || BTR16) {
+                // At least one operand is read through the transposing load.  All fragment reads of this path are
+                // inline assembly (see read_tr8 for why), so the compiler does not count them: frag16_fence() stands
+                // between a sub-step's reads and its MFMAs.  The reads of sub-step ks + 1 are issued behind that
+                // fence and ahead of the MFMAs of ks, which cover their latency.
+                const uint32_t sbase = (uint32_t)(size_t)((const __attribute__((address_space(3))) uint8_t*)s);
+                v4i fa[2][Cfg::TM], fb[2][Cfg::TN];
+                read_frags16<0>(sbase, fa[0], fb[0]);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    frag16_fence(fa[ks & 1], fb[ks & 1]);
+                    if (ks == 0) read_frags16<1>(sbase, fa[1], fb[1]);
+                    if (ks == 1) read_frags16<2>(sbase, fa[0], fb[0]);
+                    if (ks == 2) read_frags16<3>(sbase, fa[1], fb[1]);
+                    if (ks == KS - 1) sync();
+                    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+                    for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+                        for (int tn = 0; tn < Cfg::TN; ++tn) {
+                            const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                __builtin_bit_cast(v8bf, fa[ks & 1][tm]), __builtin_bit_cast(v8bf, fb[ks & 1][tn]),
+                                (FIRST && ks == 0) ? zero : acc[tm][tn], 0, 0, 0);
+                        }
+                    __builtin_amdgcn_s_setprio(0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                refill();
+                return;
+            }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 v8bf fa[Cfg::TM], fb[Cfg::TN];

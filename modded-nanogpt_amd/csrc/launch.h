@@ -46,6 +46,8 @@ int launch_gemm_fmt(const GemmOperands& g, const Epi& epi, hipStream_t st, int m
     if (cus <= 0) return fail(NGPT_EINVAL, "no HIP device");
     int slots = cus * Cfg::WGS_PER_CU;      // as many workgroups as can be resident at once
     int grid = tiles < slots ? tiles : slots;
+    // a multiple of 8 keeps the walk's XCD-aware numbering (TileOrder::seq_of); surplus workgroups find no job and leave
+    if (grid % 8 && (grid + 7) / 8 * 8 <= slots) grid = (grid + 7) / 8 * 8;
     if (max_grid > 0 && grid > max_grid) grid = max_grid;
     kernel<<<grid, Cfg::THREADS, LDS, st>>>(g, epi);
     return check_launch("gemm_tn_kernel");
@@ -55,6 +57,16 @@ struct EpiStoreBf16;
 
 template <class Cfg, class Epi>
 int launch_gemm_cfg(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {
+    if ((fa & 3) == FMT_BF16 || (fb & 3) == FMT_BF16) {   // bf16 x bf16 -> bf16: row-major or contraction-major operands
+        if constexpr (std::is_same<Epi, EpiStoreBf16>::value && std::is_same<Cfg, TileCfg<256, 256, 4, 2, 128, 2>>::value) {
+            constexpr int N = FMT_BF16, T = FMT_BF16 | FMT_TRANSPOSED;
+            if (fa == N && fb == N) return launch_gemm_fmt<Cfg, N, N>(g, epi, st, max_grid);
+            if (fa == N && fb == T) return launch_gemm_fmt<Cfg, N, T>(g, epi, st, max_grid);
+            if (fa == T && fb == T) return launch_gemm_fmt<Cfg, T, T>(g, epi, st, max_grid);
+            if (fa == T && fb == N) return launch_gemm_fmt<Cfg, T, N>(g, epi, st, max_grid);
+        }
+        return fail(NGPT_EINVAL, "bf16 operands: unsupported format / output combination");
+    }
     if (fa & FMT_TRANSPOSED) {   // only the combination the fused CE backward uses is instantiated
         if constexpr (std::is_same<Epi, EpiStoreBf16>::value) {
             if (fa == (FMT_E5M2 | FMT_TRANSPOSED) && fb == FMT_E4M3)

@@ -92,33 +92,15 @@ def linear_relu_square(a, b, aux=None, a_f8=None, b_f8=None, dequant_scale_ptr=N
                 assert partial_amax is not None
                 return ops.fc_relu2_fwd_emit(a_f8, b_f8, dequant_scale_ptr, activation_scale, partial_amax)
             return ops.fc_relu2_fwd(a_f8, b_f8, dequant_scale_ptr)
-        c = a @ b.T                                     # bf16 GEMM (hipBLASLt), fp32 accumulate
-        r = torch.clamp_min(c, 0)
-        return r * r
+        return ops.linear_relu2_bf16(a.contiguous(), b.contiguous())
     return ops.fc_relu2_bwd_dpre(a.contiguous(), b.contiguous(), aux.contiguous())
-
-
-def _tokens_contraction(a: Tensor, b: Tensor) -> Tensor:
-    """a.T @ b for a [M, P], b [M, Q] with the tokens M as contraction (the weight gradients of the MLP,
-    triton_kernels.py:722, 727).  A [P, Q] result is only a few dozen tiles for the library's GEMM, which
-    leaves most of the 256 compute units idle (451 us for 49152 x 3072 x 768); cut into 16 slices of the
-    contraction, the same library runs a batch of 16 such GEMMs in 251 us.  The slices' bf16 results are
-    summed in fp32 (measured: same error against an fp32 product as the single GEMM)."""
-    M = a.shape[0]
-    slices = 16
-    while slices > 1 and (M % slices or M // slices < 2048):
-        slices //= 2
-    if slices == 1:
-        return a.T @ b
-    parts = torch.bmm(a.view(slices, M // slices, a.shape[1]).transpose(1, 2), b.view(slices, M // slices, b.shape[1]))
-    return parts.sum(0, dtype=torch.float32).to(a.dtype)
 
 
 class FusedLinearReLUSquareFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, W1, W2, W1_f8=None, dequant_scale=None, x_f8=None, W2_f8=None, W2_scale=None,
                 activation_scale=None, partial_amax=None):
-        # Forward stores only post = relu(x @ W1.T)^2; `pre` is never materialised.
+        # saved for the backward: post = relu(x @ W1.T)^2 (the pre-activation never reaches memory)
         x_flat = x.view((-1, x.shape[-1]))
         post_f8 = None
         if W1_f8 is not None:
@@ -144,8 +126,8 @@ class FusedLinearReLUSquareFunction(torch.autograd.Function):
             x3 = ops.gemm_fp8_tn_op(post_f8, w2_dh, 1.0, True)
             x3 = (x3 * (activation_scale * W2_scale)).to(torch.bfloat16)
         else:
-            x3 = post @ W2
-        # Backward stays BF16: it consumes `post` (and W2), not their FP8 copies.
+            x3 = ops.gemm_bf16(post, W2, False, True)          # post @ W2, W2 [H, D] read with the contraction as its rows
+        # the backward is all bf16 and needs post and W2 themselves, not the e4m3 copies
         ctx.save_for_backward(x, W1, W2, post)
         return x3.view(x.shape)
 
@@ -154,10 +136,11 @@ class FusedLinearReLUSquareFunction(torch.autograd.Function):
         x, W1, W2, post = ctx.saved_tensors
         x_flat = x.view((-1, x.shape[-1]))
         g = grad_output.reshape((-1, grad_output.shape[-1]))
-        dW2 = _tokens_contraction(post, g)
+        g = g.contiguous()
+        dW2 = ops.gemm_bf16(post, g, True, True)               # post.T @ dY: contraction over the tokens
         dpre = linear_relu_square(g, W2, aux=post)
-        dW1 = _tokens_contraction(dpre, x_flat)
-        dx = dpre @ W1
+        dW1 = ops.gemm_bf16(dpre, x_flat, True, True)          # dpre.T @ x
+        dx = ops.gemm_bf16(dpre, W1, False, True)              # dpre @ W1
         return dx.view(x.shape), dW1, dW2, None, None, None, None, None, None, None
 
 

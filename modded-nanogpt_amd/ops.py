@@ -336,6 +336,52 @@ def _(x_f8, w_f8, dequant_scale, activation_scale, partial_amax):
             torch.empty((M, N), dtype=E4M3, device=x_f8.device))
 
 
+@torch.library.custom_op("nanogpt::linear_relu2_bf16", mutates_args=())
+def linear_relu2_bf16(x: Tensor, w: Tensor) -> Tensor:
+    """post [M,N] bf16 = relu(bf16(x @ w.T))^2 for bf16 x [M,K], w [N,K]: linear_relu_square without fp8 copies."""
+    _gpu(x, w)
+    assert x.dtype == w.dtype == torch.bfloat16 and x.is_contiguous() and w.is_contiguous()
+    M, K = x.shape
+    N = w.shape[0]
+    assert w.shape[1] == K
+    post = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    _lib.check(_lib.load().ngpt_linear_relu2_bf16(_p(x), _p(w), M, N, K, _p(post), _stream(x)), "ngpt_linear_relu2_bf16")
+    return post
+
+
+@linear_relu2_bf16.register_fake
+def _(x, w):
+    return torch.empty((x.shape[0], w.shape[0]), dtype=torch.bfloat16, device=x.device)
+
+
+@torch.library.custom_op("nanogpt::gemm_bf16", mutates_args=())
+def gemm_bf16(a: Tensor, b: Tensor, a_k_rows: bool, b_k_rows: bool) -> Tensor:
+    """out [R, C] bf16 = sum_k A(r, k) B(c, k) with fp32 accumulation and one rounding.  `a` is stored [R, K], or
+    [K, R] when a_k_rows (the contraction index is its row); `b` likewise [C, K] or [K, C].  The four plain products
+    of FusedLinearReLUSquareFunction (reference triton_kernels.py:715, 723, 727, 728):
+        post @ W2      = gemm_bf16(post, W2, False, True)       dpre @ W1 = gemm_bf16(dpre, W1, False, True)
+        post.T @ dY    = gemm_bf16(post, dY, True, True)        dpre.T @ x = gemm_bf16(dpre, x, True, True)"""
+    _gpu(a, b)
+    assert a.dtype == b.dtype == torch.bfloat16 and a.ndim == b.ndim == 2 and a.stride(1) == 1 and b.stride(1) == 1
+    K, R = a.shape if a_k_rows else a.shape[::-1]
+    Kb, C = b.shape if b_k_rows else b.shape[::-1]
+    assert K == Kb, "contraction lengths differ"
+    lib = _lib.load()
+    out = torch.empty((R, C), dtype=torch.bfloat16, device=a.device)
+    ws = _workspace(lib.ngpt_gemm_bf16_workspace_bytes(R, C, K), a.device)
+    _lib.check(lib.ngpt_gemm_bf16(_p(a), _lib.K_ROWS if a_k_rows else _lib.K_CONTIGUOUS, a.stride(0),
+                                  _p(b), _lib.K_ROWS if b_k_rows else _lib.K_CONTIGUOUS, b.stride(0),
+                                  R, C, K, _p(out), C, _p(ws), ws.numel(), _stream(a)), "ngpt_gemm_bf16")
+    return out
+
+
+@gemm_bf16.register_fake
+def _(a, b, a_k_rows, b_k_rows):
+    R = a.shape[1] if a_k_rows else a.shape[0]
+    C = b.shape[1] if b_k_rows else b.shape[0]
+    return a.new_empty((R, C))
+
+
 @torch.library.custom_op("nanogpt::fc_relu2_bwd_dpre", mutates_args=())
 def fc_relu2_bwd_dpre(dy: Tensor, w2: Tensor, post: Tensor) -> Tensor:
     """dpre [M,H] = bf16(2 * bf16(dy @ w2.T) * sqrt(post)) for dy [M,D], w2 [H,D], post [M,H], all bf16."""

@@ -249,7 +249,8 @@ def test_config4_twelve_layers_back_to_back(amd):
         torch.cuda.synchronize()
         for got, ref in zip(together[l], alone):
             assert torch.isfinite(got.float()).all()
-            assert _rel(got, ref) <= 1e-5, f"layer {l}"
+            # split tiles meet in fp32 in any order: a sum next to a bf16 rounding boundary may round the other way
+            assert _rel(got, ref) <= 1e-4, f"layer {l}"
     # layers differ from each other (own weights): a result that leaked from a neighbour would not pass the check above
     assert _rel(together[0][2], together[11][2]) > 0.5
 

@@ -525,17 +525,74 @@ def test_mlp_forward_with_fp8_down_projection(amd, oracle):
     assert float(partial.max()) > 0
 
 
-@pytest.mark.parametrize("M", [1000, 4096, 32768, 49152])
-def test_tokens_contraction_slices(amd, M):
-    """The weight-gradient GEMMs of the MLP backward (contraction over tokens) in slices against an fp32 product."""
-    from modded_nanogpt_amd.fused import _tokens_contraction
-    g = torch.Generator().manual_seed(M)
-    a = torch.randn(M, 96, generator=g).bfloat16().cuda()
-    b = torch.randn(M, 160, generator=g).bfloat16().cuda()
-    got = _tokens_contraction(a, b)
+@pytest.mark.parametrize("a_k_rows,b_k_rows", [(False, False), (False, True), (True, True), (True, False)])
+@pytest.mark.parametrize("R,C,K", [(256, 256, 64), (264, 40, 192), (1000, 520, 768), (3072, 768, 4096), (72, 1104, 128)])
+def test_gemm_bf16_layouts_and_ragged_tiles(amd, R, C, K, a_k_rows, b_k_rows):
+    """The plain bf16 product in all four operand layouts (contraction contiguous, or the contraction as the
+    operand's rows, read through transposing LDS loads) against a double-precision product; ragged edge tiles,
+    few tiles with a long contraction (cut along it) and many tiles."""
+    g = torch.Generator().manual_seed(R + 3 * C + K)
+    a = torch.randn(R, K, generator=g).bfloat16()
+    b = torch.randn(C, K, generator=g).bfloat16()
+    ref = a.double() @ b.double().T
+    ad = dev(a.T.contiguous() if a_k_rows else a)
+    bd = dev(b.T.contiguous() if b_k_rows else b)
+    got = torch.ops.nanogpt.gemm_bf16(ad, bd, a_k_rows, b_k_rows)
+    assert got.shape == (R, C) and got.dtype == torch.bfloat16
+    assert_close_gemm(got, ref, 5e-3)
+    # fp32 accumulation, one rounding: nearly every element is the correctly rounded bf16 of the exact product
+    assert (got.cpu() == ref.float().bfloat16()).float().mean() > 0.97
+
+
+def test_gemm_bf16_operand_orientation(amd):
+    """One-hot probe through the transposing reads: element (r, c) pairs row r of A with row c of B at the same
+    contraction position; a swapped half, a wrong swizzle or a permuted contraction fails exactly."""
+    K = 192
+    a = torch.zeros(304, K)
+    b = torch.zeros(264, K)
+    for r in range(304):
+        a[r, (r * 37) % K] = 1 + (r % 5)
+    for c in range(264):
+        b[c, (c * 11) % K] = 2 + (c % 3)
+    ref = a @ b.T
+    for a_k_rows in (False, True):
+        for b_k_rows in (False, True):
+            ad = dev((a.T.contiguous() if a_k_rows else a).bfloat16())
+            bd = dev((b.T.contiguous() if b_k_rows else b).bfloat16())
+            got = torch.ops.nanogpt.gemm_bf16(ad, bd, a_k_rows, b_k_rows).float().cpu()
+            assert torch.equal(got, ref), (a_k_rows, b_k_rows)
+
+
+@pytest.mark.parametrize("M", [4096, 49152])
+def test_gemm_bf16_token_contraction(amd, M):
+    """The weight-gradient shape of the MLP backward: [3072, 768] = a^T b over M tokens, 36 output tiles cut 7 ways
+    along the contraction with the partial sums meeting in fp32 (one rounding to bf16)."""
+    g = torch.Generator(device="cuda").manual_seed(M)
+    a = torch.randn(M, 3072, device="cuda", generator=g).bfloat16()
+    b = torch.randn(M, 768, device="cuda", generator=g).bfloat16()
+    got = torch.ops.nanogpt.gemm_bf16(a, b, True, True)
     ref = a.float().T @ b.float()
-    assert got.shape == (96, 160) and got.dtype == torch.bfloat16
-    assert_close_gemm(got, ref.cpu())
+    assert got.shape == (3072, 768)
+    assert rel_err(got.float().cpu(), ref.cpu()) <= 4e-3          # the bf16 rounding of the output alone is 2^-9 / sqrt(3)
+
+
+def test_linear_relu_square_without_fp8_copies(amd, oracle):
+    """linear_relu_square(a, b) with no fp8 arguments (the reference's DISABLE_FP8 path) and the MLP function on it."""
+    M, D, H = 512, 256, 768
+    x, w_fc, w_proj_t = oracle.make_cfg2(seed=12, M=M, D=D, H=H)
+    out_ref, post_ref = oracle.mlp_fwd(x[None], w_fc, w_proj_t)
+    post = amd.linear_relu_square(dev(x), dev(w_fc))
+    assert_close_gemm(post, post_ref)
+    assert (post.cpu() == post_ref).float().mean() > 0.97
+    dy = (torch.randn(1, M, D, generator=torch.Generator().manual_seed(13)) * 1e-3).bfloat16()
+    dx_ref, dw1_ref, dw2_ref = oracle.mlp_bwd(dy, x[None], w_fc, w_proj_t, post_ref)
+    xg, w1g, w2g = dev(x[None]).requires_grad_(), dev(w_fc).requires_grad_(), dev(w_proj_t).requires_grad_()
+    out = amd.ReLUSqrdMLP(xg, w1g, w2g)
+    assert_close_gemm(out, out_ref)
+    out.backward(dev(dy))
+    assert_close_gemm(xg.grad, dx_ref)
+    assert_close_gemm(w1g.grad, dw1_ref)
+    assert_close_gemm(w2g.grad, dw2_ref)
 
 
 @pytest.mark.parametrize("M,D,H", [(256, 64, 256), (1000, 768, 3072), (2048, 1024, 4096)])
