@@ -16,6 +16,7 @@
 #include "host_util.h"
 #include "launch.h"
 #include "panel.h"
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstring>
@@ -392,6 +393,7 @@ struct CEJobIter {
     __device__ int kt_begin(int) const { return 0; }
     __device__ int kt_end(int nk) const { return nk; }
     __device__ bool partial() const { return false; }
+    __device__ int part_slot() const { return 0; }
     __device__ bool job_begin() const { return tr_ == tr_begin; }
     __device__ bool job_end() const { return tr_ + 1 == tr_end; }
     __device__ int job_id() const { return split; }
@@ -421,7 +423,7 @@ struct EpiCEFwd {
     int* cand;            // LDS: [MAX_CAND][CE_MAX_BN] valid target column of the job's tokens, else -1
     float sum[8];
 
-    __device__ void partial(bool) {}
+    __device__ void partial(bool, int) {}
     __device__ void begin(int, int, uint8_t* extra) {
         cand = (int*)extra;
         load_table(lds_table(), gtabE);
@@ -612,7 +614,7 @@ struct EpiDlStore {
     int rslot;
     int tile_big;
 
-    __device__ void partial(bool) {}
+    __device__ void partial(bool, int) {}
     __device__ void begin(int, int, uint8_t* extra) {
         rowf_lds = (float*)extra;
         rslot = 0;
@@ -727,7 +729,8 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
 int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
                        float scale, void* out_bf16, int64_t ldc, float* part32, int a_rows_pad, hipStream_t st);
 int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
-                      float scale, float* out, int64_t ldc, bool accumulate, hipStream_t st);
+                      float scale, float* out, int64_t ldc, bool accumulate, float* part32, hipStream_t st);
+int64_t balanced_part_bytes(int R, int C, int K);
 
 extern thread_local int g_gemm_slot;
 struct GemmSlot {   // books the plain GEMM launches inside a scope under a CE profile slot
@@ -1008,12 +1011,14 @@ extern "C" int ngpt_lmhead_ce_fwd_static(const void* x_bf16, const void* w_bf16,
 
 // ------------------------------------------------------------------------------------------------
 // backward workspace: tabE | tabD | rowf [M rounded up to 256] | big [same, one int per 256 rows used] | x^T panel [Kp, Mt] | W^T panel [Kp, V] | dlogits panel [Vp, Mt] |
-// dx fp32 [Mc, K]   (Mc = tokens per pass, Mt / Kp / Vp = Mc / K / V rounded up to 256)
+// fp32 parts of the split tiles of dx, then of dW   (Mc = tokens per pass, Mt / Kp / Vp = Mc / K / V rounded up to 256)
+static int64_t bwd_part_bytes(int64_t Mc, int64_t Mt, int K, int V) {
+    return std::max(balanced_part_bytes((int)Mc, K, V), std::max(balanced_part_bytes(V, K, (int)Mt), balanced_part_bytes(K, V, (int)Mt)));
+}
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
     int64_t Mc = bwd_chunk_rows(M), Mt = round256(Mc), Kp = round256(K), Vp = round256(V);
-    return align_up(2 * TAB_BYTES, 256) + 2 * round256(M) * 4 + Kp * Mt + Kp * (int64_t)V + Vp * Mt +
-           align_up(Mc * K * 4, 256);
+    return align_up(2 * TAB_BYTES, 256) + 2 * round256(M) * 4 + Kp * Mt + Kp * (int64_t)V + Vp * Mt + bwd_part_bytes(Mc, Mt, K, V);
 }
 
 extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const int64_t* targets,
@@ -1051,7 +1056,7 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     ws += Kp * (int64_t)V;
     uint8_t* dw_panel = ws;
     ws += Vp * Mt_max;
-    float* dx32 = (float*)ws;
+    float* parts = (float*)ws;
 
     Softcap sc = make_softcap(A, B, C);
     const float coef = make_coef(A, C, grad_s, grad_scale);
@@ -1087,16 +1092,16 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         {
             GemmSlot slot(PROF_CE_DX);
             if (int e = gemm_balanced_bf16(dw_panel, FMT_E5M2 | FMT_TRANSPOSED, 0, w_t, FMT_E4M3, 0, kBlockedB | kRowsPermuted, Mc, K, V, grad_s * w_s,
-                                           (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, dx32, Mt, st)) return e;
+                                           (uint16_t*)dx_bf16 + (int64_t)m0 * K, K, parts, Mt, st)) return e;
         }
         // 4. dw (+)= dl^T . x over the tokens of the pass (zero padded to Mt)
         GemmSlot slot(PROF_CE_DW);
         if (w_layout == NGPT_W_OUT_IN) {   // dw [V, K] = dl^T [V, Mt] . (x^T [K, Mt])^T
             if (int e = gemm_balanced_f32(dw_panel, FMT_E5M2, 0, x_t, FMT_E4M3, 0, kBlockedA | kBlockedB, V, K, Mt, x_s * grad_s,
-                                          (float*)dw_f32, K, several, st)) return e;
+                                          (float*)dw_f32, K, several, parts, st)) return e;
         } else {                           // dw [K, V] = x^T [K, Mt] . (dl^T [V, Mt])^T
             if (int e = gemm_balanced_f32(x_t, FMT_E4M3, 0, dw_panel, FMT_E5M2, 0, kBlockedA | kBlockedB, K, V, Mt, x_s * grad_s,
-                                          (float*)dw_f32, V, several, st)) return e;
+                                          (float*)dw_f32, V, several, parts, st)) return e;
         }
     }
     return NGPT_OK;

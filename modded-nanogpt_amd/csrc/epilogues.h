@@ -71,21 +71,30 @@ __device__ __forceinline__ void store_tile_f32(v16f (&acc)[Cfg::TM][Cfg::TN], fl
 }
 
 // ---------------------------------------------------------------------------------------------
+// Partial results of split tiles.  A job that holds only part of its tile's contraction stores acc * scale as a whole
+// BM x BN fp32 tile at part32 + slot * BM * BN (plain stores; rows / columns past the matrix edge hold whatever the
+// clamped operands gave); a later pass adds a tile's parts up and writes the result (rem_tiles_kernel).  Adding
+// them with device-scope atomics instead costs more than the contraction of a short split: the XCDs' L2 caches are
+// not coherent with each other, so such atomics execute at the memory side.
+template <class Cfg>
+__device__ __forceinline__ void store_part_tile(v16f (&acc)[Cfg::TM][Cfg::TN], float* part32, int slot, float scale,
+                                                const AccCoords<Cfg>& co) {
+    store_tile_f32<Cfg>(acc, part32 + (int64_t)slot * (Cfg::BM * Cfg::BN), Cfg::BN, scale, Cfg::BM, Cfg::BN, 0, 0, co, false);
+}
+
 // out[r, c] = bf16(acc * scale)
-// A job that holds only part of its tile's contraction adds acc * scale into the fp32 matrix `part32`
-// (same shape, zeroed by the caller, converted to bf16 by a later pass) instead.
 struct EpiStoreBf16 {
     uint16_t* out;
     int64_t ld;
     float scale;
     int R, C;
-    float* part32;       // required when the walk splits tiles
-    int64_t ld32;
+    float* part32;       // required when the walk splits tiles: one BM x BN fp32 tile per partial job
     bool is_partial;
+    int part_slot;
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
-    __device__ void partial(bool p) { is_partial = p; }
+    __device__ void partial(bool p, int slot) { is_partial = p; part_slot = slot; }
     __device__ void begin(int, int, uint8_t*) {}
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
@@ -96,7 +105,7 @@ struct EpiStoreBf16 {
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t*, int) {
         if (is_partial) {
-            store_tile_f32<Cfg>(acc, part32, ld32, scale, R, C, r0, c0, co, true);
+            store_part_tile<Cfg>(acc, part32, part_slot, scale, co);
             return;
         }
         // address = wave-uniform pointer (tile origin + the element's fixed position inside the wave
@@ -138,10 +147,11 @@ struct EpiDpre {
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     static constexpr int TILE_STORES = 16;
+    static constexpr bool DROPS_FRAGMENTS = true;   // 16 lines of post in flight next to the accumulators
     uint8_t* stage;
     bool stored_all;
     __device__ bool all_stores_issued() const { return stored_all; }
-    __device__ void partial(bool) {}
+    __device__ void partial(bool, int) {}
     __device__ void begin(int, int, uint8_t* extra) {
         stage = extra + (threadIdx.x >> 6) * 4096;
         stored_all = false;
@@ -224,7 +234,7 @@ struct EpiDiscardT {
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     long long t_clk, t_wall;
-    __device__ void partial(bool) {}
+    __device__ void partial(bool, int) {}
     __device__ void begin(int, int, uint8_t*) {
         t_clk = clock64();
         t_wall = wall_clock64();
@@ -256,19 +266,22 @@ using EpiDiscard = EpiDiscardT<false>;
 using EpiDiscardAblate = EpiDiscardT<true>;    // honours GemmOperands::ablate, at the price of its branches
 #endif  // NGPT_BENCH_BUILD
 
-// out[r, c] (+)= acc * scale in fp32.  The += form (ACCUMULATE, or a job that holds only part of its
-// tile's contraction) uses floating-point atomics on an output the caller has initialised.
+// out[r, c] (+)= acc * scale in fp32.  The += form (ACCUMULATE) uses floating-point atomics on an output the caller
+// has initialised; so does a job that holds only part of its tile's contraction unless `part32` is given, in
+// which case its tile goes there (store_part_tile) for a later pass to add up.
 template <bool ACCUMULATE>
 struct EpiStoreF32 {
     float* out;
     int64_t ld;
     float scale;
     int R, C;
+    float* part32;       // nullable
     bool is_partial;
+    int part_slot;
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
-    __device__ void partial(bool p) { is_partial = p; }
+    __device__ void partial(bool p, int slot) { is_partial = p; part_slot = slot; }
     __device__ void begin(int, int, uint8_t*) {}
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
@@ -278,7 +291,8 @@ struct EpiStoreF32 {
     template <class Cfg>
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
                          uint8_t*, int) {
-        if (ACCUMULATE || is_partial) store_tile_f32<Cfg>(acc, out, ld, scale, R, C, r0, c0, co, true);
+        if (is_partial && part32) store_part_tile<Cfg>(acc, part32, part_slot, scale, co);
+        else if (ACCUMULATE || is_partial) store_tile_f32<Cfg>(acc, out, ld, scale, R, C, r0, c0, co, true);
         else store_tile_f32<Cfg>(acc, out, ld, scale, R, C, r0, c0, co, false);
     }
 };
@@ -300,7 +314,7 @@ struct EpiRelu2Lines {
     uint8_t* stage;
     bool stored_all;
     __device__ bool all_stores_issued() const { return stored_all; }
-    __device__ void partial(bool) {}
+    __device__ void partial(bool, int) {}
     __device__ void begin(int, int, uint8_t* extra) {
         scale = dequant ? *dequant : 1.0f;
         stage = extra + (threadIdx.x >> 6) * 4096;
@@ -371,7 +385,7 @@ struct EpiRelu2T {
     __device__ void job_begin(int) {}
     template <class Cfg>
     __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
-    __device__ void partial(bool) {}
+    __device__ void partial(bool, int) {}
     __device__ void begin(int, int, uint8_t*) {
         scale = *dequant;
         inv_act = EMIT ? 1.0f / *act_scale : 0.0f;

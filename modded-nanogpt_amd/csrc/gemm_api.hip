@@ -5,6 +5,7 @@
 #include "launch.h"
 #include "panel.h"
 #include <atomic>
+#include <algorithm>
 #include <mutex>
 #include <vector>
 
@@ -123,67 +124,80 @@ static BalancePlan plan_balance(int R, int C, int K) {
     return p;
 }
 
-// Zero (MODE 0) or convert to bf16 (MODE 1) the 256 x 256 tiles number [first, first + gridDim.x) of the
-// walk order, i.e. exactly the tiles that the balanced walk splits.
+// Adds up the parts of the split tiles and writes them out.  Tile number first + blockIdx.x of the walk order is the
+// blockIdx.x-th split tile; its `splits` parts are the fp32 tiles number s * gridDim.x + blockIdx.x of `part32`
+// (GridIter::part_slot), summed in the order of the contraction.  T = uint16_t: bf16 output, T = float: fp32.
 constexpr int kRemSlices = 8;
 static_assert(MainCfg::BM % kRemSlices == 0, "row slices of a tile");
-template <int MODE>
-__global__ void rem_tiles_kernel(float* part32, int64_t ld32, uint16_t* out, int64_t ldo, int R, int C, int first) {
+template <class T>
+__global__ __launch_bounds__(256) void rem_tiles_kernel(const float* __restrict__ part32, int splits, T* __restrict__ out, int64_t ldo,
+                                                        int R, int C, int first) {
     TileOrder order(R, C, MainCfg::BM, MainCfg::BN);
     int tr, tc;
     order.coords(first + blockIdx.x, tr, tc);
     // blockIdx.y: which slice of the tile's rows (a few dozen tiles alone would leave most of the chip idle)
-    const int rows = MainCfg::BM / gridDim.y;
-    const int r0 = tr * MainCfg::BM + blockIdx.y * rows, c0 = tc * MainCfg::BN;
-    const int cols4 = MainCfg::BN / 4;
+    constexpr int rows = MainCfg::BM / kRemSlices, cols4 = MainCfg::BN / 4, tile_elems = MainCfg::BM * MainCfg::BN;
+    const int rl0 = blockIdx.y * rows;
+    const int64_t part_stride = (int64_t)gridDim.x * tile_elems;
     for (int i = threadIdx.x; i < rows * cols4; i += blockDim.x) {
-        int r = r0 + i / cols4, c = c0 + (i % cols4) * 4;
+        const int rl = rl0 + i / cols4, cl = (i % cols4) * 4;
+        const int r = tr * MainCfg::BM + rl, c = tc * MainCfg::BN + cl;
         if (r >= R || c >= C) continue;          // C % 4 == 0 is checked by the caller
-        float* p = part32 + (int64_t)r * ld32 + c;
-        if (MODE == 0) {
-            *(v4f*)p = (v4f){0.f, 0.f, 0.f, 0.f};
-        } else {
-            v4f v = *(const v4f*)p;
-            v2i o = {(int)cvt_pk_bf16(v[0], v[1]), (int)cvt_pk_bf16(v[2], v[3])};
-            *(v2i*)(out + (int64_t)r * ldo + c) = o;
-        }
+        const float* p = part32 + (int64_t)blockIdx.x * tile_elems + rl * MainCfg::BN + cl;
+        v4f v = *(const v4f*)p;
+        for (int s_ = 1; s_ < splits; ++s_) v += *(const v4f*)(p + s_ * part_stride);
+        if constexpr (sizeof(T) == 2) *(v2i*)(out + (int64_t)r * ldo + c) = (v2i){(int)cvt_pk_bf16(v[0], v[1]), (int)cvt_pk_bf16(v[2], v[3])};
+        else *(v4f*)(out + (int64_t)r * ldo + c) = v;
     }
 }
 
+// Bytes of fp32 scratch a balanced GEMM may need for the parts of its split tiles, whatever the device: at most one
+// part per workgroup of the last round (kMaxGrid bounds the grid) and never more than tiles x splits.
+constexpr int kMaxGrid = 512;
+int64_t balanced_part_bytes(int R, int C, int K) {
+    const int64_t tiles = (int64_t)((R + MainCfg::BM - 1) / MainCfg::BM) * ((C + MainCfg::BN - 1) / MainCfg::BN);
+    int64_t max_s = K / MainCfg::BK / 8;
+    if (max_s < 1) max_s = 1;
+    int64_t parts = tiles * max_s;
+    if (parts > kMaxGrid) parts = kMaxGrid;
+    return parts * MainCfg::BM * MainCfg::BN * 4;
+}
+
 // C[R, C] = scale * A . B^T with the balanced walk.  `layout`: kBlockedA | kBlockedB.
-// bf16 output: part32 is an fp32 [R, C] scratch matrix (row stride C) that only the split tiles touch.
+// part32: balanced_part_bytes(R, C, K) bytes of scratch for the split tiles.
 // fa may carry FMT_TRANSPOSED (A = panel of the transpose, a_rows_pad = R rounded up to 256).
 int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
                        float scale, void* out_bf16, int64_t ldc, float* part32, int a_rows_pad, hipStream_t st) {
     if (R <= 0 || C <= 0 || K <= 0 || K % 128 || C % 4 || ldc % 4)
         return fail(NGPT_EALIGN, "gemm_balanced_bf16: R=%d C=%d K=%d ldc=%lld", R, C, K, (long long)ldc);
     BalancePlan p = plan_balance(R, C, K);
-    if (p.splits > 1 && !part32) return fail(NGPT_EINVAL, "gemm_balanced_bf16: split tiles need the fp32 scratch matrix");
+    if (p.splits > 1 && (!part32 || p.rem * p.splits > kMaxGrid)) return fail(NGPT_EINVAL, "gemm_balanced_bf16: split tiles need the fp32 scratch tiles");
     ProfileScope prof(g_gemm_slot, st);
-    if (p.splits > 1) rem_tiles_kernel<0><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(part32, C, nullptr, 0, R, C, p.full);
     GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full, a_rows_pad};
-    EpiStoreBf16 epi{(uint16_t*)out_bf16, ldc, scale, R, C, part32, C, false};
+    EpiStoreBf16 epi{(uint16_t*)out_bf16, ldc, scale, R, C, part32, false, 0};
     if (int e = launch_gemm<MainCfg>(g, fa, fb, epi, st)) return e;
-    if (p.splits > 1) rem_tiles_kernel<1><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(part32, C, (uint16_t*)out_bf16, ldc, R, C, p.full);
+    if (p.splits > 1) rem_tiles_kernel<uint16_t><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(part32, p.splits, (uint16_t*)out_bf16, ldc, R, C, p.full);
     return check_launch("gemm_balanced_bf16");
 }
 
-// fp32 output.  accumulate: every tile adds into `out` (which the caller initialised); otherwise whole
-// tiles are stored and the split tiles are zeroed here and then added to.
+// fp32 output.  accumulate: every tile adds into `out` (which the caller initialised) with atomics; otherwise whole
+// tiles are stored and the split tiles are added up from their parts in part32.
 int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
-                      float scale, float* out, int64_t ldc, bool accumulate, hipStream_t st) {
+                      float scale, float* out, int64_t ldc, bool accumulate, float* part32, hipStream_t st) {
     if (R <= 0 || C <= 0 || K <= 0 || K % 128 || C % 4 || ldc % 4)
         return fail(NGPT_EALIGN, "gemm_balanced_f32: R=%d C=%d K=%d ldc=%lld", R, C, K, (long long)ldc);
     BalancePlan p = plan_balance(R, C, K);
     ProfileScope prof(g_gemm_slot, st);
     GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full};
     if (accumulate) {
-        EpiStoreF32<true> epi{out, ldc, scale, R, C, false};
+        EpiStoreF32<true> epi{out, ldc, scale, R, C, nullptr, false, 0};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
-    if (p.splits > 1) rem_tiles_kernel<0><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(out, ldc, nullptr, 0, R, C, p.full);
-    EpiStoreF32<false> epi{out, ldc, scale, R, C, false};
-    return launch_gemm<MainCfg>(g, fa, fb, epi, st);
+    if (p.splits > 1 && (!part32 || p.rem * p.splits > kMaxGrid)) return fail(NGPT_EINVAL, "gemm_balanced_f32: split tiles need the fp32 scratch tiles");
+    EpiStoreF32<false> epi{out, ldc, scale, R, C, part32, false, 0};
+    if (int e = launch_gemm<MainCfg>(g, fa, fb, epi, st)) return e;
+    if (p.splits > 1) rem_tiles_kernel<float><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(part32, p.splits, out, ldc, R, C, p.full);
+    return check_launch("gemm_balanced_f32");
 }
 
 // out_kind: 0 bf16, 1 fp32, 2 fp32 accumulate (atomic), 3 discard.  splits > 1 cuts each tile's
@@ -202,7 +216,7 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
     GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, splits, ablate};
     ProfileScope prof(g_gemm_slot, st);
     if (out_kind == 0) {
-        EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C, nullptr, 0, false};
+        EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C, nullptr, false, 0};
         const int tiles = ((R + MainCfg::BM - 1) / MainCfg::BM) * ((C + MainCfg::BN - 1) / MainCfg::BN);
         if (fa == FMT_E4M3 && fb == FMT_E4M3 && splits == 1 && 2 * tiles <= num_cus())
             return launch_gemm_fmt<SmallCfg, FMT_E4M3, FMT_E4M3>(g, epi, st, 0);
@@ -221,10 +235,10 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
 #endif
     }
     if (out_kind == 2) {
-        EpiStoreF32<true> epi{(float*)out, ldc, scale, R, C, false};
+        EpiStoreF32<true> epi{(float*)out, ldc, scale, R, C, nullptr, false, 0};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
     }
-    EpiStoreF32<false> epi{(float*)out, ldc, scale, R, C, false};
+    EpiStoreF32<false> epi{(float*)out, ldc, scale, R, C, nullptr, false, 0};
     return launch_gemm<MainCfg>(g, fa, fb, epi, st);
 }
 
@@ -323,12 +337,13 @@ extern "C" int ngpt_mm_fwd(const void* x_bf16, const void* w_bf16, int M, int N,
 // rows = 128 consecutive rows of g (tokens): dW = x^T . g consumes it directly as its B operand, dx = g . w
 // reads it as the transpose of its A operand (transposed on the way from LDS to the MFMA registers).
 // Both GEMMs use the balanced walk.
-// workspace: g^T panel [Np, Mt] | x_f8^T panel [Kp, Mt] | w^T panel [Kp, N] | dx fp32 [M, K]   (p / t = rounded up to 256)
+// workspace: g^T panel [Np, Mt] | x_f8^T panel [Kp, Mt] | w^T panel [Kp, N] | fp32 parts of the split tiles of dx, then of dW   (p / t = rounded up to 256)
 static int64_t round256(int64_t n) { return (n + 255) / 256 * 256; }
 extern "C" int64_t ngpt_mm_bwd_workspace_bytes(int M, int N, int K, int w_layout) {
     (void)w_layout;
     const int64_t Mt = round256(M), Np = round256(N), Kp = round256(K);
-    return Np * Mt + Kp * Mt + Kp * (int64_t)N + align_up((int64_t)M * K * 4, 256);
+    const int64_t parts = std::max(balanced_part_bytes(M, K, N), balanced_part_bytes(K, N, (int)Mt));
+    return Np * Mt + Kp * Mt + Kp * (int64_t)N + parts;
 }
 
 extern "C" int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f8, int M, int N, int K,
@@ -349,7 +364,7 @@ extern "C" int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f
     uint8_t* g_panel = ws;
     uint8_t* x_t = g_panel + Np * Mt;
     uint8_t* w_t = x_t + Kp * Mt;
-    float* dx32 = (float*)(w_t + Kp * (int64_t)N);
+    float* parts = (float*)(w_t + Kp * (int64_t)N);
     if (int e = (panel_transpose<0, FMT_E5M2>(g_bf16, N, 0, M, N, nkt, g_panel, st, grad_s))) return e;
     if (int e = panel_transpose<0>(x_f8, K, 0, M, K, nkt, x_t, st)) return e;
     if (w_layout == NGPT_W_OUT_IN) {   // w [N, K]  ->  rows = K, contraction = N
@@ -359,10 +374,10 @@ extern "C" int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f
     }
     // dx [M,K] = g [M,N] . (w^T [K,N])^T, contraction over N, g read transposed from the panel
     if (int e = gemm_balanced_bf16(g_panel, FMT_E5M2 | FMT_TRANSPOSED, 0, w_t, FMT_E4M3, 0, kBlockedB, M, K, N, grad_s * w_s,
-                                   dx_bf16, K, dx32, (int)Mt, st)) return e;
+                                   dx_bf16, K, parts, (int)Mt, st)) return e;
     // dw [K,N] = x_f8^T [K,Mt] . (g^T [N,Mt])^T, contraction over the (zero padded) rows of g
     return gemm_balanced_f32(x_t, FMT_E4M3, 0, g_panel, FMT_E5M2, 0, kBlockedA | kBlockedB, K, N, (int)Mt, x_s * grad_s,
-                             (float*)dw_kn_f32, N, false, st);
+                             (float*)dw_kn_f32, N, false, parts, st);
 }
 
 // ------------------------------------------------------------------------------------------ dpre (bf16)
@@ -380,10 +395,7 @@ extern "C" int ngpt_fc_relu2_bwd_dpre(const void* dy_bf16, const void* w2_bf16, 
 
 // ------------------------------------------------------------------------------------------ plain bf16 GEMM
 // The four bf16 products of FusedLinearReLUSquareFunction besides dpre (triton_kernels.py:715, 723, 727, 728).
-extern "C" int64_t ngpt_gemm_bf16_workspace_bytes(int R, int C, int K) {
-    (void)K;
-    return align_up((int64_t)R * C * 4, 256);
-}
+extern "C" int64_t ngpt_gemm_bf16_workspace_bytes(int R, int C, int K) { return balanced_part_bytes(R, C, 2 * K); }
 
 extern "C" int ngpt_gemm_bf16(const void* A, int a_layout, int64_t lda, const void* B, int b_layout, int64_t ldb,
                               int R, int C, int K, void* out_bf16, int64_t ldc, void* workspace, int64_t workspace_bytes,
@@ -402,6 +414,13 @@ extern "C" int ngpt_gemm_bf16(const void* A, int a_layout, int64_t lda, const vo
     // the loader works in bytes: contraction length and row strides are 2 x the element counts
     const int fa = a_layout == NGPT_K_CONTIGUOUS ? FMT_BF16 : (FMT_BF16 | FMT_TRANSPOSED);
     const int fb = b_layout == NGPT_K_CONTIGUOUS ? FMT_BF16 : (FMT_BF16 | FMT_TRANSPOSED);
+#ifdef NGPT_BENCH_BUILD
+    if (g_tuning[3]) {   // timing aid: the contraction loop alone (whole tiles, result discarded), honouring the ablation bits
+        GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, 2 * lda, 2 * ldb, R, C, 2 * K, 1, g_tuning[2]};
+        EpiDiscardAblate epi{(float*)workspace, 0, 0};
+        return launch_gemm<MainCfg>(g, fa, fb, epi, (hipStream_t)stream);
+    }
+#endif
     return gemm_balanced_bf16(A, fa, 2 * lda, B, fb, 2 * ldb, 0, R, C, 2 * K, 1.0f, out_bf16, ldc, (float*)workspace, 0,
                               (hipStream_t)stream);
 }

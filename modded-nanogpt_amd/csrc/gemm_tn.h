@@ -192,6 +192,9 @@ struct TileMainloop {
     static constexpr bool ATR16 = (AFMT & FMT_TRANSPOSED) != 0 && BF16;     // bf16 operands with the contraction as rows
     static constexpr bool BTR16 = (BFMT & FMT_TRANSPOSED) != 0 && BF16;
     static_assert(!(BFMT & FMT_TRANSPOSED) || BF16, "a transposed B operand exists for bf16 only");
+    // bf16 fragments are read by hand-placed assembly and handed over between k-steps (the 256 x 256 configuration)
+    static constexpr bool kAsmFrags16 = BF16 && Cfg::TM == 2 && Cfg::TN == 4 && Cfg::BK == 128;
+    v4i h16a[2][Cfg::TM], h16b[2][Cfg::TN];   // kAsmFrags16: two alternating fragment sets
     static_assert(!(ATR16 || BTR16) || (Cfg::BM == 256 && Cfg::BN == 256 && Cfg::BK == 128), "transposed bf16 slabs are 64 x 256");
 
     __device__ void init() {
@@ -394,7 +397,8 @@ struct TileMainloop {
     //    They are handed to the next call in a / b0 (`have` = they are valid on entry).
     //    `refill` (issue of the operand loads two k-steps ahead into the slot just freed) runs behind the
     //    last group's MFMAs, so that its address arithmetic is hidden too.
-    template <bool FIRST, class Sync, class Refill>
+    //    FRESH: the caller knows at compile time that nothing was handed over (`have` is false).
+    template <bool FIRST, bool FRESH, class Sync, class Refill>
     __device__ __forceinline__ void compute(uint8_t* smem, int stage, int next_stage, bool have, bool want_next,
                                             v16f (&acc)[Cfg::TM][Cfg::TN], v8i (&a)[Cfg::TM], v8i& b0, Sync&& sync,
                                             Refill&& refill) {
@@ -405,35 +409,41 @@ struct TileMainloop {
             // no fragment hand-over between k-steps
             constexpr int KS = Cfg::BK / 32;
             issue_loads_b(smem);
-            if constexpr (ATR16 || BTR16) {
-                // At least one operand is read through the transposing load.  All fragment reads of this path are
-                // inline assembly (see read_tr8 for why), so the compiler does not count them: frag16_fence() stands
-                // between a sub-step's reads and its MFMAs.  The reads of sub-step ks + 1 are issued behind that
-                // fence and ahead of the MFMAs of ks, which cover their latency.
+            if constexpr (kAsmFrags16) {
+                // All fragment reads of this path are inline assembly (see read_tr8 for why), so the compiler does
+                // not count them: frag16_fence() stands between a sub-step's reads and its MFMAs.  The reads of
+                // sub-step ks + 1 are issued behind that fence and ahead of the MFMAs of ks, which cover their
+                // latency; behind the barrier of the last sub-step the first fragments of the NEXT k-step (slot
+                // `next_stage`) are read and handed to the next call in h16a / h16b[0] (`have`).
                 const uint32_t sbase = (uint32_t)(size_t)((const __attribute__((address_space(3))) uint8_t*)s);
-                v4i fa[2][Cfg::TM], fb[2][Cfg::TN];
-                read_frags16<0>(sbase, fa[0], fb[0]);
+                const uint32_t nbase = (uint32_t)(size_t)((const __attribute__((address_space(3))) uint8_t*)sn);
+                static_assert(KS == 4, "four sub-steps: the hand-over lands in fragment set 0 again");
+                if (FRESH || !have) read_frags16<0>(sbase, h16a[0], h16b[0]);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    frag16_fence(fa[ks & 1], fb[ks & 1]);
-                    if (ks == 0) read_frags16<1>(sbase, fa[1], fb[1]);
-                    if (ks == 1) read_frags16<2>(sbase, fa[0], fb[0]);
-                    if (ks == 2) read_frags16<3>(sbase, fa[1], fb[1]);
-                    if (ks == KS - 1) sync();
+                    frag16_fence(h16a[ks & 1], h16b[ks & 1]);
+                    if (ks == 0) read_frags16<1>(sbase, h16a[1], h16b[1]);
+                    if (ks == 1) read_frags16<2>(sbase, h16a[0], h16b[0]);
+                    if (ks == 2) read_frags16<3>(sbase, h16a[1], h16b[1]);
+                    if (ks == KS - 1) {
+                        sync();
+                        if (want_next) read_frags16<0>(nbase, h16a[0], h16b[0]);
+                    }
                     __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-                    for (int tm = 0; tm < Cfg::TM; ++tm)
+                    for (int tn = 0; tn < Cfg::TN; ++tn)
 #pragma unroll
-                        for (int tn = 0; tn < Cfg::TN; ++tn) {
+                        for (int tm = 0; tm < Cfg::TM; ++tm) {
                             const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                             acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                                __builtin_bit_cast(v8bf, fa[ks & 1][tm]), __builtin_bit_cast(v8bf, fb[ks & 1][tn]),
+                                __builtin_bit_cast(v8bf, h16a[ks & 1][tm]), __builtin_bit_cast(v8bf, h16b[ks & 1][tn]),
                                 (FIRST && ks == 0) ? zero : acc[tm][tn], 0, 0, 0);
                         }
                     __builtin_amdgcn_s_setprio(0);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 refill();
+                __builtin_amdgcn_sched_barrier(0);
                 return;
             }
 #pragma unroll
@@ -456,7 +466,7 @@ struct TileMainloop {
             refill();
         } else {
             v8i bcur = b0;
-            if (!have) {
+            if (FRESH || !have) {
 #pragma unroll
                 for (int t = 0; t < Cfg::TM; ++t) a[t] = frag_a_at(s, t, 0);
                 bcur = frag(s, frag_b[0], 0);
@@ -585,6 +595,8 @@ struct GridIter {
     __device__ int kt_begin(int nk) const { return nk == nk_ ? kt_lo_ : 2 * kt_lo_; }
     __device__ int kt_end(int nk) const { return nk == nk_ ? kt_hi_ : 2 * kt_hi_; }
     __device__ bool partial() const { return seq >= full; }     // the job holds part of its tile's contraction
+    // number of a partial job: split * (split tiles) + (index of its tile among the split tiles)
+    __device__ int part_slot() const { return seq - full; }
     __device__ bool job_begin() const { return false; }
     __device__ bool job_end() const { return false; }
     __device__ int job_id() const { return 0; }
@@ -597,7 +609,7 @@ struct GridIter {
 
 // The generic persistent kernel.  `Iter` walks the tiles of this workgroup (see GridIter).  `Epi` supplies
 //   void begin(int bid, int nblocks)
-//   void partial(bool)   -- before each tile(): the job holds only part of the tile's contraction
+//   void partial(bool, int slot)   -- before each tile(): the job holds only part of the tile's contraction; slot numbers such jobs
 //   void tile(acc, r0, c0, coords, scratch /* wave-private LDS */, lane)
 //   void job_begin(c0) / job_end(c0, job_id, coords, stage_scratch /* whole free LDS stage */)
 //                                                              -- only if Iter reports job boundaries
@@ -659,6 +671,14 @@ template <class E, class = void>
 struct EpiHasTileBegin : std::false_type {};
 template <class E>
 struct EpiHasTileBegin<E, std::void_t<decltype(E::HAS_TILE_BEGIN)>> : std::bool_constant<E::HAS_TILE_BEGIN> {};
+
+// Epilogues with `static constexpr bool DROPS_FRAGMENTS = true` need the registers that would carry the next
+// k-step's first operand fragments across tile(): the last k-step of a job then reads nothing ahead and the next
+// job's first k-step fetches its own fragments (one LDS round trip per tile instead of spills in the epilogue).
+template <class E, class = void>
+struct EpiDropsFragments : std::false_type {};
+template <class E>
+struct EpiDropsFragments<E, std::void_t<decltype(E::DROPS_FRAGMENTS)>> : std::bool_constant<E::DROPS_FRAGMENTS> {};
 
 template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(GemmOperands g, Epi epi) {
@@ -729,7 +749,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         auto kstep = [&](auto first, auto relaxed, bool last_kt) {
             constexpr int PENDING_OK = decltype(relaxed)::value ? EpiTileStores<Epi>::value : 0;
             // a k-step follows this one (and its first fragments may be read ahead)
-            const bool more = ahead >= 2;
+            const bool more = ahead >= 2 && !(EpiDropsFragments<Epi>::value && last_kt);
             auto sync = [&]() {
                 wait_vmem_le<PENDING_OK>();
                 if (!(ablate & 4)) wg_barrier();
@@ -741,13 +761,14 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
                 if (last_kt) ml.issue_loads_b(smem);
             };
             if (!(ablate & 2)) {
-                ml.template compute<decltype(first)::value>(smem, slot, slot ^ 1, have, more, acc, fa, fb, sync, refill_here);
+                ml.template compute<decltype(first)::value, decltype(first)::value && EpiDropsFragments<Epi>::value>(
+                    smem, slot, slot ^ 1, have, more, acc, fa, fb, sync, refill_here);
             } else {
                 ml.issue_loads_b(smem);
                 sync();
                 refill_here();
             }
-            have = more && (AFMT & 3) != FMT_BF16 && !(ablate & 2);
+            have = more && (TileMainloop<Cfg, AFMT, BFMT>::kAsmFrags16 || (AFMT & 3) != FMT_BF16) && !(ablate & 2);
             --ahead;
             slot ^= 1;
         };
@@ -762,7 +783,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{}, std::false_type{}, kt + 1 == kt1);
         // every wave passed the last k-step's barrier after its final read of slot ^ 1
         uint8_t* free_stage = smem + (slot ^ 1) * Cfg::STAGE_BYTES;
-        epi.partial(cur.partial());
+        epi.partial(cur.partial(), cur.part_slot());
         epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
         if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
         if (keep_slot) {

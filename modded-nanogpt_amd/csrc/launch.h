@@ -54,11 +54,17 @@ int launch_gemm_fmt(const GemmOperands& g, const Epi& epi, hipStream_t st, int m
 }
 
 struct EpiStoreBf16;
+#ifdef NGPT_BENCH_BUILD
+template <bool ABLATE> struct EpiDiscardT;
+template <class Epi> constexpr bool kBf16Epi = std::is_same<Epi, EpiStoreBf16>::value || std::is_same<Epi, EpiDiscardT<true>>::value;
+#else
+template <class Epi> constexpr bool kBf16Epi = std::is_same<Epi, EpiStoreBf16>::value;
+#endif
 
 template <class Cfg, class Epi>
 int launch_gemm_cfg(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {
     if ((fa & 3) == FMT_BF16 || (fb & 3) == FMT_BF16) {   // bf16 x bf16 -> bf16: row-major or contraction-major operands
-        if constexpr (std::is_same<Epi, EpiStoreBf16>::value && std::is_same<Cfg, TileCfg<256, 256, 4, 2, 128, 2>>::value) {
+        if constexpr (kBf16Epi<Epi> && std::is_same<Cfg, MainCfg>::value) {
             constexpr int N = FMT_BF16, T = FMT_BF16 | FMT_TRANSPOSED;
             if (fa == N && fb == N) return launch_gemm_fmt<Cfg, N, N>(g, epi, st, max_grid);
             if (fa == N && fb == T) return launch_gemm_fmt<Cfg, N, T>(g, epi, st, max_grid);
