@@ -50,7 +50,8 @@ int ngpt_num_cus(void);
 /* ---- optional per-kernel timing ------------------------------------------------------------
  * No counterpart in the reference (contributors patch torch.profiler in by hand).  When enabled,
  * the heavy launches of the fused lm_head + CE path are bracketed by HIP events on their own
- * stream.  Slots: 0 forward kernel, 1 dlogits recompute, 2 dx GEMM, 3 dW GEMM, 4 other GEMMs.
+ * stream.  Slots: 0 fused CE forward kernel, 1 dlogits recompute, 2 dx GEMM, 3 dW GEMM (of the fused CE backward),
+ * 4 other fp8 GEMMs, 5 up projection + ReLU^2, 6 dpre, 7 plain bf16 GEMMs of the MLP, 8 MLP input producers.
  * ngpt_profile_read waits for the recorded launches of a slot, returns the sum of their
  * durations and their count, and clears the slot. */
 int ngpt_profile_enable(int on);
@@ -64,6 +65,14 @@ int ngpt_profile_read(int slot, double* total_ms, int* launches);
  * key 7: 1 = accept operand row strides below K (overlapping rows keep the operands cache resident in
  * timing runs).  Process-global and not synchronised: one thread, set before the timed calls. */
 int ngpt_tuning_set(int key, int value);
+
+/* Microbenchmark of the fp8 GEMM's k-step skeleton (same tile shape and instructions as the shipped kernel, no
+ * epilogue): one launch of `grid` workgroups x `iters` k-steps of 256 x 256 x 128.  mode bits: 1 = operand fragments
+ * re-read from LDS every sub-step, 2 = a workgroup barrier per k-step, 4 = 64 KiB of operands per k-step through
+ * direct-to-LDS loads; 0 = the matrix pipe alone.  src: fp8 bytes, 64 KiB + 8 x 64 KiB per workgroup, src_stride
+ * bytes apart; sink: 512 floats; ticks [grid][2] int64 = shader-clock cycles and 100 MHz wall ticks per workgroup. */
+int ngpt_bench_kstep_rate(const void* src, int64_t src_stride, int mode, int iters, int grid, float* sink,
+                          long long* ticks, void* stream);
 #endif
 
 /* ---- quantisers ---------------------------------------------------------------------------

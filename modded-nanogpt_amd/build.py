@@ -18,7 +18,7 @@ CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libngpt_fp8.so"
 BENCH_LIB_PATH = LIB_DIR / "libngpt_fp8_bench.so"     # + the timing aids behind NGPT_BENCH_BUILD, for measurements only
-SOURCES = ["gemm_api.hip", "quant.hip", "ce.hip", "mlp_aux.hip"]
+SOURCES = ["gemm_api.hip", "quant.hip", "ce.hip", "mlp_aux.hip", "bench_kernels.hip"]   # the last one is empty without NGPT_BENCH_BUILD
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

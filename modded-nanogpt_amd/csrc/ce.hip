@@ -732,12 +732,6 @@ int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb,
                       float scale, float* out, int64_t ldc, bool accumulate, float* part32, hipStream_t st);
 int64_t balanced_part_bytes(int R, int C, int K);
 
-extern thread_local int g_gemm_slot;
-struct GemmSlot {   // books the plain GEMM launches inside a scope under a CE profile slot
-    int saved;
-    explicit GemmSlot(int s) : saved(g_gemm_slot) { g_gemm_slot = s; }
-    ~GemmSlot() { g_gemm_slot = saved; }
-};
 
 static Softcap make_softcap(float A, float B, float C) {
     Softcap sc;

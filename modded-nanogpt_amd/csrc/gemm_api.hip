@@ -94,8 +94,7 @@ static int check_gemm_dims(const char* who, int R, int C, int K, int64_t lda, in
     return NGPT_OK;
 }
 
-// Which profile slot the next gemm_store launches are booked under (set by the fused CE backward).
-thread_local int g_gemm_slot = PROF_GEMM;   // per host thread: entry points may be called concurrently
+thread_local int g_gemm_slot = PROF_GEMM;
 
 // ---------------------------------------------------------------------------------------------
 // Balanced walk.  A persistent grid of G workgroups finishes `tiles` tiles in ceil(tiles / G) rounds,
@@ -390,6 +389,7 @@ extern "C" int ngpt_fc_relu2_bwd_dpre(const void* dy_bf16, const void* w2_bf16, 
     // Transposed product (tile rows = hidden units, tile columns = tokens), see EpiDpre.
     GemmOperands g{(const uint8_t*)w2_bf16, (const uint8_t*)dy_bf16, 2 * (int64_t)D, 2 * (int64_t)D, H, M, 2 * D, 1, 0};
     EpiDpre epi{(uint16_t*)dpre_bf16, (const uint16_t*)post_bf16, H, H, M};
+    ProfileScope prof(PROF_DPRE, (hipStream_t)stream);
     return launch_gemm_fmt<MainCfg, FMT_BF16, FMT_BF16>(g, epi, (hipStream_t)stream, 0);
 }
 
@@ -421,6 +421,7 @@ extern "C" int ngpt_gemm_bf16(const void* A, int a_layout, int64_t lda, const vo
         return launch_gemm<MainCfg>(g, fa, fb, epi, (hipStream_t)stream);
     }
 #endif
+    GemmSlot slot(PROF_GEMM_BF16);
     return gemm_balanced_bf16(A, fa, 2 * lda, B, fb, 2 * ldb, 0, R, C, 2 * K, 1.0f, out_bf16, ldc, (float*)workspace, 0,
                               (hipStream_t)stream);
 }
@@ -434,6 +435,7 @@ extern "C" int ngpt_linear_relu2_bf16(const void* x_bf16, const void* w_bf16, in
     if (K % 64 || N % 8) return fail(NGPT_EALIGN, "ngpt_linear_relu2_bf16: need K %% 64 == 0 and N %% 8 == 0 (N=%d K=%d)", N, K);
     GemmOperands gt{(const uint8_t*)w_bf16, (const uint8_t*)x_bf16, 2 * (int64_t)K, 2 * (int64_t)K, N, M, 2 * K, 1, 0};
     EpiRelu2Lines epi{(uint16_t*)post_bf16, N, nullptr, N, M};
+    ProfileScope prof(PROF_FC_RELU2, (hipStream_t)stream);
     return launch_gemm_fmt<MainCfg, FMT_BF16, FMT_BF16>(gt, epi, (hipStream_t)stream, 0);
 }
 
@@ -447,6 +449,7 @@ extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float
     if (int e = check_gemm_dims("ngpt_fc_relu2_fwd", M, N, K, K, K)) return e;
     if (N % 16) return fail(NGPT_EALIGN, "ngpt_fc_relu2_fwd: N=%d must be a multiple of 16", N);
     GemmOperands g{(const uint8_t*)x_f8, (const uint8_t*)w_f8, K, K, M, N, K, 1, 0};
+    ProfileScope prof(PROF_FC_RELU2, (hipStream_t)stream);
     auto fill = [&](auto& epi) {
         epi.post = (uint16_t*)post_bf16;
         epi.ld = N;

@@ -48,8 +48,12 @@ enum ProfileSlot : int {
     PROF_CE_DLOGITS = 1,  // logits recompute + e5m2 dlogits
     PROF_CE_DX = 2,       // dx GEMM
     PROF_CE_DW = 3,       // dW GEMM
-    PROF_GEMM = 4,        // any other plain GEMM launch
-    PROF_SLOTS = 5
+    PROF_GEMM = 4,        // any other fp8 GEMM launch (nanogpt::mm forward / backward, the FP8 down projection)
+    PROF_FC_RELU2 = 5,    // up projection with the ReLU^2 epilogue (fp8 or bf16 operands)
+    PROF_DPRE = 6,        // dpre GEMM of the MLP backward
+    PROF_GEMM_BF16 = 7,   // plain bf16 GEMMs of the MLP (c_proj, dx, dW1, dW2), their summing pass included
+    PROF_PRODUCERS = 8,   // rms-norm + amax + quantise of the MLP input, the norm's backward
+    PROF_SLOTS = 9
 };
 bool profiling_on();
 void profile_begin(int slot, hipStream_t st);
@@ -65,6 +69,15 @@ struct ProfileScope {
     ~ProfileScope() {
         if (on) profile_end(slot, st);
     }
+};
+
+// Which profile slot the balanced GEMM launches inside a scope are booked under (per host thread: entry points may
+// be called concurrently).
+extern thread_local int g_gemm_slot;
+struct GemmSlot {
+    int saved;
+    explicit GemmSlot(int s) : saved(g_gemm_slot) { g_gemm_slot = s; }
+    ~GemmSlot() { g_gemm_slot = saved; }
 };
 
 inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }

@@ -311,6 +311,7 @@ extern "C" int ngpt_mlp_input_quant(const void* x_bf16, int rows, int dim, const
         return fail(NGPT_EWORKSPACE, "ngpt_mlp_input_quant: workspace %lld < %lld bytes", (long long)workspace_bytes,
                     (long long)ngpt_mlp_input_quant_workspace_bytes());
     hipStream_t st = (hipStream_t)stream;
+    ProfileScope prof(PROF_PRODUCERS, st);
     float* partial = (float*)workspace;
     int blocks = (rows + 3) / 4;
     if (blocks > kNormPartials) blocks = kNormPartials;
@@ -380,6 +381,7 @@ extern "C" int ngpt_rmsnorm_bwd(const void* x_bf16, const void* g_bf16, int rows
     int blocks = (rows + 3) / 4;
     const int cap = num_cus() * 16;
     if (blocks > cap) blocks = cap;
+    ProfileScope prof(PROF_PRODUCERS, (hipStream_t)stream);
     rmsnorm_bwd_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x_bf16, (const uint16_t*)g_bf16, rows, dim, (uint16_t*)dx_bf16);
     return check_launch("rmsnorm_bwd_kernel");
 }

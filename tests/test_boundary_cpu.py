@@ -164,7 +164,7 @@ def test_package_never_imports_the_oracle():
 
 
 def test_bench_uses_the_oracle_only_as_the_cpu_baseline():
-    """In bench.py the oracle may be imported by the cpu_baseline function and nowhere else."""
+    """In bench.py the oracle may be imported by the cpu_baseline* functions (the timed CPU leg) and nowhere else."""
     import ast
     tree = ast.parse((ROOT / "bench.py").read_text())
     def imports_oracle(node):
@@ -175,7 +175,7 @@ def test_bench_uses_the_oracle_only_as_the_cpu_baseline():
                 return True
         return False
     for node in tree.body:
-        if isinstance(node, ast.FunctionDef) and node.name == "cpu_baseline":
+        if isinstance(node, ast.FunctionDef) and node.name.startswith("cpu_baseline"):
             assert imports_oracle(node)
         else:
             assert not imports_oracle(node), getattr(node, "name", node)
