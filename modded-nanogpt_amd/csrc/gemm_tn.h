@@ -142,8 +142,10 @@ struct LaneOffsets {
         chunk = min(chunk, lim / 8 - 1);
         return (uint32_t)((int64_t)m * ld + chunk * 16);
     }
-    __device__ void init(const GemmOperands& g, int wave, int lane, int r0, int c0, bool a_transposed, bool a_tr16 = false,
-                         bool b_tr16 = false) {
+    // A tile's offsets depend on its position only where rows (or, for a transposed bf16 slab, columns) past the end of
+    // the operand are clamped, i.e. in the last tile row / column of a matrix that is not a multiple of the tile:
+    // init_a / init_b are called again only when the new or the previous tile is such an edge tile.
+    __device__ void init_a(const GemmOperands& g, int wave, int lane, int r0, bool a_transposed, bool a_tr16) {
         int lrow = lane / Cfg::CPR, lchunk = lane % Cfg::CPR;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i) {
@@ -162,6 +164,9 @@ struct LaneOffsets {
             int rr = min(R, g.R - 1 - r0);                       // clamp rows past the end
             a_off[i] = (uint32_t)((int64_t)rr * g.lda + q * 16);
         }
+    }
+    __device__ void init_b(const GemmOperands& g, int wave, int lane, int c0, bool b_tr16) {
+        int lrow = lane / Cfg::CPR, lchunk = lane % Cfg::CPR;
 #pragma unroll
         for (int i = 0; i < Cfg::B_LOADS; ++i) {
             if (b_tr16) { b_off[i] = tr16_off(i, wave, lane, g.ldb, g.C - c0); continue; }
@@ -184,6 +189,7 @@ struct TileMainloop {
     int a_step, b_step;      // bytes from one k-step's slab to the next
     const uint8_t* b_pending;   // B slab whose loads issue_loads_b() still has to issue, or null
     int pending_stage;
+    int lo_state;            // bit 0 / 1: a_off / b_off hold the offsets of a tile that needs no clamping (they fit every such tile)
     int a_kt;                // transposed A: index of the next k-step to load; a_next then is the tile's base
     int64_t a_pair_stride;   // transposed A: bytes between the panel rows of two consecutive 256-blocks of the contraction
     int wave, lane, wr, wc;
@@ -202,6 +208,7 @@ struct TileMainloop {
         lane = tid & 63;
         b_pending = nullptr;
         pending_stage = 0;
+        lo_state = 0;
         wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         wr = wave / Cfg::WAVES_N;
         wc = wave % Cfg::WAVES_N;
@@ -271,7 +278,10 @@ struct TileMainloop {
             b_step = (int)(64 * g.ldb);
             b_next = g.B + 2 * (int64_t)c0 + (int64_t)kt * b_step;
         }
-        lo.init(g, wave, lane, r0, c0, ATR, ATR16, BTR16);
+        const bool a_inner = g.R - r0 >= Cfg::BM, b_inner = g.C - c0 >= Cfg::BN;
+        if (!(a_inner && (lo_state & 1))) lo.init_a(g, wave, lane, r0, ATR, ATR16);
+        if (!(b_inner && (lo_state & 2))) lo.init_b(g, wave, lane, c0, BTR16);
+        lo_state = (a_inner ? 1 : 0) | (b_inner ? 2 : 0);
     }
 
     // Loads the next k-step of the current tile into LDS slot `stage` and moves on to the one after: the A
