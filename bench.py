@@ -273,23 +273,41 @@ def workload_lmhead_ce(args, amd, lib, dev):
     pt = torch.full((M,), -1, dtype=torch.int64, device=dev)
     pw = torch.zeros(1, device=dev)
 
-    def step():
-        losses, lse, sig, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(
-            xd, wd, td, mtp, pt, pw, sc["x_s"], sc["w_s"], sc["A"], sc["B"], sc["C"], False)
-        dx, dw = torch.ops.nanogpt.lmhead_ce_bwd(
-            x_f8, w_f8, td, mtp, pt, pw, lse, sig, sc["x_s"], sc["w_s"], sc["grad_s"], sc["grad_scale"],
-            sc["A"], sc["B"], sc["C"], False)
+    fwd_args = (xd, wd, td, mtp, pt, pw, sc["x_s"], sc["w_s"], sc["A"], sc["B"], sc["C"], False)
+    bwd_tail = (sc["x_s"], sc["w_s"], sc["grad_s"], sc["grad_scale"], sc["A"], sc["B"], sc["C"], False)
+
+    def step_recompute():      # nothing of size [tokens, vocabulary] kept: the backward runs the logits GEMM again
+        losses, lse, sig, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(*fwd_args)
+        dx, dw = torch.ops.nanogpt.lmhead_ce_bwd(x_f8, w_f8, td, mtp, pt, pw, lse, sig, *bwd_tail)
         return losses, dx, dw
 
+    def step_codes():          # the forward keeps one code byte of bf16(sigma) per logit, the backward rebuilds dl from it
+        losses, lse, sig, x_f8, w_f8, codes = torch.ops.nanogpt.lmhead_ce_fwd_codes(*fwd_args)
+        dx, dw = torch.ops.nanogpt.lmhead_ce_bwd_codes(x_f8, w_f8, td, mtp, pt, pw, lse, sig, codes, *bwd_tail)
+        return losses, dx, dw
+
+    codes_mode = args.ce_backward == "codes"
+    step, other = (step_codes, step_recompute) if codes_mode else (step_recompute, step_codes)
     if args.calibrate_copy:
         calibrate_copy(dev)
     out, ms, median_ms, kernels = run_timed(lib, step, args.steps, args.warmup)
-    gemm = 2.0 * M * K * V      # executed FLOP of each of the four GEMM-shaped kernels per step
+    gemm = 2.0 * M * K * V      # executed FLOP of each GEMM-shaped kernel per step
     work = {n: (gemm, "mfma-fp8") for n in ("lm_head_ce_fwd", "dlogits_recompute", "dx_gemm", "dw_gemm")}
+    mode_desc = "the backward recomputes the logits (four GEMM passes)"
+    if codes_mode:              # the second slot then is the code -> e5m2 conversion, a memory-bound pass over 2 x M x V bytes
+        kernels["dlogits_from_codes"] = kernels.pop("dlogits_recompute")
+        del work["dlogits_recompute"]
+        work["dlogits_from_codes"] = (2.0 * M * V, "hbm")
+        mode_desc = "the forward keeps one sigma code byte per logit for the backward (three GEMM passes)"
+    extra = {"mean_loss": float(out[0].mean()), "ce_backward": args.ce_backward}
+    if not args.no_other_mode:  # the other mode of the backward, timed the same way on a few steps, for the record
+        _, o_ms, o_med, _ = run_timed(lib, other, max(5, args.steps // 5), 3)
+        extra["other_mode"] = {"ce_backward": "recompute" if codes_mode else "codes", "ms_per_step": o_ms,
+                               "median_ms_per_step": o_med, "tokens_per_s": M / (o_ms * 1e-3)}
     cpu = None if args.no_cpu_baseline else cpu_baseline(x, w, t, sc)
     emit(args, lib, "config 3: FP8 lm_head + fused softcapped cross-entropy, forward+backward, M=49152 K=768 V=50304, "
-                    "(out,in) weight, n_predict=1", M, 6.0 * M * K * V, ms, median_ms, kernels, work, "lmhead_ce",
-         extra={"mean_loss": float(out[0].mean())}, cpu=cpu,
+                    "(out,in) weight, n_predict=1; " + mode_desc, M, 6.0 * M * K * V, ms, median_ms, kernels, work,
+         "lmhead_ce" if codes_mode else "lmhead_ce_recompute", extra=extra, cpu=cpu,
          metric="lm_head+CE fwd+bwd tokens/s at M=49152 (FP8 TFLOP/s and fraction of dense FP8 peak alongside)")
     return 0
 
@@ -381,7 +399,9 @@ def secondary(args, amd, lib, dev) -> int:
         flops = 6.0 * Mm * D * Vv + 12.0 * Mm * D * H
         desc, tokens = "config 5: lm_head + softcapped CE forward+backward and one FP8 MLP layer forward+backward, M=65536 D=1024 H=4096 V=50304", Mm
         work = mlp_work(Mm, D, H, True)
-        work.update({n: (2.0 * Mm * D * Vv, "mfma-fp8") for n in ("lm_head_ce_fwd", "dlogits_recompute", "dx_gemm", "dw_gemm")})
+        work.update({n: (2.0 * Mm * D * Vv, "mfma-fp8") for n in ("lm_head_ce_fwd", "dx_gemm", "dw_gemm")})
+        # the slot named dlogits_recompute holds the code -> e5m2 pass (2 x M x V bytes) unless the backward recomputes the logits
+        work["dlogits_recompute"] = (2.0 * Mm * Vv, "hbm") if amd.fused.CE_BACKWARD == "codes" else (2.0 * Mm * D * Vv, "mfma-fp8")
         if not args.no_cpu_baseline:
             a = cpu_baseline(xh_c, wh_c, tg_c, sc, budget_s=10.0)
             b = cpu_baseline_mlp(x, w_fc_c[0], w_pt_c[0], dy_c, True, budget_s=8.0)
@@ -510,6 +530,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ce-backward", choices=("codes", "recompute"), default="codes",
+                    help="headline workload: where the backward takes the e5m2 gradient of the logits from")
+    ap.add_argument("--no-other-mode", action="store_true", help="headline workload: do not also time the other --ce-backward mode")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy, the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")

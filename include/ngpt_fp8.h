@@ -276,6 +276,29 @@ int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const int64_t* tar
                        float A, float B, float C, void* dx_bf16, void* dw_f32, int w_layout,
                        void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same pair with the softcap's output kept between them instead of recomputed (what FusedSoftcappedCrossEntropy
+ * saves between forward and backward is one byte per logit either way: the reference keeps the e5m2 gradient,
+ * triton_kernels.py:1231-1253, this pair keeps an 8-bit code of bf16(sigmoid(..)), never the logits).  The forward
+ * also writes sigma_codes, ngpt_lmhead_ce_codes_bytes(M, V) bytes; the backward turns them into the e5m2 gradient
+ * (bit-identical to what ngpt_lmhead_ce_bwd recomputes) without running the logits GEMM a second time.  Token tiles in
+ * which some sigma lies below the 255 codes' range (logits under about -13 with A, B, C = 23, 5, 7.5) are detected on
+ * the device and recomputed from the logits as ngpt_lmhead_ce_bwd does, so results never depend on the range.
+ * Everything else (arguments, alignment, workspaces) is as in ngpt_lmhead_ce_fwd / ngpt_lmhead_ce_bwd. */
+int64_t ngpt_lmhead_ce_codes_bytes(int M, int V);
+int ngpt_lmhead_ce_fwd_codes(const void* x_bf16, const void* w_bf16, const int64_t* targets,
+                             const float* mtp_weights, int n_predict,
+                             const int64_t* prefix_targets, const float* prefix_weight,
+                             int M, int K, int V, float x_s, float w_s, float A, float B, float C,
+                             float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
+                             void* sigma_codes, int w_layout, void* workspace, int64_t workspace_bytes, void* stream);
+int ngpt_lmhead_ce_bwd_codes(const void* x_f8, const void* w_f8_vk, const int64_t* targets,
+                             const float* mtp_weights, int n_predict,
+                             const int64_t* prefix_targets, const float* prefix_weight,
+                             const float* lse, const float* saved_sigma, const void* sigma_codes, int M, int K, int V,
+                             float x_s, float w_s, float grad_s, float grad_scale,
+                             float A, float B, float C, void* dx_bf16, void* dw_f32, int w_layout,
+                             void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

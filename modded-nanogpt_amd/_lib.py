@@ -62,6 +62,11 @@ SIGNATURES = {
     "ngpt_lmhead_ce_bwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
     "ngpt_lmhead_ce_bwd": (_I, [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _F, _F, _F, _F,
                                 _F, _F, _F, _P, _P, _I, _P, _L, _P]),
+    "ngpt_lmhead_ce_codes_bytes": (_L, [_I, _I]),
+    "ngpt_lmhead_ce_fwd_codes": (_I, [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _F, _F, _F, _F, _F,
+                                      _P, _P, _P, _P, _P, _P, _I, _P, _L, _P]),
+    "ngpt_lmhead_ce_bwd_codes": (_I, [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _F, _F, _F,
+                                      _F, _F, _F, _P, _P, _I, _P, _L, _P]),
 }
 
 _lib = None

@@ -30,6 +30,17 @@ constexpr int TAB_ENTRIES = TAB_NEG + TAB_N;
 constexpr int TAB_BYTES = TAB_ENTRIES * 4;
 constexpr int MAX_CAND = NGPT_MAX_PREDICT + 1;   // shifted targets + the prefix target
 
+// Sigma codes.  The gradient factor D(l) depends on the logit only through sigma = bf16(sigmoid(..)), and the bf16
+// values in [SIGC_LOW, 1.0] are 255 consecutive bit patterns: code = bits - SIGC_LOW + 1 in 1..255 names one of them
+// exactly, code 0 says "sigma below the window" (logits under about -13 with the reference's constants).  A forward
+// that stores one code byte per logit (1 byte, like the reference's saved e5m2 gradient, instead of the 2-byte logit)
+// lets the backward rebuild dl = e5m2(rowf * D) bit for bit without running the logits GEMM again.
+constexpr int SIGC_LOW = 0x3f80 - 254;           // bf16 bits of 0.25390625
+__device__ __forceinline__ uint32_t sigma_code(float sigma_bf16) {
+    const int c = (int)(__float_as_uint(sigma_bf16) >> 16) - SIGC_LOW + 1;
+    return (c >= 1 && c <= 255) ? (uint32_t)c : 0u;
+}
+
 struct Softcap {
     float A, inv_C, B_div_C;
 };
@@ -76,7 +87,10 @@ __device__ __forceinline__ float softcap_sigma(float l, const Softcap& sc) {
 }
 __device__ __forceinline__ float softcap_E(float sigma, const Softcap& sc) { return expf(sc.A * sigma - sc.A); }
 
-__global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc) {
+// embed_codes: every tabE entry carries the sigma code of its logit in the low 8 bits of its fp32 pattern, and the
+// upper 24 bits are chosen so that the pattern read as a float is as close to exp(z - A) as those 8 bits allow
+// (relative error at most 2^-16, either sign): one table read then serves the sum of exponentials and the code.
+__global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc, bool embed_codes) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= TAB_ENTRIES) return;
     int t = i % TAB_NEG, neg = i / TAB_NEG;
@@ -85,8 +99,29 @@ __global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc) {
     float l = bf16_bits_to_f32(bits | (neg ? 0x8000u : 0u));
     float s = softcap_sigma(l, sc);
     float e = softcap_E(s, sc);
-    tabE[i] = e;
     tabD[i] = e * s * (1.0f - s);
+    if (embed_codes) {
+        const uint32_t code = sigma_code(s), hi = __float_as_uint(e) & ~0xffu;
+        float best = __uint_as_float(hi | code);
+#pragma unroll
+        for (int d = -1; d <= 1; d += 2) {
+            const float cand = __uint_as_float((hi + (uint32_t)(d * 0x100)) | code);
+            if (fabsf(cand - e) < fabsf(best - e)) best = cand;
+        }
+        e = best;
+    }
+    tabE[i] = e;
+}
+
+// dcode[c] = D of the sigma with code c (the expression of ce_table_kernel's tabD), dcode[0] = 0.
+__global__ void ce_dcode_kernel(float* dcode, Softcap sc) {
+    const int c = threadIdx.x;
+    float d = 0.0f;
+    if (c >= 1) {
+        const float s = bf16_bits_to_f32((uint32_t)(SIGC_LOW + c - 1));
+        d = softcap_E(s, sc) * s * (1.0f - s);
+    }
+    dcode[c] = d;
 }
 
 __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
@@ -409,10 +444,25 @@ constexpr int CE_MAX_BN = 256;                                  // widest token 
 constexpr int CAND_LDS_BYTES = MAX_CAND * CE_MAX_BN * 4;
 constexpr int CE_FWD_EXTRA_LDS = (CAND_LDS_BYTES + 1023) / 1024 * 1024;
 
-struct EpiCEFwd {
+// Four code bytes (the low bytes of four table words) as one word, lowest register first.
+__device__ __forceinline__ uint32_t pack_codes4(float w0, float w1, float w2, float w3) {
+    const uint32_t t01 = __builtin_amdgcn_perm(__float_as_uint(w1), __float_as_uint(w0), 0x0c0c0400);
+    const uint32_t t23 = __builtin_amdgcn_perm(__float_as_uint(w3), __float_as_uint(w2), 0x0c0c0400);
+    return __builtin_amdgcn_perm(t23, t01, 0x05040100);
+}
+
+// CODES: the table entries carry sigma codes (ce_table_kernel with embed_codes) and every tile also writes its
+// 256 x 256 codes into the token-major code panel: blocks [token tile][vocabulary / 128] of 256 rows (tokens) x 128
+// bytes, a lane's 16 accumulator registers (16 vocabulary rows of one token, in register order, i.e. dw_pos order
+// inside every 32-group) as one 16-byte store.
+template <bool CODES>
+struct EpiCEFwdT {
     static constexpr int EXTRA_LDS = CE_FWD_EXTRA_LDS;
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = true;    // job_end reduces through the stage
+    static constexpr int TILE_STORES = CODES ? 8 : 0;      // 16-byte panel stores per wave and tile (the rare sigma stores come on top)
+    uint8_t* codes;       // CODES: the code panel
+    int nkp;              // CODES: 128-byte k-steps per token tile of the panel = vocabulary rounded up to 256, / 128
     const float* gtabE;
     float* part;          // [CE_SPLITS][M] partial sums of exp(z - A)
     float* saved_sigma;   // [MAX_CAND][M] bf16-rounded sigma at each candidate target column
@@ -448,14 +498,29 @@ struct EpiCEFwd {
     __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0 /* vocab */, int c0 /* token */,
                          const AccCoords<Cfg>& co, uint8_t*, int lane) {
         static_assert(Cfg::TN <= 8, "per-lane token columns");
+        static_assert(!CODES || (Cfg::BM == kPanelRows && Cfg::BN == kPanelRows && Cfg::WTM == 64 && Cfg::WTN == 128),
+                      "the code stores assume a 256 x 256 tile of 64 x 128 wave tiles");
         const int V = ca.V, M = ca.M;
         const float* tab = lds_table();
+        // code panel: row = this lane's token, 16 bytes = the 16 vocabulary rows of one (tm, lane half) group;
+        // address = wave-uniform pointer + ONE 32-bit per-lane offset + a constant per store
+        uint8_t* cd_base = nullptr;
+        uint32_t cd_lane = 0;
+        if constexpr (CODES) {
+            const int wr = co.wave_row0 >> 6, wc = co.wave_col0 >> 7;
+            cd_base = codes + ((int64_t)(c0 >> 8) * nkp + (r0 >> 7) + (wr >> 1)) * kPanelBytes;
+            cd_lane = (uint32_t)((128 * wc + (lane & 31)) * 128 + 64 * (wr & 1) + 16 * (lane >> 5));
+        }
+        auto code_store = [&](int tm, int tn, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+            *(v4i*)(cd_base + (cd_lane + tn * 4096 + tm * 32)) = (v4i){(int)w0, (int)w1, (int)w2, (int)w3};
+        };
         if (r0 + Cfg::BM <= V) {
             // Batches of 8 accumulator registers, software-pipelined by hand: index arithmetic of batch b, its 8
             // table reads, then the additions of batch b - 1, whose reads have had the arithmetic of b to return.
             // (Left to itself the scheduler sometimes waits for every pair of reads right behind their issue.)
             constexpr int NB = Cfg::TN * Cfg::TM * 2;
             float pv[8];
+            uint32_t cw[4];
 #pragma unroll
             for (int b = 0; b <= NB; ++b) {
                 float nv[8];
@@ -473,7 +538,15 @@ struct EpiCEFwd {
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if (b > 0) sum[(b - 1) / (2 * Cfg::TM)] += ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
+                if (b > 0) {
+                    sum[(b - 1) / (2 * Cfg::TM)] += ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
+                    if constexpr (CODES) {
+                        const int q = b - 1;
+                        cw[2 * (q & 1)] = pack_codes4(pv[0], pv[1], pv[2], pv[3]);
+                        cw[2 * (q & 1) + 1] = pack_codes4(pv[4], pv[5], pv[6], pv[7]);
+                        if (q & 1) code_store((q >> 1) % Cfg::TM, q / (2 * Cfg::TM), cw[0], cw[1], cw[2], cw[3]);
+                    }
+                }
 #pragma unroll
                 for (int k = 0; k < 8; ++k) pv[k] = nv[k];
             }
@@ -483,14 +556,22 @@ struct EpiCEFwd {
 #pragma unroll
                 for (int tm = 0; tm < Cfg::TM; ++tm) {
                     float s0 = 0.0f;
+                    uint32_t cwe[4];
 #pragma unroll
-                    for (int v = 0; v < 16; v += 2) {
-                        uint32_t off = tab_offsets2(pack_logits(acc[tm][tn][v] * scale, acc[tm][tn][v + 1] * scale));
-                        float e0 = tab_at(tab, off & 0xffffu), e1 = tab_at(tab, off >> 16);
+                    for (int v = 0; v < 16; v += 4) {
+                        uint32_t o01 = tab_offsets2(pack_logits(acc[tm][tn][v] * scale, acc[tm][tn][v + 1] * scale));
+                        uint32_t o23 = tab_offsets2(pack_logits(acc[tm][tn][v + 2] * scale, acc[tm][tn][v + 3] * scale));
+                        const float e0 = tab_at(tab, o01 & 0xffffu), e1 = tab_at(tab, o01 >> 16);
+                        const float e2 = tab_at(tab, o23 & 0xffffu), e3 = tab_at(tab, o23 >> 16);
                         s0 += (r0 + co.row(tm, v) < V) ? e0 : 0.0f;
                         s0 += (r0 + co.row(tm, v + 1) < V) ? e1 : 0.0f;
+                        s0 += (r0 + co.row(tm, v + 2) < V) ? e2 : 0.0f;
+                        s0 += (r0 + co.row(tm, v + 3) < V) ? e3 : 0.0f;
+                        if constexpr (CODES) cwe[v >> 2] = pack_codes4(e0, e1, e2, e3);
                     }
                     sum[tn] += s0;
+                    if constexpr (CODES)   // rows past V: codes of the clamped duplicates, which no reader of the panel looks at
+                        code_store(tm, tn, cwe[0], cwe[1], cwe[2], cwe[3]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
         }
@@ -547,6 +628,7 @@ struct EpiCEFwd {
         }
     }
 };
+using EpiCEFwd = EpiCEFwdT<false>;
 
 __global__ void ce_finalize_kernel(const float* __restrict__ part, const float* __restrict__ saved_sigma,
                                    CandArgs ca, Softcap sc, float* __restrict__ losses, float* __restrict__ lse_out) {
@@ -723,6 +805,66 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
     }
 }
 
+// Backward from the forward's sigma codes: the code panel (token-major, see EpiCEFwdT) of one pass becomes that
+// pass's dlogits panel (vocabulary-major, tokens of a k-step in dw_pos order), dl = e5m2_sat(rowf[token] * dcode[code]):
+// the same product and conversion as EpiDlStore, so the two agree bit for bit.  One workgroup moves 128 tokens x 128
+// vocabulary entries: 16 KiB of one code block in, converted on the way into LDS, transposed as in
+// panel_transpose_kernel, 16 KiB of one panel block out.  A code of 0 (sigma below the window) inside the matrix sets
+// the flag of its token tile: EpiDlStore then recomputes that tile's part of the panel from the logits.
+__global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __restrict__ codes, int nkp, int m0, int M,
+                                                             const float* __restrict__ rowf, const float* __restrict__ dcode,
+                                                             int nkt, uint8_t* __restrict__ dl_panel, int* __restrict__ flags) {
+    constexpr int kStride = 33;
+    __shared__ uint32_t tile[128 * kStride];
+    __shared__ float dtab[256];
+    const int kv = blockIdx.x, a = blockIdx.y, tid = threadIdx.x;
+    dtab[tid] = dcode[tid];
+    __syncthreads();
+    auto word_at = [&](int r, int w) -> uint32_t& { return tile[r * kStride + (w ^ (((r >> 4) & 7) << 2))]; };
+    const int tok0 = m0 + a * 128;
+    const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes + ((tok0 >> 7) & 1) * (kPanelBytes / 2);
+    bool below = false;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int i = tid + 256 * j, r = i >> 3, ch = i & 7;     // 16 codes of token tok0 + r
+        const v4i c = *(const v4i*)(src + r * 128 + ch * 16);
+        const float rf = rowf[tok0 + r];                          // zero past the last token
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t w = (uint32_t)c[k];
+            below |= (tok0 + r < M) && (((w - 0x01010101u) & ~w & 0x80808080u) != 0u);
+            word_at(r, ch * 4 + k) = f32x4_to_e5m2_sat<true>(rf * dtab[w & 0xffu], rf * dtab[(w >> 8) & 0xffu],
+                                                             rf * dtab[(w >> 16) & 0xffu], rf * dtab[w >> 24]);
+        }
+    }
+    if (below) flags[(tok0 - m0) >> 8] = 1;
+    __syncthreads();
+    // as panel_transpose_kernel with PERM = 2: piece `sub` of a vocabulary entry's 128-byte row holds the tokens
+    // 32 (sub / 2) + 8 g + 4 (sub % 2) + i at byte 4 g + i; the four code columns 4 cgp ..+3 of a thread are the
+    // vocabulary entries vloc ..+3 (dw_pos order of the code panel's bytes undone)
+    const int sub = tid & 7, cgp = tid >> 3;
+    const int rbase = 32 * (sub >> 1) + 4 * (sub & 1);
+    uint32_t w[4][4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[g][i] = word_at(rbase + 8 * g + i, cgp);
+        transpose4x4_bytes(w[g]);
+    }
+    const int vloc = 32 * (cgp >> 3) + 8 * (cgp & 3) + 4 * ((cgp >> 2) & 1);
+    uint8_t* dst = dl_panel + ((int64_t)(kv >> 1) * nkt + a) * kPanelBytes + ((kv & 1) * 128 + vloc) * 128 + sub * 16;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) *(v4i*)(dst + c * 128) = (v4i){(int)w[0][c], (int)w[1][c], (int)w[2][c], (int)w[3][c]};
+}
+
+// list[0 .. *count) = the token tiles of the pass whose flag is set (n <= 256 of them; one thread, a few hundred cycles)
+__global__ void ce_flag_list_kernel(const int* __restrict__ flags, int n, int* __restrict__ list, int* __restrict__ count) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    int c = 0;
+    for (int i = 0; i < n; ++i)
+        if (flags[i]) list[c++] = i;
+    *count = c;
+}
 
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
                float scale, void* out, int64_t ldc, int out_kind, hipStream_t st, int splits);
@@ -801,10 +943,10 @@ static int check_cand(const char* who, const int64_t* targets, const float* mtp_
 }
 
 // One launch of the fused forward kernel for tile configuration Cfg.
-template <class Cfg>
-static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwd& epi, hipStream_t st) {
-    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, EpiCEFwd, CEJobIter>;
-    constexpr int LDS = Cfg::SMEM_BYTES + EpiCEFwd::EXTRA_LDS;   // dynamic part; the table is static LDS
+template <class Cfg, bool CODES>
+static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwdT<CODES>& epi, hipStream_t st) {
+    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, EpiCEFwdT<CODES>, CEJobIter>;
+    constexpr int LDS = Cfg::SMEM_BYTES + EpiCEFwdT<CODES>::EXTRA_LDS;   // dynamic part; the table is static LDS
     static PerDeviceOnce configured;
     if (int e = configured.run([&] { return allow_lds(kernel, LDS); })) return e;
     int cus = num_cus();
@@ -821,9 +963,9 @@ static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwd& epi, hipStream_t
     return check_launch("lm_head CE forward");
 }
 
-template <class Cfg, class Epi>
+template <class Cfg, class Iter, class Epi>
 static int launch_grid_kernel(const GemmOperands& g, const Epi& epi, hipStream_t st, int slot, const char* what) {
-    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, Epi, GridIter>;
+    auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, Epi, Iter>;
     constexpr int LDS = Cfg::SMEM_BYTES + Epi::EXTRA_LDS;
     static PerDeviceOnce configured;
     if (int e = configured.run([&] { return allow_lds(kernel, LDS); })) return e;
@@ -833,7 +975,7 @@ static int launch_grid_kernel(const GemmOperands& g, const Epi& epi, hipStream_t
     int per_cu = Cfg::WGS_PER_CU > 1 ? Cfg::WGS_PER_CU : 1;
     int grid = tiles < cus * per_cu ? tiles : cus * per_cu;
     {
-        ProfileScope prof(slot, st);
+        ProfileScope prof(slot >= 0 ? slot : 0, st, slot >= 0);
         kernel<<<grid, Cfg::THREADS, LDS, st>>>(g, epi);
     }
     return check_launch(what);
@@ -867,7 +1009,7 @@ extern "C" int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, 
     Softcap sc = make_softcap(A, B, C);
     float* tabE = (float*)workspace;
     float* tabD = tabE + TAB_ENTRIES;
-    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
+    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc, false);
     CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, n_rows, n_cols};
     int grid = num_cus();
     if (grid <= 0) return fail(NGPT_EINVAL, "no HIP device");
@@ -907,7 +1049,7 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
                               const float* mtp_weights, int n_predict, const int64_t* prefix_targets, const float* prefix_weight,
                               int M, int K, int V, float x_s, float w_s, float A, float B, float C,
                               float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
-                              int w_layout, void* workspace, int64_t workspace_bytes, void* stream) {
+                              int w_layout, void* workspace, int64_t workspace_bytes, void* stream, void* sigma_codes = nullptr) {
     if (!x_bf16 || !w_bf16 || !losses || !lse || !saved_sigma || !x_f8 || !w_f8_vk || !workspace)
         return fail(NGPT_EINVAL, "%s: null pointer", who);
     if (int e = check_cand(who, targets, mtp_weights, n_predict)) return e;
@@ -926,7 +1068,7 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
     float* part = (float*)(ws + align_up(2 * TAB_BYTES, 256));
 
     Softcap sc = make_softcap(A, B, C);
-    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
+    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc, sigma_codes != nullptr);
     // a vocabulary split can be empty for a tiny V; its partial sums must read as zero
     fill_f32_kernel<<<(CE_SPLITS * M + 255) / 256, 256, 0, st>>>(part, (int64_t)CE_SPLITS * M, 0.0f);
     if (w_layout == NGPT_W_OUT_IN) {
@@ -937,16 +1079,28 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
     }
 
     GemmOperands g{(const uint8_t*)w_f8_vk, (const uint8_t*)x_f8, K, K, V, M, K, 1, 0};
-    EpiCEFwd epi{};
-    epi.gtabE = tabE;
-    epi.part = part;
-    epi.saved_sigma = saved_sigma;
-    epi.ca = CandArgs{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
-    epi.sc = sc;
-    epi.scale = x_s * w_s;
-    epi.ncand = prefix_targets ? n_predict + 1 : n_predict;
-    if (int e = launch_ce_fwd<MainCfg>(g, epi, st)) return e;
-    ce_finalize_kernel<<<(M + 255) / 256, 256, 0, st>>>(part, saved_sigma, epi.ca, sc, losses, lse);
+    const CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
+    auto fill = [&](auto& epi) {
+        epi.gtabE = tabE;
+        epi.part = part;
+        epi.saved_sigma = saved_sigma;
+        epi.ca = ca;
+        epi.sc = sc;
+        epi.scale = x_s * w_s;
+        epi.ncand = prefix_targets ? n_predict + 1 : n_predict;
+    };
+    if (sigma_codes) {
+        EpiCEFwdT<true> epi{};
+        fill(epi);
+        epi.codes = (uint8_t*)sigma_codes;
+        epi.nkp = (int)(round256(V) / 128);
+        if (int e = launch_ce_fwd<MainCfg, true>(g, epi, st)) return e;
+    } else {
+        EpiCEFwd epi{};
+        fill(epi);
+        if (int e = launch_ce_fwd<MainCfg, false>(g, epi, st)) return e;
+    }
+    ce_finalize_kernel<<<(M + 255) / 256, 256, 0, st>>>(part, saved_sigma, ca, sc, losses, lse);
     return check_launch("ce_finalize_kernel");
 }
 }  // namespace ngpt
@@ -1009,30 +1163,34 @@ extern "C" int ngpt_lmhead_ce_fwd_static(const void* x_bf16, const void* w_bf16,
 static int64_t bwd_part_bytes(int64_t Mc, int64_t Mt, int K, int V) {
     return std::max(balanced_part_bytes((int)Mc, K, V), std::max(balanced_part_bytes(V, K, (int)Mt), balanced_part_bytes(K, V, (int)Mt)));
 }
+constexpr int64_t kFlagBytes = 4096;    // codes backward: flags [256] | list [256] | count of the pass's token tiles
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
     int64_t Mc = bwd_chunk_rows(M), Mt = round256(Mc), Kp = round256(K), Vp = round256(V);
-    return align_up(2 * TAB_BYTES, 256) + 2 * round256(M) * 4 + Kp * Mt + Kp * (int64_t)V + Vp * Mt + bwd_part_bytes(Mc, Mt, K, V);
+    return align_up(2 * TAB_BYTES, 256) + 2 * round256(M) * 4 + Kp * Mt + Kp * (int64_t)V + Vp * Mt + bwd_part_bytes(Mc, Mt, K, V) + kFlagBytes;
 }
 
-extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const int64_t* targets,
-                                  const float* mtp_weights, int n_predict,
-                                  const int64_t* prefix_targets, const float* prefix_weight,
-                                  const float* lse, const float* saved_sigma, int M, int K, int V,
-                                  float x_s, float w_s, float grad_s, float grad_scale,
-                                  float A, float B, float C, void* dx_bf16, void* dw_f32, int w_layout,
-                                  void* workspace, int64_t workspace_bytes, void* stream) {
+extern "C" int64_t ngpt_lmhead_ce_codes_bytes(int M, int V) { return round256(M) * round256(V); }
+
+namespace ngpt {
+static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f8_vk, const int64_t* targets,
+                              const float* mtp_weights, int n_predict,
+                              const int64_t* prefix_targets, const float* prefix_weight,
+                              const float* lse, const float* saved_sigma, const void* sigma_codes, int M, int K, int V,
+                              float x_s, float w_s, float grad_s, float grad_scale,
+                              float A, float B, float C, void* dx_bf16, void* dw_f32, int w_layout,
+                              void* workspace, int64_t workspace_bytes, void* stream) {
     if (!x_f8 || !w_f8_vk || !lse || !saved_sigma || !dx_bf16 || !dw_f32 || !workspace)
-        return fail(NGPT_EINVAL, "ngpt_lmhead_ce_bwd: null pointer");
-    if (int e = check_cand("ngpt_lmhead_ce_bwd", targets, mtp_weights, n_predict)) return e;
-    if (int e = check_softcap("ngpt_lmhead_ce_bwd", A, B, C)) return e;
-    if (M <= 0 || K <= 0 || V <= 0) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_bwd: empty problem M=%d K=%d V=%d", M, K, V);
+        return fail(NGPT_EINVAL, "%s: null pointer", who);
+    if (int e = check_cand(who, targets, mtp_weights, n_predict)) return e;
+    if (int e = check_softcap(who, A, B, C)) return e;
+    if (M <= 0 || K <= 0 || V <= 0) return fail(NGPT_EINVAL, "%s: empty problem M=%d K=%d V=%d", who, M, K, V);
     if (K % 128 || M % 128 || V % 128)
-        return fail(NGPT_EALIGN, "ngpt_lmhead_ce_bwd: need M, K, V multiples of 128 (M=%d K=%d V=%d)", M, K, V);
-    if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_bwd: w_layout=%d", w_layout);
+        return fail(NGPT_EALIGN, "%s: need M, K, V multiples of 128 (M=%d K=%d V=%d)", who, M, K, V);
+    if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "%s: w_layout=%d", who, w_layout);
     int64_t need = ngpt_lmhead_ce_bwd_workspace_bytes(M, K, V, w_layout);
     if (workspace_bytes < need)
-        return fail(NGPT_EWORKSPACE, "ngpt_lmhead_ce_bwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
+        return fail(NGPT_EWORKSPACE, "%s: workspace %lld < %lld bytes", who, (long long)workspace_bytes, (long long)need);
     hipStream_t st = (hipStream_t)stream;
     const int Mc_max = bwd_chunk_rows(M);
     const int64_t Mt_max = round256(Mc_max), Kp = round256(K), Vp = round256(V);
@@ -1051,11 +1209,18 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
     uint8_t* dw_panel = ws;
     ws += Vp * Mt_max;
     float* parts = (float*)ws;
+    ws += bwd_part_bytes(Mc_max, Mt_max, K, V);
+    int* flags = (int*)ws;                   // per token tile of the pass: some sigma of it lies below the code window
+    int* list = flags + 256;
+    int* count = list + 256;
+    static_assert(BWD_CHUNK_ROWS / 256 <= 256 && 3 * 256 * 4 <= kFlagBytes, "flag and list arrays of one pass");
 
     Softcap sc = make_softcap(A, B, C);
     const float coef = make_coef(A, C, grad_s, grad_scale);
     CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
-    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc);
+    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc, false);
+    float* dcode = tabE;                     // the backward does not read tabE: its first 256 entries serve as the code table
+    if (sigma_codes) ce_dcode_kernel<<<1, 256, 0, st>>>(dcode, sc);
     ce_rowf_kernel<<<(M + 255) / 256, 256, 0, st>>>(lse, ca, sc, coef, rowf, big);
     if (int e = check_launch("ce_rowf_kernel")) return e;
     const int nkv = V / 128;
@@ -1078,7 +1243,20 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         epi.V = V;
         epi.nkt = nkt;
         epi.scale = x_s * w_s;
-        if (int e = launch_grid_kernel<MainCfg>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
+        if (sigma_codes) {
+            // 1'. the pass's dlogits panel from the forward's sigma codes; token tiles with a sigma below the code
+            //     window (none, normally) are then redone from the logits
+            ProfileScope prof(PROF_CE_DLOGITS, st);
+            const int nt = Mt / 256;
+            fill_f32_kernel<<<1, 256, 0, st>>>((float*)flags, nt, 0.0f);
+            ce_codes_to_dl_kernel<<<dim3(V / 128, nkt), 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, rowf, dcode,
+                                                                      nkt, dw_panel, flags);
+            if (int e = check_launch("ce_codes_to_dl_kernel")) return e;
+            ce_flag_list_kernel<<<1, 64, 0, st>>>(flags, nt, list, count);
+            g.row_list = list;
+            g.row_count = count;
+            if (int e = launch_grid_kernel<MainCfg, ListGridIter>(g, epi, st, -1, "lm_head CE backward (dlogits of the flagged token tiles)")) return e;
+        } else if (int e = launch_grid_kernel<MainCfg, GridIter>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
         ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, nkt, dw_panel);
         if (int e = check_launch("ce_dl_fix_kernel")) return e;
@@ -1099,4 +1277,42 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
         }
     }
     return NGPT_OK;
+}
+}  // namespace ngpt
+
+extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const int64_t* targets,
+                                  const float* mtp_weights, int n_predict,
+                                  const int64_t* prefix_targets, const float* prefix_weight,
+                                  const float* lse, const float* saved_sigma, int M, int K, int V,
+                                  float x_s, float w_s, float grad_s, float grad_scale,
+                                  float A, float B, float C, void* dx_bf16, void* dw_f32, int w_layout,
+                                  void* workspace, int64_t workspace_bytes, void* stream) {
+    return lmhead_ce_bwd_impl("ngpt_lmhead_ce_bwd", x_f8, w_f8_vk, targets, mtp_weights, n_predict, prefix_targets, prefix_weight,
+                              lse, saved_sigma, nullptr, M, K, V, x_s, w_s, grad_s, grad_scale, A, B, C, dx_bf16, dw_f32,
+                              w_layout, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ngpt_lmhead_ce_fwd_codes(const void* x_bf16, const void* w_bf16, const int64_t* targets,
+                                        const float* mtp_weights, int n_predict,
+                                        const int64_t* prefix_targets, const float* prefix_weight,
+                                        int M, int K, int V, float x_s, float w_s, float A, float B, float C,
+                                        float* losses, float* lse, float* saved_sigma, void* x_f8, void* w_f8_vk,
+                                        void* sigma_codes, int w_layout, void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!sigma_codes) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_fwd_codes: null pointer");
+    return lmhead_ce_fwd_impl("ngpt_lmhead_ce_fwd_codes", x_bf16, w_bf16, targets, mtp_weights, n_predict, prefix_targets, prefix_weight,
+                              M, K, V, x_s, w_s, A, B, C, losses, lse, saved_sigma, x_f8, w_f8_vk, w_layout,
+                              workspace, workspace_bytes, stream, sigma_codes);
+}
+
+extern "C" int ngpt_lmhead_ce_bwd_codes(const void* x_f8, const void* w_f8_vk, const int64_t* targets,
+                                        const float* mtp_weights, int n_predict,
+                                        const int64_t* prefix_targets, const float* prefix_weight,
+                                        const float* lse, const float* saved_sigma, const void* sigma_codes, int M, int K, int V,
+                                        float x_s, float w_s, float grad_s, float grad_scale,
+                                        float A, float B, float C, void* dx_bf16, void* dw_f32, int w_layout,
+                                        void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!sigma_codes) return fail(NGPT_EINVAL, "ngpt_lmhead_ce_bwd_codes: null pointer");
+    return lmhead_ce_bwd_impl("ngpt_lmhead_ce_bwd_codes", x_f8, w_f8_vk, targets, mtp_weights, n_predict, prefix_targets, prefix_weight,
+                              lse, saved_sigma, sigma_codes, M, K, V, x_s, w_s, grad_s, grad_scale, A, B, C, dx_bf16, dw_f32,
+                              w_layout, workspace, workspace_bytes, stream);
 }

@@ -56,6 +56,9 @@ struct GemmOperands {
     int layout;         // kBlockedA | kBlockedB | kRowsPermuted
     int full_tiles;     // the first full_tiles tiles (in walk order) are never split; 0 = `splits` applies to every tile
     int a_rows_pad;     // transposed A only: R rounded up to 256
+    // ListGridIter only: the kernel works on the tile rows row_list[0 .. *row_count) instead of on all of them
+    const int* row_list;
+    const int* row_count;
 };
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1>
@@ -617,6 +620,19 @@ struct GridIter {
     }
 };
 
+// GridIter over a subset of the tile rows: row_list[i], i < *row_count (both written by an earlier kernel and
+// read through the constant address space, i.e. as scalar loads that stay out of the vector memory counter).
+struct ListGridIter : GridIter {
+    const int* list;
+    static __device__ GemmOperands listed(GemmOperands g, int BM) {
+        g.R = ((const __attribute__((address_space(4))) int*)(uintptr_t)g.row_count)[0] * BM;
+        return g;
+    }
+    __device__ ListGridIter(const GemmOperands& g, int BM, int BN, int bid_, int G_)
+        : GridIter(listed(g, BM), BM, BN, bid_, G_), list(g.row_list) {}
+    __device__ int tr() const { return ((const __attribute__((address_space(4))) int*)(uintptr_t)list)[tr_]; }
+};
+
 // The generic persistent kernel.  `Iter` walks the tiles of this workgroup (see GridIter).  `Epi` supplies
 //   void begin(int bid, int nblocks)
 //   void partial(bool, int slot)   -- before each tile(): the job holds only part of the tile's contraction; slot numbers such jobs
@@ -745,6 +761,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     bool have = false;
     int slot = 0;
     bool first_job = true;
+    bool prev_deferred = false;    // the previous job's epilogue kept its slot: the refill went out after its stores
     while (cur.valid()) {
         const int r0 = cur.tr() * Cfg::BM, c0 = cur.tc() * Cfg::BN;
         if (cur.job_begin()) epi.template job_begin<Cfg>(c0);   // made visible by the k-loop's barriers
@@ -756,12 +773,14 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         // landed (its loads are the newest load group in flight; the memory counter retires in issue
         // order, so anything issued after them -- the previous epilogue's stores -- may still be
         // pending), the workgroup meets, and the slot just read is refilled two k-steps ahead.
-        auto kstep = [&](auto first, auto relaxed, bool last_kt) {
-            constexpr int PENDING_OK = decltype(relaxed)::value ? EpiTileStores<Epi>::value : 0;
+        auto kstep = [&](auto first, bool relaxed, bool last_kt) {
             // a k-step follows this one (and its first fragments may be read ahead)
             const bool more = ahead >= 2 && !(EpiDropsFragments<Epi>::value && last_kt);
             auto sync = [&]() {
-                wait_vmem_le<PENDING_OK>();
+                // only the wait differs between the relaxed and the plain first k-step: a scalar branch around it
+                // instead of a second copy of the k-step
+                if (decltype(first)::value && EpiTileStores<Epi>::value > 0 && relaxed) wait_vmem_le<EpiTileStores<Epi>::value>();
+                else wait_vmem_le<0>();
                 if (!(ablate & 4)) wg_barrier();
             };
             auto refill_here = [&]() {
@@ -784,13 +803,12 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         };
         // relaxed wait: only behind an epilogue that stored (not the first job), with a later k-step of
         // the same job to wait for tile_begin's load, and only if that epilogue's refill was not deferred
-        constexpr bool kNeverDefers = !Epi::NEEDS_SCRATCH && !Epi::JOB_END_NEEDS_SCRATCH;
-        bool relax = kNeverDefers && EpiTileStores<Epi>::value > 0 && !first_job && kt1 - kt0 >= 2;
+        constexpr bool kMayRelax = !Epi::NEEDS_SCRATCH && EpiTileStores<Epi>::value > 0;
+        bool relax = kMayRelax && !first_job && !prev_deferred && kt1 - kt0 >= 2;
         if constexpr (EpiReportsStores<Epi>::value) relax = relax && epi.all_stores_issued();
-        if (relax) kstep(std::true_type{}, std::true_type{}, kt0 + 1 == kt1);
-        else kstep(std::true_type{}, std::false_type{}, kt0 + 1 == kt1);
+        kstep(std::true_type{}, relax, kt0 + 1 == kt1);
         first_job = false;
-        for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{}, std::false_type{}, kt + 1 == kt1);
+        for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{}, false, kt + 1 == kt1);
         // every wave passed the last k-step's barrier after its final read of slot ^ 1
         uint8_t* free_stage = smem + (slot ^ 1) * Cfg::STAGE_BYTES;
         epi.partial(cur.partial(), cur.part_slot());
@@ -801,6 +819,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
             refill(slot ^ 1);
             ml.issue_loads_b(smem);
         }
+        prev_deferred = keep_slot;
         cur.advance();
     }
     wg_barrier();

@@ -63,7 +63,7 @@ struct ProfileScope {
     int slot;
     hipStream_t st;
     bool on;
-    ProfileScope(int s, hipStream_t stream) : slot(s), st(stream), on(profiling_on()) {
+    ProfileScope(int s, hipStream_t stream, bool enable = true) : slot(s), st(stream), on(enable && profiling_on()) {
         if (on) profile_begin(slot, st);
     }
     ~ProfileScope() {

@@ -12,9 +12,20 @@ from __future__ import annotations
 import torch
 from torch import Tensor
 
+import os
+
 from . import _lib, ops
 
 E4M3 = torch.float8_e4m3fn
+
+# Where the backward of FusedSoftcappedCrossEntropy takes the e5m2 gradient of the logits from:
+#   "codes"      the forward keeps one byte per logit, the 8-bit code of bf16(sigmoid(..)) (the reference keeps one
+#                byte per logit as well, the e5m2 gradient itself; the logits are never stored), and the backward
+#                rebuilds the gradient from it: three GEMM passes per step;
+#   "recompute"  nothing of size [tokens, vocabulary] is kept and the backward runs the logits GEMM again: four passes.
+# Both give bit-identical gradients.  Set before the forward runs (module attribute or NGPT_CE_BACKWARD).
+CE_BACKWARD = os.environ.get("NGPT_CE_BACKWARD", "codes")
+assert CE_BACKWARD in ("codes", "recompute"), f"NGPT_CE_BACKWARD={CE_BACKWARD!r}: expected 'codes' or 'recompute'"
 
 
 def transpose_copy(src: Tensor, dst: Tensor) -> None:
@@ -171,10 +182,16 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
             prefix_weight = torch.zeros(1, dtype=torch.float32, device=dev)
         prefix_weight = prefix_weight.reshape(1).to(torch.float32).contiguous()
 
-        losses, lse, saved_sigma, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(
-            x.contiguous(), lm_head_weight.contiguous(), targets, mtp_weights, prefix_targets, prefix_weight,
-            x_s, w_s, A, B, C, w_in_out)
-        ctx.save_for_backward(targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma, x_f8, w_f8)
+        if CE_BACKWARD == "codes" and n_rows % 128 == 0:
+            losses, lse, saved_sigma, x_f8, w_f8, codes = torch.ops.nanogpt.lmhead_ce_fwd_codes(
+                x.contiguous(), lm_head_weight.contiguous(), targets, mtp_weights, prefix_targets, prefix_weight,
+                x_s, w_s, A, B, C, w_in_out)
+        else:
+            losses, lse, saved_sigma, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(
+                x.contiguous(), lm_head_weight.contiguous(), targets, mtp_weights, prefix_targets, prefix_weight,
+                x_s, w_s, A, B, C, w_in_out)
+            codes = None
+        ctx.save_for_backward(targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma, x_f8, w_f8, codes)
         ctx.params = (A, B, C, x_s, w_s, grad_s, grad_scale, w_in_out)
         return losses
 
@@ -182,9 +199,14 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
     def backward(ctx, grad_output):
         # grad_output is ignored: grad_scale is folded into the gradient, as in the reference
         # (triton_kernels.py:1117, 1262).
-        targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma, x_f8, w_f8 = ctx.saved_tensors
+        targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma, x_f8, w_f8, codes = ctx.saved_tensors
         A, B, C, x_s, w_s, grad_s, grad_scale, w_in_out = ctx.params
-        grad_x, grad_w = torch.ops.nanogpt.lmhead_ce_bwd(
-            x_f8, w_f8, targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma,
-            x_s, w_s, grad_s, grad_scale, A, B, C, w_in_out)
+        if codes is not None:
+            grad_x, grad_w = torch.ops.nanogpt.lmhead_ce_bwd_codes(
+                x_f8, w_f8, targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma, codes,
+                x_s, w_s, grad_s, grad_scale, A, B, C, w_in_out)
+        else:
+            grad_x, grad_w = torch.ops.nanogpt.lmhead_ce_bwd(
+                x_f8, w_f8, targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma,
+                x_s, w_s, grad_s, grad_scale, A, B, C, w_in_out)
         return grad_x, None, None, None, None, grad_w, None, None, None, None, None, None, None, None

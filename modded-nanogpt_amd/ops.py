@@ -287,6 +287,84 @@ def _(x_f8, w_f8, targets, mtp_weights, prefix_targets, prefix_weight, lse, save
             torch.empty((K, V) if w_in_out else (V, K), dtype=torch.float32, device=x_f8.device))
 
 
+# The same pair with the softcap's output kept between forward and backward instead of recomputed: one byte per
+# logit, the 8-bit code of bf16(sigmoid(..)) -- the reference keeps one byte per logit too, its e5m2 gradient
+# (triton_kernels.py:1231-1253) -- and never the logits.  The backward rebuilds the e5m2 gradient from the codes,
+# bit-identical to the recomputed one, and skips the second logits GEMM.
+
+@torch.library.custom_op("nanogpt::lmhead_ce_fwd_codes", mutates_args=())
+def lmhead_ce_fwd_codes(x: Tensor, w: Tensor, targets: Tensor, mtp_weights: Tensor, prefix_targets: Tensor,
+                        prefix_weight: Tensor, x_s: float, w_s: float, A: float, B: float, C: float,
+                        w_in_out: bool) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
+    """-> (losses, lse, saved_sigma, x_f8, w_f8 as lmhead_ce_fwd, sigma_codes uint8 [ceil256(M) * ceil256(V)])."""
+    _gpu(x, w, targets, mtp_weights, prefix_targets, prefix_weight)
+    assert x.is_contiguous() and w.is_contiguous() and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    assert targets.dtype == torch.int64 and prefix_targets.dtype == torch.int64
+    lib = _lib.load()
+    M, K = x.shape
+    V = w.shape[1] if w_in_out else w.shape[0]
+    assert (w.shape[0] if w_in_out else w.shape[1]) == K
+    n_predict = mtp_weights.shape[0]
+    dev = x.device
+    losses = torch.empty(M, dtype=torch.float32, device=dev)
+    lse = torch.empty(M, dtype=torch.float32, device=dev)
+    saved_sigma = torch.zeros((MAX_PREDICT + 1, M), dtype=torch.float32, device=dev)
+    x_f8 = torch.empty((M, K), dtype=E4M3, device=dev)
+    w_f8 = torch.empty((V, K), dtype=E4M3, device=dev)
+    codes = torch.empty(lib.ngpt_lmhead_ce_codes_bytes(M, V), dtype=torch.uint8, device=dev)
+    layout = _lib.W_IN_OUT if w_in_out else _lib.W_OUT_IN
+    ws = _workspace(lib.ngpt_lmhead_ce_fwd_workspace_bytes(M, K, V, layout), dev)
+    _lib.check(lib.ngpt_lmhead_ce_fwd_codes(_p(x), _p(w), _p(targets), _p(mtp_weights), n_predict,
+                                            _p(prefix_targets), _p(prefix_weight), M, K, V, x_s, w_s, A, B, C,
+                                            _p(losses), _p(lse), _p(saved_sigma), _p(x_f8), _p(w_f8), _p(codes), layout,
+                                            _p(ws), ws.numel(), _stream(x)), "ngpt_lmhead_ce_fwd_codes")
+    return losses, lse, saved_sigma, x_f8, w_f8, codes
+
+
+@lmhead_ce_fwd_codes.register_fake
+def _(x, w, targets, mtp_weights, prefix_targets, prefix_weight, x_s, w_s, A, B, C, w_in_out):
+    M, K = x.shape
+    V = w.shape[1] if w_in_out else w.shape[0]
+    f32 = dict(dtype=torch.float32, device=x.device)
+    ncodes = (-(-M // 256) * 256) * (-(-V // 256) * 256)
+    return (torch.empty(M, **f32), torch.empty(M, **f32), torch.empty((MAX_PREDICT + 1, M), **f32),
+            torch.empty((M, K), dtype=E4M3, device=x.device), torch.empty((V, K), dtype=E4M3, device=x.device),
+            torch.empty(ncodes, dtype=torch.uint8, device=x.device))
+
+
+@torch.library.custom_op("nanogpt::lmhead_ce_bwd_codes", mutates_args=())
+def lmhead_ce_bwd_codes(x_f8: Tensor, w_f8: Tensor, targets: Tensor, mtp_weights: Tensor, prefix_targets: Tensor,
+                        prefix_weight: Tensor, lse: Tensor, saved_sigma: Tensor, sigma_codes: Tensor,
+                        x_s: float, w_s: float, grad_s: float, grad_scale: float, A: float, B: float, C: float,
+                        w_in_out: bool) -> tuple[Tensor, Tensor]:
+    """-> (dx [M,K] bf16, dW fp32 in the weight's layout), from the forward's sigma codes."""
+    _gpu(x_f8, w_f8, targets, lse, saved_sigma, sigma_codes)
+    lib = _lib.load()
+    M, K = x_f8.shape
+    V = w_f8.shape[0]
+    assert sigma_codes.dtype == torch.uint8 and sigma_codes.is_contiguous()
+    assert sigma_codes.numel() >= lib.ngpt_lmhead_ce_codes_bytes(M, V)
+    dev = x_f8.device
+    dx = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
+    dw = torch.empty((K, V) if w_in_out else (V, K), dtype=torch.float32, device=dev)
+    layout = _lib.W_IN_OUT if w_in_out else _lib.W_OUT_IN
+    ws = _workspace(lib.ngpt_lmhead_ce_bwd_workspace_bytes(M, K, V, layout), dev)
+    _lib.check(lib.ngpt_lmhead_ce_bwd_codes(_p(x_f8), _p(w_f8), _p(targets), _p(mtp_weights), mtp_weights.shape[0],
+                                            _p(prefix_targets), _p(prefix_weight), _p(lse), _p(saved_sigma), _p(sigma_codes),
+                                            M, K, V, x_s, w_s, grad_s, grad_scale, A, B, C, _p(dx), _p(dw), layout,
+                                            _p(ws), ws.numel(), _stream(x_f8)), "ngpt_lmhead_ce_bwd_codes")
+    return dx, dw
+
+
+@lmhead_ce_bwd_codes.register_fake
+def _(x_f8, w_f8, targets, mtp_weights, prefix_targets, prefix_weight, lse, saved_sigma, sigma_codes,
+      x_s, w_s, grad_s, grad_scale, A, B, C, w_in_out):
+    M, K = x_f8.shape
+    V = w_f8.shape[0]
+    return (torch.empty((M, K), dtype=torch.bfloat16, device=x_f8.device),
+            torch.empty((K, V) if w_in_out else (V, K), dtype=torch.float32, device=x_f8.device))
+
+
 # ------------------------------------------------------------------------------------------------
 # FP8 up-projection + ReLU^2
 

@@ -142,6 +142,35 @@ def test_two_passes(amd, oracle):
     _check_dw_columns(oracle, t, sc, torch.arange(0, V, 37), lse, x_f8, w_f8, dw)
 
 
+@pytest.mark.parametrize("M,K,V", [(49152, 768, 50304), (65536 + 2048, 256, 2048)])
+def test_backward_from_sigma_codes_full_size(amd, M, K, V):
+    """Config 3, and more tokens than one pass of the backward holds: the gradients rebuilt from the forward's sigma
+    codes equal the recomputed ones bit for bit (same row statistics), and the code-writing forward agrees with the
+    plain one."""
+    g = torch.Generator().manual_seed(11)
+    d = "cuda"
+    x = torch.randn(M, K, generator=g).bfloat16().to(d)
+    w = (torch.randn(V, K, generator=g) / math.sqrt(K)).bfloat16().to(d)
+    t = torch.randint(0, V, (M,), generator=g).to(d)
+    mtp = torch.tensor([1.0], device=d)
+    pt = torch.full((M,), -1, dtype=torch.int64, device=d)
+    pw = torch.zeros(1, device=d)
+    x_s, w_s, grad_s = 100 / 448, 1.6 / 448, 0.75 / 448
+    fwd = (x, w, t, mtp, pt, pw, x_s, w_s, 23.0, 5.0, 7.5, False)
+    l0, lse0, sig0, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(*fwd)
+    l1, lse1, sig1, _, _, codes = torch.ops.nanogpt.lmhead_ce_fwd_codes(*fwd)
+    assert torch.equal(sig0, sig1) and (lse0 - lse1).abs().max().item() <= 2e-5 and (l0 - l1).abs().max().item() <= 1e-4
+    assert abs(float(l0.mean() - l1.mean())) <= 1e-5
+    tail = (x_s, w_s, grad_s, 1.0, 23.0, 5.0, 7.5, False)
+    dx0, dw0 = torch.ops.nanogpt.lmhead_ce_bwd(x_f8, w_f8, t, mtp, pt, pw, lse1, sig1, *tail)
+    dx1, dw1 = torch.ops.nanogpt.lmhead_ce_bwd_codes(x_f8, w_f8, t, mtp, pt, pw, lse1, sig1, codes, *tail)
+    assert torch.equal(dx0, dx1)
+    if M <= 65536:
+        assert torch.equal(dw0, dw1)
+    else:   # dW of several passes is accumulated with floating-point atomics: the order of the additions varies from run to run
+        assert _rel(dw1, dw0) <= 1e-5
+
+
 def test_config2_mlp_forward_full_size(amd, oracle):
     """FP8 MLP forward at M = 49152: norm + quantise producers, c_fc with the ReLU^2 epilogue, down projection."""
     g = torch.Generator().manual_seed(2)

@@ -352,7 +352,9 @@ def test_fused_lmhead_ce(amd, oracle, layout, M, K, V, n_predict, prefix):
     pwd = dev(pw) if pw is not None else torch.zeros(1, device="cuda")
     l2, lse, sig, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(dev(x), dev(wl), dev(t), dev(mtp), ptd, pwd,
                                                                sc["x_s"], sc["w_s"], 23.0, 5.0, 7.5, layout == "in_out")
-    assert torch.equal(l2, losses.detach())
+    # the autograd function's forward also wrote the sigma codes: its table entries carry the code in their low
+    # mantissa bits (2^-16 relative per term, either sign), otherwise it is this same kernel
+    assert (l2 - losses.detach()).abs().max().item() <= 1e-4
     # Per-token losses.  The MFMA sums a logit in another order than the oracle's matmul, so a logit that sits on a
     # bf16 rounding boundary may round the other way, which moves the bf16 sigma at a target column by one unit in
     # its last place (z by 23 * 2^-8 or less).  Nothing else may differ: every row's loss must equal the oracle's
@@ -408,6 +410,70 @@ def test_fused_lmhead_ce_gradient_saturates(amd, oracle, grad_scale):
     assert torch.isfinite(dx.float()).all() and torch.isfinite(dw).all()
     assert_close_gemm(dx, dx_ref)
     assert_close_gemm(dw, dw_ref)
+
+
+def _codes_case(oracle, M, K, V, seed, n_predict, prefix, below_window):
+    x, w, t, sc, mtp, pt, pw = _fused_case(oracle, M, K, V, seed=seed, n_predict=n_predict, prefix=prefix)
+    if below_window:
+        # some vocabulary rows far below zero for the first tokens: sigma under the 255 codes' range (logits < -13)
+        w[:64] = -w[64:128].abs() * 3
+        x[:below_window] = x[:below_window].abs().clamp(max=2.0) * 2
+    ptd = dev(pt) if pt is not None else torch.full((M,), -1, dtype=torch.int64, device="cuda")
+    pwd = dev(pw) if pw is not None else torch.zeros(1, device="cuda")
+    return x, w, t, sc, mtp, ptd, pwd
+
+
+@pytest.mark.parametrize("M,K,V,n_predict,prefix,in_out,below_window", [
+    (256, 128, 512, 1, False, False, 0),        # one tile
+    (640, 256, 2432, 1, False, False, 0),       # ragged token and vocabulary tiles (rows / columns of clamped duplicates)
+    (384, 768, 5120, 3, True, True, 0),         # multi-token prediction + prefix targets, (in, out) weight
+    (1024, 256, 2048, 1, False, False, 300),    # sigmas below the code window in two of four token tiles: those are recomputed
+    (1024, 256, 2048, 2, True, True, 1024),     # ... in every token tile
+])
+def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, prefix, in_out, below_window):
+    """The backward that rebuilds the e5m2 gradient from the forward's sigma codes gives bit for bit what the
+    recomputing backward gives from the same row statistics; the forward that writes the codes agrees with the plain
+    one (its table entries carry the code in their low mantissa bits: relative error 2^-16 per term, either sign)."""
+    x, w, t, sc, mtp, ptd, pwd = _codes_case(oracle, M, K, V, M + V + n_predict, n_predict, prefix, below_window)
+    wl = w.T.contiguous() if in_out else w
+    fwd = (dev(x), dev(wl), dev(t), dev(mtp), ptd, pwd, sc["x_s"], sc["w_s"], 23.0, 5.0, 7.5, in_out)
+    l0, lse0, sig0, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(*fwd)
+    l1, lse1, sig1, x_f8c, w_f8c, codes = torch.ops.nanogpt.lmhead_ce_fwd_codes(*fwd)
+    assert torch.equal(u8(x_f8), u8(x_f8c)) and torch.equal(u8(w_f8), u8(w_f8c)) and torch.equal(sig0, sig1)
+    assert (lse0 - lse1).abs().max().item() <= 2e-5 and (l0 - l1).abs().max().item() <= 1e-4
+    assert codes.numel() == -(-M // 256) * 256 * (-(-V // 256) * 256)
+    # code panel: blocks [token tile][vocabulary / 128] of 256 tokens x 128 bytes; count zero codes inside the matrix
+    blocks = codes.view(-(-M // 256), -(-V // 256) * 2, 256, 128)[:, : V // 128]
+    valid = blocks.permute(0, 2, 1, 3).reshape(-1, V)[:M]
+    assert bool((valid == 0).any()) == (below_window > 0)
+    bwd = (x_f8, w_f8, dev(t), dev(mtp), ptd, pwd, lse1, sig1)
+    tail = (sc["x_s"], sc["w_s"], sc["grad_s"], sc["grad_scale"], 23.0, 5.0, 7.5, in_out)
+    dx0, dw0 = torch.ops.nanogpt.lmhead_ce_bwd(*bwd, *tail)
+    dx1, dw1 = torch.ops.nanogpt.lmhead_ce_bwd_codes(*bwd, codes, *tail)
+    assert torch.isfinite(dw0).all() and dw0.abs().max() > 0
+    assert torch.equal(dx0, dx1) and torch.equal(dw0, dw1)
+
+
+def test_fused_lmhead_ce_backward_modes(amd, oracle, monkeypatch):
+    """FusedSoftcappedCrossEntropy in both settings of fused.CE_BACKWARD against the oracle."""
+    M, K, V = 512, 256, 3072
+    x, w, t, sc, mtp, pt, pw = _fused_case(oracle, M, K, V, seed=321, n_predict=2, prefix=True)
+    l_ref, ctx = oracle.lm_head_ce_fwd(x, t, mtp, pt, pw, w, sc["x_s"], sc["w_s"], sc["grad_s"], sc["grad_scale"], w_layout="out_in")
+    dx_ref, dw_ref = oracle.lm_head_ce_bwd(ctx)
+    grads = {}
+    for mode in ("codes", "recompute"):
+        monkeypatch.setattr(amd.fused, "CE_BACKWARD", mode)
+        xg, wg = dev(x).requires_grad_(), dev(w).float().requires_grad_()
+        losses = amd.FusedSoftcappedCrossEntropy.apply(xg, dev(t), dev(mtp), dev(pt), dev(pw), wg.bfloat16(), sc["x_s"], sc["w_s"],
+                                                       sc["grad_s"], sc["grad_scale"], 23.0, 5.0, 7.5, "out_in")
+        assert abs(float(losses.detach().mean().cpu() - l_ref.mean())) <= LOSS_TOL
+        losses.sum().backward()
+        assert_close_gemm(xg.grad, dx_ref)
+        assert_close_gemm(wg.grad, dw_ref)
+        grads[mode] = (xg.grad.clone(), wg.grad.clone())
+    # the two modes differ only through the last bits of lse (sum of exponentials), i.e. in a few e5m2 roundings
+    assert_close_gemm(grads["codes"][0], grads["recompute"][0], tol=2e-3)
+    assert_close_gemm(grads["codes"][1], grads["recompute"][1], tol=2e-3)
 
 
 def test_fused_lmhead_ce_reduces_to_cross_entropy(amd, oracle):
