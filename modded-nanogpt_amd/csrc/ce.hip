@@ -857,13 +857,19 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
     for (int c = 0; c < 4; ++c) *(v4i*)(dst + c * 128) = (v4i){(int)w[0][c], (int)w[1][c], (int)w[2][c], (int)w[3][c]};
 }
 
-// list[0 .. *count) = the token tiles of the pass whose flag is set (n <= 256 of them; one thread, a few hundred cycles)
+// list[0 .. *count) = the token tiles of the pass whose flag is set, in ascending order (n <= 256; one wave of 64 lanes,
+// four flags per lane)
 __global__ void ce_flag_list_kernel(const int* __restrict__ flags, int n, int* __restrict__ list, int* __restrict__ count) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    int c = 0;
-    for (int i = 0; i < n; ++i)
-        if (flags[i]) list[c++] = i;
-    *count = c;
+    const int lane = threadIdx.x;
+    int base = 0;
+    for (int i0 = 0; i0 < n; i0 += 64) {
+        const int i = i0 + lane;
+        const bool set = i < n && flags[i] != 0;
+        const unsigned long long m = __ballot(set);
+        if (set) list[base + __popcll(m & ((1ull << lane) - 1ull))] = i;
+        base += __popcll(m);
+    }
+    if (lane == 0) *count = base;
 }
 
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,

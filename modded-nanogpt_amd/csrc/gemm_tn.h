@@ -719,6 +719,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     const int nk = g.K / Cfg::BK;
     AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane, (g.layout & kRowsPermuted) != 0);
     Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
+    // a walk over listed rows usually has no job at all: leave before the epilogue's set-up (other walks go on, their
+    // epilogues may have something to write for a workgroup without work)
+    if constexpr (std::is_same<Iter, ListGridIter>::value) { if (!cur.valid()) return; }
 
     // `pre` walks the (job, k-step) sequence of this workgroup ahead of the MFMAs; `ahead` counts the
     // k-steps whose operand loads have been issued and not yet consumed (at most one per slot).
