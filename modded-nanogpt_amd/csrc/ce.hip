@@ -515,40 +515,42 @@ struct EpiCEFwdT {
             *(v4i*)(cd_base + (cd_lane + tn * 4096 + tm * 32)) = (v4i){(int)w0, (int)w1, (int)w2, (int)w3};
         };
         if (r0 + Cfg::BM <= V) {
-            // Batches of 8 accumulator registers, software-pipelined by hand: index arithmetic of batch b, its 8
-            // table reads, then the additions of batch b - 1, whose reads have had the arithmetic of b to return.
-            // (Left to itself the scheduler sometimes waits for every pair of reads right behind their issue.)
+            // Batches of 8 accumulator registers, software-pipelined by hand: while the 8 table reads of batch b are in
+            // flight the index arithmetic of batch b + 1 runs; then batch b is consumed (the compiler waits for every
+            // outstanding LDS read at that point, so nothing may be issued between a batch's reads and that arithmetic
+            // that it would have to wait for as well) and the reads of batch b + 1 go out.
             constexpr int NB = Cfg::TN * Cfg::TM * 2;
-            float pv[8];
-            uint32_t cw[4];
+            auto offsets_of = [&](int b, uint32_t (&off)[4]) {
+                const v16f& a = acc[(b >> 1) % Cfg::TM][b / (2 * Cfg::TM)];
 #pragma unroll
-            for (int b = 0; b <= NB; ++b) {
-                float nv[8];
-                if (b < NB) {
-                    const v16f& a = acc[(b >> 1) % Cfg::TM][b / (2 * Cfg::TM)];
-                    uint32_t off[4];
+                for (int k = 0; k < 4; ++k)
+                    off[k] = tab_offsets2(pack_logits(a[8 * (b & 1) + 2 * k] * scale, a[8 * (b & 1) + 2 * k + 1] * scale));
+            };
+            auto gather = [&](const uint32_t (&off)[4], float (&v)[8]) {
 #pragma unroll
-                    for (int k = 0; k < 4; ++k)
-                        off[k] = tab_offsets2(pack_logits(a[8 * (b & 1) + 2 * k] * scale, a[8 * (b & 1) + 2 * k + 1] * scale));
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        nv[2 * k] = tab_at(tab, off[k] & 0xffffu);
-                        nv[2 * k + 1] = tab_at(tab, off[k] >> 16);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
+                for (int k = 0; k < 4; ++k) {
+                    v[2 * k] = tab_at(tab, off[k] & 0xffffu);
+                    v[2 * k + 1] = tab_at(tab, off[k] >> 16);
                 }
-                if (b > 0) {
-                    sum[(b - 1) / (2 * Cfg::TM)] += ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
-                    if constexpr (CODES) {
-                        const int q = b - 1;
-                        cw[2 * (q & 1)] = pack_codes4(pv[0], pv[1], pv[2], pv[3]);
-                        cw[2 * (q & 1) + 1] = pack_codes4(pv[4], pv[5], pv[6], pv[7]);
-                        if (q & 1) code_store((q >> 1) % Cfg::TM, q / (2 * Cfg::TM), cw[0], cw[1], cw[2], cw[3]);
-                    }
-                }
+            };
+            float cur[8];
+            uint32_t off[4], cw[4];
+            offsets_of(0, off);
+            gather(off, cur);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int k = 0; k < 8; ++k) pv[k] = nv[k];
+            for (int b = 0; b < NB; ++b) {
+                if (b + 1 < NB) offsets_of(b + 1, off);
+                __builtin_amdgcn_sched_barrier(0);
+                sum[b / (2 * Cfg::TM)] += ((cur[0] + cur[1]) + (cur[2] + cur[3])) + ((cur[4] + cur[5]) + (cur[6] + cur[7]));
+                if constexpr (CODES) {
+                    cw[2 * (b & 1)] = pack_codes4(cur[0], cur[1], cur[2], cur[3]);
+                    cw[2 * (b & 1) + 1] = pack_codes4(cur[4], cur[5], cur[6], cur[7]);
+                    if (b & 1) code_store((b >> 1) % Cfg::TM, b / (2 * Cfg::TM), cw[0], cw[1], cw[2], cw[3]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (b + 1 < NB) gather(off, cur);
+                __builtin_amdgcn_sched_barrier(0);
             }
         } else {   // last vocabulary tile: rows past V are clamped duplicates and must not count
 #pragma unroll
