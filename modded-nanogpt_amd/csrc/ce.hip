@@ -113,7 +113,9 @@ __global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc, bool embed
     tabE[i] = e;
 }
 
-// dcode[c] = D of the sigma with code c (the expression of ce_table_kernel's tabD), dcode[0] = 0.
+// dcode[c] = D of the sigma with code c (the expression of ce_table_kernel's tabD), dcode[0] = 0; dcode[256] = D of
+// the largest sigma below the window, which bounds D of every sigma there if D grows with sigma up to it, and
+// infinity if it does not (D = exp(A sigma - A) sigma (1 - sigma) grows on (0, 1/2) whatever A > 0 is).
 __global__ void ce_dcode_kernel(float* dcode, Softcap sc) {
     const int c = threadIdx.x;
     float d = 0.0f;
@@ -122,6 +124,10 @@ __global__ void ce_dcode_kernel(float* dcode, Softcap sc) {
         d = softcap_E(s, sc) * s * (1.0f - s);
     }
     dcode[c] = d;
+    if (c == 0) {
+        const float s = bf16_bits_to_f32((uint32_t)(SIGC_LOW - 1));
+        dcode[256] = s < 0.5f ? softcap_E(s, sc) * s * (1.0f - s) : __builtin_inff();
+    }
 }
 
 __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
@@ -811,8 +817,11 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
 // pass's dlogits panel (vocabulary-major, tokens of a k-step in dw_pos order), dl = e5m2_sat(rowf[token] * dcode[code]):
 // the same product and conversion as EpiDlStore, so the two agree bit for bit.  One workgroup moves 128 tokens x 128
 // vocabulary entries: 16 KiB of one code block in, converted on the way into LDS, transposed as in
-// panel_transpose_kernel, 16 KiB of one panel block out.  A code of 0 (sigma below the window) inside the matrix sets
-// the flag of its token tile: EpiDlStore then recomputes that tile's part of the panel from the logits.
+// panel_transpose_kernel, 16 KiB of one panel block out.  A code of 0 (sigma below the window) stands for a gradient of
+// zero, which is exact whenever |rowf| * D(largest sigma below the window) is under half the smallest e5m2 subnormal
+// (2^-17): every such product then rounds to zero in the recompute epilogue too.  Only a code of 0 inside the matrix in
+// a row whose factor is larger than that sets the flag of its token tile: EpiDlStore then recomputes that tile's part
+// of the panel from the logits.
 __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __restrict__ codes, int nkp, int m0, int M,
                                                              const float* __restrict__ rowf, const float* __restrict__ dcode,
                                                              int nkt, uint8_t* __restrict__ dl_panel, int* __restrict__ flags) {
@@ -821,6 +830,7 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
     __shared__ float dtab[256];
     const int kv = blockIdx.x, a = blockIdx.y, tid = threadIdx.x;
     dtab[tid] = dcode[tid];
+    const float d_below = dcode[256];
     __syncthreads();
     auto word_at = [&](int r, int w) -> uint32_t& { return tile[r * kStride + (w ^ (((r >> 4) & 7) << 2))]; };
     const int tok0 = m0 + a * 128;
@@ -834,7 +844,7 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const uint32_t w = (uint32_t)c[k];
-            below |= (tok0 + r < M) && (((w - 0x01010101u) & ~w & 0x80808080u) != 0u);
+            below |= (tok0 + r < M) && (((w - 0x01010101u) & ~w & 0x80808080u) != 0u) && !(fabsf(rf) * d_below < 0x1p-17f);
             word_at(r, ch * 4 + k) = f32x4_to_e5m2_sat<true>(rf * dtab[w & 0xffu], rf * dtab[(w >> 8) & 0xffu],
                                                              rf * dtab[(w >> 16) & 0xffu], rf * dtab[w >> 24]);
         }
@@ -1227,7 +1237,7 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
     const float coef = make_coef(A, C, grad_s, grad_scale);
     CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
     ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc, false);
-    float* dcode = tabE;                     // the backward does not read tabE: its first 256 entries serve as the code table
+    float* dcode = tabE;                     // the backward does not read tabE: its first 257 entries serve as the code table
     if (sigma_codes) ce_dcode_kernel<<<1, 256, 0, st>>>(dcode, sc);
     ce_rowf_kernel<<<(M + 255) / 256, 256, 0, st>>>(lse, ca, sc, coef, rowf, big);
     if (int e = check_launch("ce_rowf_kernel")) return e;

@@ -423,14 +423,16 @@ def _codes_case(oracle, M, K, V, seed, n_predict, prefix, below_window):
     return x, w, t, sc, mtp, ptd, pwd
 
 
-@pytest.mark.parametrize("M,K,V,n_predict,prefix,in_out,below_window", [
-    (256, 128, 512, 1, False, False, 0),        # one tile
-    (640, 256, 2432, 1, False, False, 0),       # ragged token and vocabulary tiles (rows / columns of clamped duplicates)
-    (384, 768, 5120, 3, True, True, 0),         # multi-token prediction + prefix targets, (in, out) weight
-    (1024, 256, 2048, 1, False, False, 300),    # sigmas below the code window in two of four token tiles: those are recomputed
-    (1024, 256, 2048, 2, True, True, 1024),     # ... in every token tile
+@pytest.mark.parametrize("M,K,V,n_predict,prefix,in_out,below_window,grad_scale", [
+    (256, 128, 512, 1, False, False, 0, 1.0),        # one tile
+    (640, 256, 2432, 1, False, False, 0, 1.0),       # ragged token and vocabulary tiles (rows / columns of clamped duplicates)
+    (384, 768, 5120, 3, True, True, 0, 1.0),         # multi-token prediction + prefix targets, (in, out) weight
+    (1024, 256, 2048, 1, False, False, 300, 1.0),    # sigmas below the code window in two of four token tiles: those are recomputed
+    (1024, 256, 2048, 2, True, True, 1024, 1.0),     # ... in every token tile
+    (1024, 256, 2048, 1, False, False, 300, 0.01),   # ... with row factors so small that those gradients are exact zeros: nothing is recomputed
+    (1024, 256, 2048, 1, False, False, 300, 0.5),    # ... around the limit between the two (some rows on either side)
 ])
-def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, prefix, in_out, below_window):
+def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, prefix, in_out, below_window, grad_scale):
     """The backward that rebuilds the e5m2 gradient from the forward's sigma codes gives bit for bit what the
     recomputing backward gives from the same row statistics; the forward that writes the codes agrees with the plain
     one (its table entries carry the code in their low mantissa bits: relative error 2^-16 per term, either sign)."""
@@ -447,10 +449,19 @@ def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, pr
     valid = blocks.permute(0, 2, 1, 3).reshape(-1, V)[:M]
     assert bool((valid == 0).any()) == (below_window > 0)
     bwd = (x_f8, w_f8, dev(t), dev(mtp), ptd, pwd, lse1, sig1)
-    tail = (sc["x_s"], sc["w_s"], sc["grad_s"], sc["grad_scale"], 23.0, 5.0, 7.5, in_out)
+    tail = (sc["x_s"], sc["w_s"], sc["grad_s"], grad_scale, 23.0, 5.0, 7.5, in_out)
     dx0, dw0 = torch.ops.nanogpt.lmhead_ce_bwd(*bwd, *tail)
     dx1, dw1 = torch.ops.nanogpt.lmhead_ce_bwd_codes(*bwd, codes, *tail)
     assert torch.isfinite(dw0).all() and dw0.abs().max() > 0
+    if below_window and not prefix:
+        # rows with a sigma below the window, and their factor coef * S_w * exp(A - lse) against the limit
+        # 2^-17 / D(largest sigma below the window) = 1138 under which those gradients are exact zeros
+        rows0 = (valid == 0).any(dim=1)
+        rowf = grad_scale * (23.0 / 7.5) / sc["grad_s"] * float(mtp.sum()) * torch.exp(23.0 - lse1[rows0])
+        if grad_scale == 0.01:
+            assert (rowf < 1100).all()        # nothing is recomputed
+        if grad_scale == 1.0:
+            assert (rowf > 1200).any()        # some token tile is
     assert torch.equal(dx0, dx1) and torch.equal(dw0, dw1)
 
 
