@@ -517,6 +517,35 @@ def workload_ceiling(args, amd, dev) -> int:
         except Exception as e:    # a shape the library refuses is reported, not fatal
             res["rows"].append({"what": f"vendor library torch._scaled_mm {Mm} x {Nn} x {Kk}", "error": str(e)[:200]})
         del a, b
+    # What the output of a store-heavy epilogue costs, and whether it matters which waves carry it: the FP8 c_fc
+    # (49152 x 3072 x 768, ReLU^2, whole-line stores) complete, with half of its output stored by waves that also
+    # issue operand loads, with the same half stored by waves that issue none (the memory counter retires in issue
+    # order, so only such waves never wait for their stores), and with nothing stored.
+    Mm, Nn, Kk = 49152, 3072, 768
+    xq = torch.randn(Mm, Kk, device=dev).to(E4)
+    wq = (torch.randn(Nn, Kk, device=dev) * 0.05).to(E4)
+    post = torch.zeros(Mm, Nn, dtype=torch.bfloat16, device=dev)
+    modes = ((0, "complete"), (1, "half of the output, stored by 4 of 8 waves; all 8 waves issue operand loads"),
+             (2, "half of the output, stored by the 4 waves that issue no operand load"),
+             (3, "epilogue skipped; all 8 waves issue operand loads"), (4, "epilogue skipped; 4 waves issue operand loads"))
+    samples = {m: [] for m, _ in modes}
+    for rep in range(7):
+        for m, _ in modes:
+            lib.ngpt_tuning_set(5, m)
+            call = lambda: lib.ngpt_fc_relu2_fwd(xq.data_ptr(), wq.data_ptr(), one.data_ptr(), Mm, Nn, Kk, post.data_ptr(), None, None, None, 0, st)
+            for _ in range(3):
+                assert call() == 0, lib.ngpt_last_error()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(30):
+                call()
+            e1.record()
+            torch.cuda.synchronize()
+            samples[m].append(e0.elapsed_time(e1) / 30)
+    lib.ngpt_tuning_set(5, 0)
+    res["store_rows"] = [{"what": f"FP8 c_fc {Mm} x {Nn} x {Kk}, {what}", "ms": statistics.median(samples[m]), "ms_min": min(samples[m])}
+                         for m, what in modes]
     print(json.dumps(res))
     return 0
 

@@ -444,4 +444,21 @@ struct EpiRelu2T {
     }
 };
 
+#ifdef NGPT_BENCH_BUILD
+// Timing aid: EpiRelu2Lines in which only waves store_from .. NWAVES - 1 run the epilogue for their part of the tile
+// (the rest of the output is never written).  With TileCfg::LOADERS = 4 and store_from = 4 the storing waves are the
+// ones that issue no operand load: what the output costs when it does not sit in a loading wave's memory counter.
+struct EpiRelu2LinesHalf : EpiRelu2Lines {
+    int store_from;
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co, uint8_t* scratch, int lane) {
+        if ((int)(threadIdx.x >> 6) < store_from) {
+            stored_all = false;   // this wave issued no store: no relaxed wait
+            return;
+        }
+        EpiRelu2Lines::template tile<Cfg>(acc, r0, c0, co, scratch, lane);
+    }
+};
+#endif
+
 }  // namespace ngpt

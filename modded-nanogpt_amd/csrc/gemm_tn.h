@@ -61,13 +61,18 @@ struct GemmOperands {
     const int* row_count;
 };
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1, int LOADERS_ = 0>
 struct TileCfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, NSTAGES = NSTAGES_;
     static constexpr int WGS_PER_CU = WGS_PER_CU_;                 // co-resident workgroups the register budget allows
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int NWAVES = WAVES_M * WAVES_N;
     static constexpr int THREADS = NWAVES * 64;
+    // Waves that issue the operand loads (the first LOADERS of the workgroup; 0 = all of them).  With fewer loaders
+    // than waves the other waves never wait on the memory counter in the k-loop: the stores of their epilogue drain
+    // while the next tile is computed (the counter retires in issue order, so a wave that loads cannot do that).
+    static constexpr int LOADERS = LOADERS_ ? LOADERS_ : NWAVES;
+    static constexpr bool SPLIT_DUTIES = LOADERS != NWAVES;
     static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;   // wave tile
     static constexpr int TM = WTM / 32, TN = WTN / 32;             // MFMA tiles per wave
     static constexpr int KSUB = BK / 64;                           // 64-byte MFMA contraction steps per k-step
@@ -77,13 +82,14 @@ struct TileCfg {
     static constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int SMEM_BYTES = NSTAGES * STAGE_BYTES;
-    static constexpr int A_LOADS = BM / ROWS_PER_LOAD / NWAVES;    // wave-level loads per k-step
-    static constexpr int B_LOADS = BN / ROWS_PER_LOAD / NWAVES;
+    static constexpr int A_LOADS = BM / ROWS_PER_LOAD / LOADERS;   // wave-level loads per k-step and loading wave
+    static constexpr int B_LOADS = BN / ROWS_PER_LOAD / LOADERS;
     static constexpr int LOADS = A_LOADS + B_LOADS;
     static constexpr int WAVE_SCRATCH = STAGE_BYTES / NWAVES;      // epilogue staging per wave
     static_assert(BK == 64 || BK == 128, "BK is 64 or 128 bytes");
     static_assert(NSTAGES >= 2 && NSTAGES <= 4, "2..4 LDS stages");
-    static_assert(BM % (ROWS_PER_LOAD * NWAVES) == 0 && BN % (ROWS_PER_LOAD * NWAVES) == 0,
+    static_assert(LOADERS <= NWAVES && BM % (ROWS_PER_LOAD * LOADERS) == 0 && BN % (ROWS_PER_LOAD * LOADERS) == 0 &&
+                      BM % (ROWS_PER_LOAD * NWAVES) == 0 && BN % (ROWS_PER_LOAD * NWAVES) == 0,
                   "tile rows must split over waves");
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be made of 32x32 MFMA tiles");
     // LDS swizzle: chunk q of row r is stored at chunk position q ^ swz(r)
@@ -140,7 +146,7 @@ struct LaneOffsets {
     // lanes that a transposing read serves together hit 32 distinct 8-byte bank pairs (see frag offsets below).
     // `lim` = columns of this operand left from the tile's origin (a multiple of 8): chunks past it are clamped.
     static __device__ uint32_t tr16_off(int load, int wave, int lane, int64_t ld, int lim) {
-        const int m = 2 * (wave + load * Cfg::NWAVES) + (lane >> 5);
+        const int m = 2 * (wave + load * Cfg::LOADERS) + (lane >> 5);
         int chunk = (lane & 31) ^ (4 * (m & 3));
         chunk = min(chunk, lim / 8 - 1);
         return (uint32_t)((int64_t)m * ld + chunk * 16);
@@ -156,12 +162,12 @@ struct LaneOffsets {
             if (a_transposed) {
                 // 1 KiB piece `c32` of the k-step's 32: half (token block) c32 / 16, contraction rows 8 * (c32 % 16) ..+7;
                 // the 16-byte chunk q of contraction row r lands at chunk position q ^ (r & 7)
-                const int c32 = wave + i * Cfg::NWAVES;
+                const int c32 = wave + i * Cfg::LOADERS;
                 const int r = 8 * (c32 & 15) + lrow;
                 a_off[i] = (uint32_t)((c32 >> 4) * kPanelBytes + r * 128 + ((lchunk ^ (r & 7)) << 4));
                 continue;
             }
-            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
+            int R = (wave + i * Cfg::LOADERS) * Cfg::ROWS_PER_LOAD + lrow;
             int q = lchunk ^ Cfg::swz(R);
             if (g.layout & kBlockedA) { a_off[i] = (uint32_t)(R * 128 + q * 16); continue; }   // padded: no clamp
             int rr = min(R, g.R - 1 - r0);                       // clamp rows past the end
@@ -173,7 +179,7 @@ struct LaneOffsets {
 #pragma unroll
         for (int i = 0; i < Cfg::B_LOADS; ++i) {
             if (b_tr16) { b_off[i] = tr16_off(i, wave, lane, g.ldb, g.C - c0); continue; }
-            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
+            int R = (wave + i * Cfg::LOADERS) * Cfg::ROWS_PER_LOAD + lrow;
             int q = lchunk ^ Cfg::swz(R);
             if (g.layout & kBlockedB) { b_off[i] = (uint32_t)(R * 128 + q * 16); continue; }
             int rr = min(R, g.C - 1 - c0);
@@ -302,16 +308,20 @@ struct TileMainloop {
             a_next += a_step;
         }
         b_next += b_step;
+        if (!loader()) return;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i)
-            global_to_lds16(ab + lo.a_off[i], s + (wave + i * Cfg::NWAVES) * 1024);
+            global_to_lds16(ab + lo.a_off[i], s + (wave + i * Cfg::LOADERS) * 1024);
     }
+    __device__ __forceinline__ bool loader() const { return !Cfg::SPLIT_DUTIES || wave < Cfg::LOADERS; }
     __device__ void issue_loads_b(uint8_t* smem) {
         if (b_pending == nullptr) return;
         uint8_t* s = smem + pending_stage * Cfg::STAGE_BYTES;
+        if (loader()) {
 #pragma unroll
-        for (int i = 0; i < Cfg::B_LOADS; ++i)
-            global_to_lds16(b_pending + lo.b_off[i], s + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
+            for (int i = 0; i < Cfg::B_LOADS; ++i)
+                global_to_lds16(b_pending + lo.b_off[i], s + Cfg::A_BYTES + (wave + i * Cfg::LOADERS) * 1024);
+        }
         b_pending = nullptr;
     }
 
@@ -745,8 +755,10 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     ml.issue_loads_b(smem);
     epi.begin(bid, G, smem_all);
     // operands of the first k-step
-    if (ahead == 2) wait_vmem_le<Cfg::LOADS>();
-    else wait_vmem_le<0>();
+    if (ml.loader()) {
+        if (ahead == 2) wait_vmem_le<Cfg::LOADS>();
+        else wait_vmem_le<0>();
+    }
     wg_barrier();
 
     v16f acc[Cfg::TM][Cfg::TN];
@@ -782,7 +794,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
             auto sync = [&]() {
                 // only the wait differs between the relaxed and the plain first k-step: a scalar branch around it
                 // instead of a second copy of the k-step
-                if (decltype(first)::value && EpiTileStores<Epi>::value > 0 && relaxed) wait_vmem_le<EpiTileStores<Epi>::value>();
+                // (split duties: a loading wave stores nothing, the others wait for no load -- the barrier tells them)
+                if (Cfg::SPLIT_DUTIES) { if (ml.loader()) wait_vmem_le<0>(); }
+                else if (decltype(first)::value && EpiTileStores<Epi>::value > 0 && relaxed) wait_vmem_le<EpiTileStores<Epi>::value>();
                 else wait_vmem_le<0>();
                 if (!(ablate & 4)) wg_barrier();
             };
