@@ -336,9 +336,11 @@ struct EpiRelu2Lines {
         // address = wave-uniform pointer (tile origin + the block's and line group's fixed position) + ONE per-lane offset
         uint16_t* origin = post + ((int64_t)c0 * ld + r0);
         const uint32_t lane_off = (uint32_t)(co.wave_col0 + rd_row) * (uint32_t)ld + (uint32_t)(co.wave_row0 + rd_chunk * 8);
+        // relu(bf16(x)) == bf16(relu(x)) (rounding keeps the sign, a NaN becomes 0 either way): the maximum is taken on
+        // the product, which spares the canonicalising pass that a maximum on re-expanded bf16 bits needs
         auto relu2 = [&](float a0, float a1) {
-            const uint32_t pre = cvt_pk_bf16(a0 * scale, a1 * scale);
-            const float c0f = fmaxf(__uint_as_float(pre << 16), 0.0f), c1f = fmaxf(__uint_as_float(pre & 0xffff0000u), 0.0f);
+            const uint32_t pre = cvt_pk_bf16(fmaxf(a0 * scale, 0.0f), fmaxf(a1 * scale, 0.0f));
+            const float c0f = __uint_as_float(pre << 16), c1f = __uint_as_float(pre & 0xffff0000u);
             return (int)cvt_pk_bf16(c0f * c0f, c1f * c1f);
         };
 #pragma unroll
@@ -407,8 +409,9 @@ struct EpiRelu2T {
                 for (int v = 0; v < 16; v += 2) {
                     const int dr = co.dr(tm, v), dc = tn * 32;
                     // c = bf16(acc * dequant); post = bf16(max(c, 0)^2): both roundings by the packed converter
-                    const uint32_t pre = cvt_pk_bf16(acc[tm][tn][v] * scale, acc[tm][tn][v + 1] * scale);
-                    const float c0f = fmaxf(__uint_as_float(pre << 16), 0.0f), c1f = fmaxf(__uint_as_float(pre & 0xffff0000u), 0.0f);
+                    // (the maximum on the product: relu(bf16(x)) == bf16(relu(x)), see EpiRelu2Lines)
+                    const uint32_t pre = cvt_pk_bf16(fmaxf(acc[tm][tn][v] * scale, 0.0f), fmaxf(acc[tm][tn][v + 1] * scale, 0.0f));
+                    const float c0f = __uint_as_float(pre << 16), c1f = __uint_as_float(pre & 0xffff0000u);
                     const uint32_t pk = cvt_pk_bf16(c0f * c0f, c1f * c1f);
                     uint16_t* pu = origin + ((int64_t)dr * ld + dc);
                     const bool ok0 = full || (dr < rlim && dc < clim), ok1 = full || (dr + 1 < rlim && dc < clim);
