@@ -268,6 +268,14 @@ def emit(args, lib, desc, tokens, flops, ms, median_ms, kernels, work, traffic_k
 # ---------------------------------------------------------------------------------------------- workloads
 def workload_lmhead_ce(args, amd, lib, dev):
     x, w, t, sc = make_cfg3(seed=0)
+    if args.tail_columns:
+        # What a trained model looks like to the sigma-code backward: the last vocabulary entries (ids that never occur
+        # as targets, such as the padding ids 50257..50303) have logits near -20 for every token, below the code window,
+        # and the rows' factors are above the limit under which such gradients are exact zeros (here by a larger
+        # grad_scale; in a trained model by a smaller lse).  The tiles that hold those columns are then recomputed.
+        x[:, 0] = 13.5
+        w[w.shape[0] - args.tail_columns:, 0] = -1.5      # inside the e4m3 range of w / w_s
+        sc["grad_scale"] = 64.0
     xd, wd, td = x.to(dev), w.to(dev), t.to(dev)
     mtp = torch.tensor([1.0], device=dev)
     pt = torch.full((M,), -1, dtype=torch.int64, device=dev)
@@ -300,6 +308,8 @@ def workload_lmhead_ce(args, amd, lib, dev):
         work["dlogits_from_codes"] = (2.0 * M * V, "hbm")
         mode_desc = "the forward keeps one sigma code byte per logit for the backward (three GEMM passes)"
     extra = {"mean_loss": float(out[0].mean()), "ce_backward": args.ce_backward}
+    if args.tail_columns:
+        extra["tail_columns"] = args.tail_columns
     if not args.no_other_mode:  # the other mode of the backward, timed the same way on a few steps, for the record
         _, o_ms, o_med, _ = run_timed(lib, other, max(5, args.steps // 5), 3)
         extra["other_mode"] = {"ce_backward": "recompute" if codes_mode else "codes", "ms_per_step": o_ms,
@@ -561,6 +571,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ce-backward", choices=("codes", "recompute"), default="codes",
                     help="headline workload: where the backward takes the e5m2 gradient of the logits from")
+    ap.add_argument("--tail-columns", type=int, default=0,
+                    help="headline workload: this many of the last vocabulary entries get logits far below the sigma-code window "
+                         "in every row (and grad_scale = 64, so that they matter): measures the fallback of the codes backward")
     ap.add_argument("--no-other-mode", action="store_true", help="headline workload: do not also time the other --ce-backward mode")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy, the known-size kernel that scales "

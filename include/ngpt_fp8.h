@@ -282,8 +282,8 @@ int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const int64_t* tar
  * also writes sigma_codes, ngpt_lmhead_ce_codes_bytes(M, V) bytes; the backward turns them into the e5m2 gradient
  * (bit-identical to what ngpt_lmhead_ce_bwd recomputes) without running the logits GEMM a second time.  A sigma below
  * the 255 codes' range (logits under about -13 with A, B, C = 23, 5, 7.5) reads as a zero gradient where that is exact
- * (the row's factor is small enough for every such gradient to round to zero in e5m2); token tiles where it is not are
- * detected on the device and recomputed from the logits as ngpt_lmhead_ce_bwd does, so results never depend on the range.
+ * (the row's factor is small enough for every such gradient to round to zero in e5m2); the 256 x 256 tiles of the logits
+ * where it is not are listed on the device and recomputed as ngpt_lmhead_ce_bwd does, so results never depend on the range.
  * Everything else (arguments, alignment, workspaces) is as in ngpt_lmhead_ce_fwd / ngpt_lmhead_ce_bwd. */
 int64_t ngpt_lmhead_ce_codes_bytes(int M, int V);
 int ngpt_lmhead_ce_fwd_codes(const void* x_bf16, const void* w_bf16, const int64_t* targets,

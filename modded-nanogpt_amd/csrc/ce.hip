@@ -820,11 +820,13 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
 // panel_transpose_kernel, 16 KiB of one panel block out.  A code of 0 (sigma below the window) stands for a gradient of
 // zero, which is exact whenever |rowf| * D(largest sigma below the window) is under half the smallest e5m2 subnormal
 // (2^-17): every such product then rounds to zero in the recompute epilogue too.  Only a code of 0 inside the matrix in
-// a row whose factor is larger than that sets the flag of its token tile: EpiDlStore then recomputes that tile's part
-// of the panel from the logits.
+// a row whose factor is larger than that puts the 256 x 256 tile it lies in on the list of tiles (each tile once:
+// flags) that EpiDlStore then recomputes from the logits.  Such entries cluster in vocabulary columns (tokens
+// that never occur as targets keep being pushed down), so the list stays a small part of the matrix.
 __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __restrict__ codes, int nkp, int m0, int M,
                                                              const float* __restrict__ rowf, const float* __restrict__ dcode,
-                                                             int nkt, uint8_t* __restrict__ dl_panel, int* __restrict__ flags) {
+                                                             int nkt, uint8_t* __restrict__ dl_panel, int nvt, int* __restrict__ flags,
+                                                             int* __restrict__ list, int* __restrict__ count) {
     constexpr int kStride = 33;
     __shared__ uint32_t tile[128 * kStride];
     __shared__ float dtab[256];
@@ -849,8 +851,10 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
                                                              rf * dtab[(w >> 16) & 0xffu], rf * dtab[w >> 24]);
         }
     }
-    if (below) flags[(tok0 - m0) >> 8] = 1;
-    __syncthreads();
+    if (__syncthreads_or(below) && tid == 0) {
+        const int tt = (tok0 - m0) >> 8, vt = kv >> 1;
+        if (atomicExch(&flags[tt * nvt + vt], 1) == 0) list[atomicAdd(count, 1)] = (tt << 16) | vt;
+    }
     // as panel_transpose_kernel with PERM = 2: piece `sub` of a vocabulary entry's 128-byte row holds the tokens
     // 32 (sub / 2) + 8 g + 4 (sub % 2) + i at byte 4 g + i; the four code columns 4 cgp ..+3 of a thread are the
     // vocabulary entries vloc ..+3 (dw_pos order of the code panel's bytes undone)
@@ -867,21 +871,6 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
     uint8_t* dst = dl_panel + ((int64_t)(kv >> 1) * nkt + a) * kPanelBytes + ((kv & 1) * 128 + vloc) * 128 + sub * 16;
 #pragma unroll
     for (int c = 0; c < 4; ++c) *(v4i*)(dst + c * 128) = (v4i){(int)w[0][c], (int)w[1][c], (int)w[2][c], (int)w[3][c]};
-}
-
-// list[0 .. *count) = the token tiles of the pass whose flag is set, in ascending order (n <= 256; one wave of 64 lanes,
-// four flags per lane)
-__global__ void ce_flag_list_kernel(const int* __restrict__ flags, int n, int* __restrict__ list, int* __restrict__ count) {
-    const int lane = threadIdx.x;
-    int base = 0;
-    for (int i0 = 0; i0 < n; i0 += 64) {
-        const int i = i0 + lane;
-        const bool set = i < n && flags[i] != 0;
-        const unsigned long long m = __ballot(set);
-        if (set) list[base + __popcll(m & ((1ull << lane) - 1ull))] = i;
-        base += __popcll(m);
-    }
-    if (lane == 0) *count = base;
 }
 
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
@@ -1181,11 +1170,12 @@ extern "C" int ngpt_lmhead_ce_fwd_static(const void* x_bf16, const void* w_bf16,
 static int64_t bwd_part_bytes(int64_t Mc, int64_t Mt, int K, int V) {
     return std::max(balanced_part_bytes((int)Mc, K, V), std::max(balanced_part_bytes(V, K, (int)Mt), balanced_part_bytes(K, V, (int)Mt)));
 }
-constexpr int64_t kFlagBytes = 4096;    // codes backward: flags [256] | list [256] | count of the pass's token tiles
+// codes backward: count | flags [tiles] | list [tiles] of the 256 x 256 tiles of one pass's logits
+static int64_t flag_bytes(int64_t Mt, int64_t Vp) { return align_up((1 + 2 * (Mt / 256) * (Vp / 256)) * 4, 256); }
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
     int64_t Mc = bwd_chunk_rows(M), Mt = round256(Mc), Kp = round256(K), Vp = round256(V);
-    return align_up(2 * TAB_BYTES, 256) + 2 * round256(M) * 4 + Kp * Mt + Kp * (int64_t)V + Vp * Mt + bwd_part_bytes(Mc, Mt, K, V) + kFlagBytes;
+    return align_up(2 * TAB_BYTES, 256) + 2 * round256(M) * 4 + Kp * Mt + Kp * (int64_t)V + Vp * Mt + bwd_part_bytes(Mc, Mt, K, V) + flag_bytes(Mt, Vp);
 }
 
 extern "C" int64_t ngpt_lmhead_ce_codes_bytes(int M, int V) { return round256(M) * round256(V); }
@@ -1228,10 +1218,11 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
     ws += Vp * Mt_max;
     float* parts = (float*)ws;
     ws += bwd_part_bytes(Mc_max, Mt_max, K, V);
-    int* flags = (int*)ws;                   // per token tile of the pass: some sigma of it lies below the code window
-    int* list = flags + 256;
-    int* count = list + 256;
-    static_assert(BWD_CHUNK_ROWS / 256 <= 256 && 3 * 256 * 4 <= kFlagBytes, "flag and list arrays of one pass");
+    int* count = (int*)ws;                   // number of listed tiles
+    int* flags = count + 1;                  // per 256 x 256 tile of the pass's logits: a sigma of it lies below the code window and matters
+    int* list = flags + (Mt_max / 256) * (Vp / 256);
+    static_assert(BWD_CHUNK_ROWS / 256 < 65536, "a list entry holds the token tile in its upper 16 bits");
+    if (Vp / 256 >= 65536) return fail(NGPT_ERANGE, "%s: V=%d", who, V);
 
     Softcap sc = make_softcap(A, B, C);
     const float coef = make_coef(A, C, grad_s, grad_scale);
@@ -1262,18 +1253,17 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
         epi.nkt = nkt;
         epi.scale = x_s * w_s;
         if (sigma_codes) {
-            // 1'. the pass's dlogits panel from the forward's sigma codes; token tiles with a sigma below the code
-            //     window (none, normally) are then redone from the logits
+            // 1'. the pass's dlogits panel from the forward's sigma codes; tiles with a sigma below the code window
+            //     that matters (none, normally) are then redone from the logits
             ProfileScope prof(PROF_CE_DLOGITS, st);
-            const int nt = Mt / 256;
-            fill_f32_kernel<<<1, 256, 0, st>>>((float*)flags, nt, 0.0f);
+            const int nvt = (int)(Vp / 256), nflags = 1 + (Mt / 256) * nvt;
+            fill_f32_kernel<<<(nflags + 255) / 256, 256, 0, st>>>((float*)count, nflags, 0.0f);
             ce_codes_to_dl_kernel<<<dim3(V / 128, nkt), 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, rowf, dcode,
-                                                                      nkt, dw_panel, flags);
+                                                                      nkt, dw_panel, nvt, flags, list, count);
             if (int e = check_launch("ce_codes_to_dl_kernel")) return e;
-            ce_flag_list_kernel<<<1, 64, 0, st>>>(flags, nt, list, count);
-            g.row_list = list;
-            g.row_count = count;
-            if (int e = launch_grid_kernel<MainCfg, ListGridIter>(g, epi, st, -1, "lm_head CE backward (dlogits of the flagged token tiles)")) return e;
+            g.tile_list = list;
+            g.tile_count = count;
+            if (int e = launch_grid_kernel<MainCfg, TileListIter>(g, epi, st, -1, "lm_head CE backward (dlogits of the listed tiles)")) return e;
         } else if (int e = launch_grid_kernel<MainCfg, GridIter>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
         ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, nkt, dw_panel);

@@ -56,9 +56,9 @@ struct GemmOperands {
     int layout;         // kBlockedA | kBlockedB | kRowsPermuted
     int full_tiles;     // the first full_tiles tiles (in walk order) are never split; 0 = `splits` applies to every tile
     int a_rows_pad;     // transposed A only: R rounded up to 256
-    // ListGridIter only: the kernel works on the tile rows row_list[0 .. *row_count) instead of on all of them
-    const int* row_list;
-    const int* row_count;
+    // TileListIter only: the kernel works on the tiles tile_list[0 .. *tile_count) instead of on all of them
+    const int* tile_list;
+    const int* tile_count;
 };
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1, int LOADERS_ = 0>
@@ -630,17 +630,21 @@ struct GridIter {
     }
 };
 
-// GridIter over a subset of the tile rows: row_list[i], i < *row_count (both written by an earlier kernel and
-// read through the constant address space, i.e. as scalar loads that stay out of the vector memory counter).
-struct ListGridIter : GridIter {
+// GridIter over a list of tiles: tile_list[i] = (tile row << 16) | tile column, i < *tile_count (both written by an
+// earlier kernel and read through the constant address space, i.e. as scalar loads that stay out of the vector memory
+// counter).  The base class walks a 1 x count grid; its column index is the position in the list.
+struct TileListIter : GridIter {
     const int* list;
-    static __device__ GemmOperands listed(GemmOperands g, int BM) {
-        g.R = ((const __attribute__((address_space(4))) int*)(uintptr_t)g.row_count)[0] * BM;
+    static __device__ GemmOperands listed(GemmOperands g, int BM, int BN) {
+        g.R = BM;
+        g.C = ((const __attribute__((address_space(4))) int*)(uintptr_t)g.tile_count)[0] * BN;
         return g;
     }
-    __device__ ListGridIter(const GemmOperands& g, int BM, int BN, int bid_, int G_)
-        : GridIter(listed(g, BM), BM, BN, bid_, G_), list(g.row_list) {}
-    __device__ int tr() const { return ((const __attribute__((address_space(4))) int*)(uintptr_t)list)[tr_]; }
+    __device__ TileListIter(const GemmOperands& g, int BM, int BN, int bid_, int G_)
+        : GridIter(listed(g, BM, BN), BM, BN, bid_, G_), list(g.tile_list) {}
+    __device__ int entry() const { return ((const __attribute__((address_space(4))) int*)(uintptr_t)list)[tc_]; }
+    __device__ int tr() const { return entry() >> 16; }
+    __device__ int tc() const { return entry() & 0xffff; }
 };
 
 // The generic persistent kernel.  `Iter` walks the tiles of this workgroup (see GridIter).  `Epi` supplies
@@ -729,9 +733,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     const int nk = g.K / Cfg::BK;
     AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane, (g.layout & kRowsPermuted) != 0);
     Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
-    // a walk over listed rows usually has no job at all: leave before the epilogue's set-up (other walks go on, their
+    // a walk over listed tiles usually has no job at all: leave before the epilogue's set-up (other walks go on, their
     // epilogues may have something to write for a workgroup without work)
-    if constexpr (std::is_same<Iter, ListGridIter>::value) { if (!cur.valid()) return; }
+    if constexpr (std::is_same<Iter, TileListIter>::value) { if (!cur.valid()) return; }
 
     // `pre` walks the (job, k-step) sequence of this workgroup ahead of the MFMAs; `ahead` counts the
     // k-steps whose operand loads have been issued and not yet consumed (at most one per slot).

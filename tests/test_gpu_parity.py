@@ -415,8 +415,11 @@ def test_fused_lmhead_ce_gradient_saturates(amd, oracle, grad_scale):
 def _codes_case(oracle, M, K, V, seed, n_predict, prefix, below_window):
     x, w, t, sc, mtp, pt, pw = _fused_case(oracle, M, K, V, seed=seed, n_predict=n_predict, prefix=prefix)
     if below_window:
-        # some vocabulary rows far below zero for the first tokens: sigma under the 255 codes' range (logits < -13)
-        w[:64] = -w[64:128].abs() * 3
+        # some vocabulary rows far below zero for the first tokens: sigma under the 255 codes' range (logits < -13);
+        # a negative count puts them into the last (ragged) vocabulary tile instead of the first
+        cold = slice(0, 64) if below_window > 0 else slice(V - 64, V)
+        below_window = abs(below_window)
+        w[cold] = -w[64:128].abs() * 3
         x[:below_window] = x[:below_window].abs().clamp(max=2.0) * 2
     ptd = dev(pt) if pt is not None else torch.full((M,), -1, dtype=torch.int64, device="cuda")
     pwd = dev(pw) if pw is not None else torch.zeros(1, device="cuda")
@@ -427,10 +430,11 @@ def _codes_case(oracle, M, K, V, seed, n_predict, prefix, below_window):
     (256, 128, 512, 1, False, False, 0, 1.0),        # one tile
     (640, 256, 2432, 1, False, False, 0, 1.0),       # ragged token and vocabulary tiles (rows / columns of clamped duplicates)
     (384, 768, 5120, 3, True, True, 0, 1.0),         # multi-token prediction + prefix targets, (in, out) weight
-    (1024, 256, 2048, 1, False, False, 300, 1.0),    # sigmas below the code window in two of four token tiles: those are recomputed
+    (1024, 256, 2048, 1, False, False, 300, 1.0),    # sigmas below the code window in two of four token tiles, first vocabulary tile: those two tiles are recomputed
     (1024, 256, 2048, 2, True, True, 1024, 1.0),     # ... in every token tile
     (1024, 256, 2048, 1, False, False, 300, 0.01),   # ... with row factors so small that those gradients are exact zeros: nothing is recomputed
     (1024, 256, 2048, 1, False, False, 300, 0.5),    # ... around the limit between the two (some rows on either side)
+    (640, 256, 2432, 1, False, False, -640, 16.0),    # ... in the last, half-filled vocabulary tile of every token tile, the last one ragged
 ])
 def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, prefix, in_out, below_window, grad_scale):
     """The backward that rebuilds the e5m2 gradient from the forward's sigma codes gives bit for bit what the
@@ -447,7 +451,7 @@ def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, pr
     # code panel: blocks [token tile][vocabulary / 128] of 256 tokens x 128 bytes; count zero codes inside the matrix
     blocks = codes.view(-(-M // 256), -(-V // 256) * 2, 256, 128)[:, : V // 128]
     valid = blocks.permute(0, 2, 1, 3).reshape(-1, V)[:M]
-    assert bool((valid == 0).any()) == (below_window > 0)
+    assert bool((valid == 0).any()) == (below_window != 0)
     bwd = (x_f8, w_f8, dev(t), dev(mtp), ptd, pwd, lse1, sig1)
     tail = (sc["x_s"], sc["w_s"], sc["grad_s"], grad_scale, 23.0, 5.0, 7.5, in_out)
     dx0, dw0 = torch.ops.nanogpt.lmhead_ce_bwd(*bwd, *tail)
@@ -460,8 +464,8 @@ def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, pr
         rowf = grad_scale * (23.0 / 7.5) / sc["grad_s"] * float(mtp.sum()) * torch.exp(23.0 - lse1[rows0])
         if grad_scale == 0.01:
             assert (rowf < 1100).all()        # nothing is recomputed
-        if grad_scale == 1.0:
-            assert (rowf > 1200).any()        # some token tile is
+        if grad_scale >= 1.0:
+            assert (rowf > 1200).any()        # some tile is
     assert torch.equal(dx0, dx1) and torch.equal(dw0, dw1)
 
 
