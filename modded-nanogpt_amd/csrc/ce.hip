@@ -823,13 +823,47 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
 // a row whose factor is larger than that puts the 256 x 256 tile it lies in on the list of tiles (each tile once:
 // flags) that EpiDlStore then recomputes from the logits.  Such entries cluster in vocabulary columns (tokens
 // that never occur as targets keep being pushed down), so the list stays a small part of the matrix.
+// Some code of the word is 0 (a sigma below the window) in a row whose factor is too large for that to mean an exact zero.
+__device__ __forceinline__ bool code_needs_logit(uint32_t w, float rf, float d_below) {
+    return (((w - 0x01010101u) & ~w & 0x80808080u) != 0u) && !(fabsf(rf) * d_below < 0x1p-17f);
+}
+
+// Looks at every `stride`-th 256 x 256 tile of the pass's codes and counts those that the conversion would put on the
+// list.  If more than a given share of the sample is, the conversion below is skipped and the whole panel recomputed
+// from the logits (CondGridIter): conversion plus the recompute of that many tiles would cost more than the recompute
+// alone.  A step with codes then never costs much more than one without.
+__global__ __launch_bounds__(256) void ce_codes_probe_kernel(const uint8_t* __restrict__ codes, int nkp, int m0, int M, int nbx, int nvt, int ntiles,
+                                                            int stride, const float* __restrict__ rowf, const float* __restrict__ dcode,
+                                                            int* __restrict__ hits) {
+    const int idx = blockIdx.x * stride, tid = threadIdx.x;
+    if (idx >= ntiles) return;
+    const int vt = idx % nvt, tt = idx / nvt;
+    const float d_below = dcode[256];
+    const int tok0 = m0 + tt * 256;
+    bool below = false;
+    for (int kv = 2 * vt; kv < 2 * vt + 2 && kv < nbx; ++kv) {
+        const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes;    // 256 tokens x 128 codes
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = tid + 256 * j, r = i >> 3, ch = i & 7;
+            const v4i c = *(const v4i*)(src + r * 128 + ch * 16);
+            const float rf = rowf[tok0 + r];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) below |= (tok0 + r < M) && code_needs_logit((uint32_t)c[k], rf, d_below);
+        }
+    }
+    if (__syncthreads_or(below) && tid == 0) atomicAdd(hits, 1);
+}
+
 __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __restrict__ codes, int nkp, int m0, int M,
                                                              const float* __restrict__ rowf, const float* __restrict__ dcode,
                                                              int nkt, uint8_t* __restrict__ dl_panel, int nvt, int* __restrict__ flags,
-                                                             int* __restrict__ list, int* __restrict__ count) {
+                                                             int* __restrict__ list, int* __restrict__ count,
+                                                             const int* __restrict__ probe_hits, int probe_limit) {
     constexpr int kStride = 33;
     __shared__ uint32_t tile[128 * kStride];
     __shared__ float dtab[256];
+    if (*probe_hits > probe_limit) return;      // the whole panel is recomputed instead (see ce_codes_probe_kernel)
     const int kv = blockIdx.x, a = blockIdx.y, tid = threadIdx.x;
     dtab[tid] = dcode[tid];
     const float d_below = dcode[256];
@@ -846,7 +880,7 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const uint32_t w = (uint32_t)c[k];
-            below |= (tok0 + r < M) && (((w - 0x01010101u) & ~w & 0x80808080u) != 0u) && !(fabsf(rf) * d_below < 0x1p-17f);
+            below |= (tok0 + r < M) && code_needs_logit(w, rf, d_below);
             word_at(r, ch * 4 + k) = f32x4_to_e5m2_sat<true>(rf * dtab[w & 0xffu], rf * dtab[(w >> 8) & 0xffu],
                                                              rf * dtab[(w >> 16) & 0xffu], rf * dtab[w >> 24]);
         }
@@ -1170,8 +1204,8 @@ extern "C" int ngpt_lmhead_ce_fwd_static(const void* x_bf16, const void* w_bf16,
 static int64_t bwd_part_bytes(int64_t Mc, int64_t Mt, int K, int V) {
     return std::max(balanced_part_bytes((int)Mc, K, V), std::max(balanced_part_bytes(V, K, (int)Mt), balanced_part_bytes(K, V, (int)Mt)));
 }
-// codes backward: count | flags [tiles] | list [tiles] of the 256 x 256 tiles of one pass's logits
-static int64_t flag_bytes(int64_t Mt, int64_t Vp) { return align_up((1 + 2 * (Mt / 256) * (Vp / 256)) * 4, 256); }
+// codes backward: count | probe hits | flags [tiles] | list [tiles] of the 256 x 256 tiles of one pass's logits
+static int64_t flag_bytes(int64_t Mt, int64_t Vp) { return align_up((2 + 2 * (Mt / 256) * (Vp / 256)) * 4, 256); }
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
     int64_t Mc = bwd_chunk_rows(M), Mt = round256(Mc), Kp = round256(K), Vp = round256(V);
@@ -1219,7 +1253,8 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
     float* parts = (float*)ws;
     ws += bwd_part_bytes(Mc_max, Mt_max, K, V);
     int* count = (int*)ws;                   // number of listed tiles
-    int* flags = count + 1;                  // per 256 x 256 tile of the pass's logits: a sigma of it lies below the code window and matters
+    int* hits = count + 1;                   // sampled code blocks that would list a tile
+    int* flags = count + 2;                  // per 256 x 256 tile of the pass's logits: a sigma of it lies below the code window and matters
     int* list = flags + (Mt_max / 256) * (Vp / 256);
     static_assert(BWD_CHUNK_ROWS / 256 < 65536, "a list entry holds the token tile in its upper 16 bits");
     if (Vp / 256 >= 65536) return fail(NGPT_ERANGE, "%s: V=%d", who, V);
@@ -1256,14 +1291,22 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
             // 1'. the pass's dlogits panel from the forward's sigma codes; tiles with a sigma below the code window
             //     that matters (none, normally) are then redone from the logits
             ProfileScope prof(PROF_CE_DLOGITS, st);
-            const int nvt = (int)(Vp / 256), nflags = 1 + (Mt / 256) * nvt;
+            const int nvt = (int)(Vp / 256), nflags = 2 + (Mt / 256) * nvt;
             fill_f32_kernel<<<(nflags + 255) / 256, 256, 0, st>>>((float*)count, nflags, 0.0f);
-            ce_codes_to_dl_kernel<<<dim3(V / 128, nkt), 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, rowf, dcode,
-                                                                      nkt, dw_panel, nvt, flags, list, count);
+            // a sample of the tiles decides between the two ways (stride coprime to the tiles per row, so that the
+            // sample covers all vocabulary columns); the recompute of 45 % of the tiles costs what the conversion does
+            const int nbx = V / 128, ntiles = (Mt / 256) * nvt, stride = ntiles >= 64 * 61 ? 61 : 1, nsample = (ntiles + stride - 1) / stride;
+            const int limit = nsample * 45 / 100;
+            ce_codes_probe_kernel<<<nsample, 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, nbx, nvt, ntiles, stride, rowf, dcode, hits);
+            ce_codes_to_dl_kernel<<<dim3(nbx, nkt), 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, rowf, dcode,
+                                                                  nkt, dw_panel, nvt, flags, list, count, hits, limit);
             if (int e = check_launch("ce_codes_to_dl_kernel")) return e;
             g.tile_list = list;
             g.tile_count = count;
+            g.probe_hits = hits;
+            g.probe_limit = limit;
             if (int e = launch_grid_kernel<MainCfg, TileListIter>(g, epi, st, -1, "lm_head CE backward (dlogits of the listed tiles)")) return e;
+            if (int e = launch_grid_kernel<MainCfg, CondGridIter>(g, epi, st, -1, "lm_head CE backward (dlogits, all tiles)")) return e;
         } else if (int e = launch_grid_kernel<MainCfg, GridIter>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
         ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, nkt, dw_panel);

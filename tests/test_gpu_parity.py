@@ -418,8 +418,11 @@ def _codes_case(oracle, M, K, V, seed, n_predict, prefix, below_window):
         # some vocabulary rows far below zero for the first tokens: sigma under the 255 codes' range (logits < -13);
         # a negative count puts them into the last (ragged) vocabulary tile instead of the first
         cold = slice(0, 64) if below_window > 0 else slice(V - 64, V)
+        if below_window >= 10 ** 6:      # ... every vocabulary row
+            cold, below_window = slice(0, V), below_window - 10 ** 6
+            w[64:128] = w[64:128].abs().clamp(min=0.02)
         below_window = abs(below_window)
-        w[cold] = -w[64:128].abs() * 3
+        w[cold] = -w[64:128].abs().repeat(-(-V // 64), 1)[: cold.stop - cold.start] * 3
         x[:below_window] = x[:below_window].abs().clamp(max=2.0) * 2
     ptd = dev(pt) if pt is not None else torch.full((M,), -1, dtype=torch.int64, device="cuda")
     pwd = dev(pw) if pw is not None else torch.zeros(1, device="cuda")
@@ -435,6 +438,8 @@ def _codes_case(oracle, M, K, V, seed, n_predict, prefix, below_window):
     (1024, 256, 2048, 1, False, False, 300, 0.01),   # ... with row factors so small that those gradients are exact zeros: nothing is recomputed
     (1024, 256, 2048, 1, False, False, 300, 0.5),    # ... around the limit between the two (some rows on either side)
     (640, 256, 2432, 1, False, False, -640, 16.0),    # ... in the last, half-filled vocabulary tile of every token tile, the last one ragged
+    (1024, 256, 2048, 1, False, False, 10 ** 6 + 512, 1.0),   # ... in every vocabulary tile of half of the token tiles: the sample of
+                                                              # the codes finds too many, the whole panel is recomputed instead
 ])
 def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, prefix, in_out, below_window, grad_scale):
     """The backward that rebuilds the e5m2 gradient from the forward's sigma codes gives bit for bit what the
