@@ -1295,7 +1295,7 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
             fill_f32_kernel<<<(nflags + 255) / 256, 256, 0, st>>>((float*)count, nflags, 0.0f);
             // a sample of the tiles decides between the two ways (stride coprime to the tiles per row, so that the
             // sample covers all vocabulary columns); the recompute of 45 % of the tiles costs what the conversion does
-            const int nbx = V / 128, ntiles = (Mt / 256) * nvt, stride = ntiles >= 64 * 61 ? 61 : 1, nsample = (ntiles + stride - 1) / stride;
+            const int nbx = V / 128, ntiles = (Mt / 256) * nvt, stride = ntiles >= 64 * 127 ? 127 : 1, nsample = (ntiles + stride - 1) / stride;
             const int limit = nsample * 45 / 100;
             ce_codes_probe_kernel<<<nsample, 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, nbx, nvt, ntiles, stride, rowf, dcode, hits);
             ce_codes_to_dl_kernel<<<dim3(nbx, nkt), 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, rowf, dcode,
