@@ -825,7 +825,7 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
 // that never occur as targets keep being pushed down), so the list stays a small part of the matrix.
 // Some code of the word is 0 (a sigma below the window) in a row whose factor is too large for that to mean an exact zero.
 __device__ __forceinline__ bool code_needs_logit(uint32_t w, float rf, float d_below) {
-    return (((w - 0x01010101u) & ~w & 0x80808080u) != 0u) && !(fabsf(rf) * d_below < 0x1p-17f);
+    return (((w - 0x01010101u) & ~w & 0x80808080u) != 0u) & !(fabsf(rf) * d_below < 0x1p-17f);
 }
 
 // Looks at every `stride`-th 256 x 256 tile of the pass's codes and counts those that the conversion would put on the
@@ -840,17 +840,26 @@ __global__ __launch_bounds__(256) void ce_codes_probe_kernel(const uint8_t* __re
     const int vt = idx % nvt, tt = idx / nvt;
     const float d_below = dcode[256];
     const int tok0 = m0 + tt * 256;
-    bool below = false;
-    for (int kv = 2 * vt; kv < 2 * vt + 2 && kv < nbx; ++kv) {
+    // all loads first (branch-free), then the tests: the kernel is a handful of round trips to memory long
+    v4i c[2][8];
+    float rf[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) rf[j] = rowf[tok0 + ((tid + 256 * j) >> 3)];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int kv = min(2 * vt + q, nbx - 1);     // the last tile of an odd count holds one block: read it twice
         const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes;    // 256 tokens x 128 codes
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int i = tid + 256 * j, r = i >> 3, ch = i & 7;
-            const v4i c = *(const v4i*)(src + r * 128 + ch * 16);
-            const float rf = rowf[tok0 + r];
+        for (int j = 0; j < 8; ++j) c[q][j] = *(const v4i*)(src + (tid + 256 * j) * 16);
+    }
+    bool below = false;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) below |= (tok0 + r < M) && code_needs_logit((uint32_t)c[k], rf, d_below);
-        }
+    for (int j = 0; j < 8; ++j) {
+        const bool inside = tok0 + ((tid + 256 * j) >> 3) < M;
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) below |= inside & code_needs_logit((uint32_t)c[q][j][k], rf[j], d_below);
     }
     if (__syncthreads_or(below) && tid == 0) atomicAdd(hits, 1);
 }
