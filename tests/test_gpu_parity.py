@@ -244,6 +244,38 @@ def test_fc_relu2_forward(amd, oracle, M, D, H):
     assert_close_gemm(out, out_ref)
 
 
+def test_operand_loads_by_half_of_the_waves(amd):
+    """TileCfg::LOADERS: the kernel in which the first four waves of a workgroup issue every operand load (and the other
+    four wait on the barrier only) computes the same tile.  It exists in the measurement build, where the upper four
+    waves store their half of the FP8 c_fc output: that half equals the shipped kernel's bit for bit, the rest stays
+    untouched."""
+    lib = amd._lib.load_bench()
+    M, D, H = 1024, 768, 3072
+    torch.manual_seed(5)
+    x8 = torch.randn(M, D, device="cuda").to(torch.float8_e4m3fn)
+    w8 = (torch.randn(H, D, device="cuda") * 0.05).to(torch.float8_e4m3fn)
+    deq = torch.tensor([0.37], device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    outs = {}
+    try:
+        for mode in (0, 1, 2):      # shipped kernel; half stored, all waves load; half stored, four waves load
+            assert lib.ngpt_tuning_set(5, mode) == 0
+            post = torch.full((M, H), -1.0, dtype=torch.bfloat16, device="cuda")
+            rc = lib.ngpt_fc_relu2_fwd(x8.data_ptr(), w8.data_ptr(), deq.data_ptr(), M, H, D, post.data_ptr(), None, None, None, 0, st)
+            assert rc == 0, lib.ngpt_last_error()
+            torch.cuda.synchronize()
+            outs[mode] = post
+    finally:
+        lib.ngpt_tuning_set(5, 0)
+    ref = outs[0]
+    assert (ref >= 0).all()
+    for mode in (1, 2):
+        written = outs[mode] >= 0
+        assert 0.49 < written.float().mean().item() < 0.51
+        assert torch.equal(outs[mode][written], ref[written])
+    assert torch.equal(outs[1] >= 0, outs[2] >= 0)
+
+
 def test_fc_relu2_emit_fp8_and_amax(amd, oracle):
     M, D, H = 1024, 256, 1024
     x, w_fc, w_proj_t = oracle.make_cfg2(seed=8, M=M, D=D, H=H)
