@@ -554,6 +554,33 @@ def workload_ceiling(args, amd, dev) -> int:
             torch.cuda.synchronize()
             samples[m].append(e0.elapsed_time(e1) / 30)
     lib.ngpt_tuning_set(5, 0)
+    # Where the time of the fused CE forward goes, against the plain GEMM of the same shape: cycles of workgroup 0's waves
+    # inside the epilogue calls and outside them (per tile and per k-step), from the kernels' own cycle counters.
+    res["phase_rows"] = []
+    x, w, t, sc = make_cfg3(seed=0)
+    xd, wd, td = x.to(dev), w.to(dev), t.to(dev)
+    mtp = torch.tensor([1.0], device=dev)
+    pt = torch.full((x.shape[0],), -1, dtype=torch.int64, device=dev)
+    pw = torch.zeros(1, device=dev)
+    fwd_args = (xd, wd, td, mtp, pt, pw, sc["x_s"], sc["w_s"], sc["A"], sc["B"], sc["C"], False)
+    product_lib, amd._lib._lib = amd._lib._lib, lib          # the operators call through the measurement build here
+    try:
+        for what, op in (("fused CE forward writing sigma codes", torch.ops.nanogpt.lmhead_ce_fwd_codes), ("fused CE forward", torch.ops.nanogpt.lmhead_ce_fwd)):
+            for _ in range(3):
+                op(*fwd_args)
+            buf = (ctypes.c_longlong * 64)()
+            assert lib.ngpt_bench_ce_phase_ticks(buf) == 0, lib.ngpt_last_error()
+            res["phase_rows"].append({"what": what, "ticks": list(buf[:32])})
+    finally:
+        amd._lib._lib = product_lib
+    a = torch.randint(0, 120, (R, 768), dtype=torch.uint8, device=dev).view(E4)
+    b = torch.randint(0, 120, (C, 768), dtype=torch.uint8, device=dev).view(E4)
+    out = torch.zeros(16, device=dev)
+    for _ in range(3):
+        assert lib.ngpt_gemm_fp8_tn(a.data_ptr(), 0, 768, b.data_ptr(), 0, 768, R, C, 768, 1.0, out.data_ptr(), C, 3, st) == 0, lib.ngpt_last_error()
+    buf = (ctypes.c_longlong * 64)()
+    assert lib.ngpt_bench_gemm_phase_ticks(buf) == 0, lib.ngpt_last_error()
+    res["phase_rows"].append({"what": f"plain GEMM {R} x {C} x 768, result discarded", "ticks": list(buf[:32])})
     res["store_rows"] = [{"what": f"FP8 c_fc {Mm} x {Nn} x {Kk}, {what}", "ms": statistics.median(samples[m]), "ms_min": min(samples[m])}
                          for m, what in modes]
     print(json.dumps(res))

@@ -73,6 +73,15 @@ int ngpt_tuning_set(int key, int value);
  * bytes apart; sink: 512 floats; ticks [grid][2] int64 = shader-clock cycles and 100 MHz wall ticks per workgroup. */
 int ngpt_bench_kstep_rate(const void* src, int64_t src_stride, int mode, int iters, int grid, float* sink,
                           long long* ticks, void* stream);
+
+/* Where the time of a GEMM-shaped kernel goes: every such kernel of the measurement build counts shader-clock
+ * cycles in its workgroup 0, per wave w < 16: out64[4 w + 0] whole kernel, [4 w + 1] inside the epilogue calls of
+ * its tiles, [4 w + 2] number of tiles, [4 w + 3] from leaving an epilogue to passing the barrier of the next tile's
+ * first k-step (three quarters of that k-step's MFMAs plus the wait for slower waves).  These two calls wait for the
+ * device and return the counts of the last launch: _ce_ of the fused lm_head + CE kernels (forward, dlogits
+ * recompute), _gemm_ of every other GEMM of the library.  out64: 64 int64 in host memory. */
+int ngpt_bench_ce_phase_ticks(long long* out64);
+int ngpt_bench_gemm_phase_ticks(long long* out64);
 #endif
 
 /* ---- quantisers ---------------------------------------------------------------------------

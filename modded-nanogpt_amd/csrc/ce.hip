@@ -1352,6 +1352,17 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
                               w_layout, workspace, workspace_bytes, stream);
 }
 
+#ifdef NGPT_BENCH_BUILD
+// Measurement build: cycle counts of the last GEMM-shaped kernel launched from this file (g_phase_ticks in gemm_tn.h:
+// 16 waves x 4 numbers of workgroup 0), after a device synchronisation.
+extern "C" int ngpt_bench_ce_phase_ticks(long long* out64) {
+    if (!out64) return fail(NGPT_EINVAL, "ngpt_bench_ce_phase_ticks: null pointer");
+    if (hipDeviceSynchronize() != hipSuccess) return fail(NGPT_EINVAL, "ngpt_bench_ce_phase_ticks: device error");
+    if (hipMemcpyFromSymbol(out64, HIP_SYMBOL(g_phase_ticks), 64 * sizeof(long long)) != hipSuccess) return fail(NGPT_EINVAL, "ngpt_bench_ce_phase_ticks: copy failed");
+    return NGPT_OK;
+}
+#endif
+
 extern "C" int ngpt_lmhead_ce_fwd_codes(const void* x_bf16, const void* w_bf16, const int64_t* targets,
                                         const float* mtp_weights, int n_predict,
                                         const int64_t* prefix_targets, const float* prefix_weight,

@@ -250,6 +250,17 @@ extern "C" const char* ngpt_last_error(void) { return last_error_buf(); }
 extern "C" int ngpt_num_cus(void) { return num_cus(); }
 
 #ifdef NGPT_BENCH_BUILD
+// Measurement build: cycle counts of the last GEMM-shaped kernel launched from this file (g_phase_ticks in gemm_tn.h:
+// 16 waves x 4 numbers of workgroup 0), after a device synchronisation.
+extern "C" int ngpt_bench_gemm_phase_ticks(long long* out64) {
+    if (!out64) return fail(NGPT_EINVAL, "ngpt_bench_gemm_phase_ticks: null pointer");
+    if (hipDeviceSynchronize() != hipSuccess) return fail(NGPT_EINVAL, "ngpt_bench_gemm_phase_ticks: device error");
+    if (hipMemcpyFromSymbol(out64, HIP_SYMBOL(g_phase_ticks), 64 * sizeof(long long)) != hipSuccess) return fail(NGPT_EINVAL, "ngpt_bench_gemm_phase_ticks: copy failed");
+    return NGPT_OK;
+}
+#endif
+
+#ifdef NGPT_BENCH_BUILD
 extern "C" int ngpt_tuning_set(int key, int value) {
     if (key < 0 || key >= 8) return fail(NGPT_EINVAL, "ngpt_tuning_set: key=%d", key);
     g_tuning[key] = value;

@@ -736,6 +736,14 @@ struct EpiDropsFragments : std::false_type {};
 template <class E>
 struct EpiDropsFragments<E, std::void_t<decltype(E::DROPS_FRAGMENTS)>> : std::bool_constant<E::DROPS_FRAGMENTS> {};
 
+#ifdef NGPT_BENCH_BUILD
+// Measurement build: shader-clock cycles that wave w (< 16) of workgroup 0 spent in the last launch of a kernel of this
+// translation unit: [4 w + 0] whole kernel, [4 w + 1] inside the epilogue calls of its tiles, [4 w + 2] number of tiles,
+// [4 w + 3] between leaving an epilogue and passing the barrier of the next tile's first k-step (three quarters of that
+// k-step's MFMAs plus the wait for the slower waves).
+static __device__ long long g_phase_ticks[64];
+#endif
+
 template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(GemmOperands g, Epi epi) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_all[];
@@ -745,6 +753,10 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     const int ablate = EpiAblatable<Epi>::value ? __builtin_amdgcn_readfirstlane(g.ablate) : 0;
     TileMainloop<Cfg, AFMT, BFMT> ml;
     ml.init();
+#ifdef NGPT_BENCH_BUILD
+    const long long tick_start = clock64();
+    long long tick_epi = 0, tick_tiles = 0, tick_wait = 0, tick_left = 0;
+#endif
     const int bid = blockIdx.x, G = gridDim.x;
     const int nk = g.K / Cfg::BK;
     AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane, (g.layout & kRowsPermuted) != 0);
@@ -819,6 +831,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
                 else if (decltype(first)::value && EpiTileStores<Epi>::value > 0 && relaxed) wait_vmem_le<EpiTileStores<Epi>::value>();
                 else wait_vmem_le<0>();
                 if (!(ablate & 4)) wg_barrier();
+#ifdef NGPT_BENCH_BUILD
+                if (decltype(first)::value && tick_left) { tick_wait += clock64() - tick_left; tick_left = 0; }
+#endif
             };
             auto refill_here = [&]() {
                 if (!(last_kt && keep_slot)) refill(slot);
@@ -848,9 +863,17 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{}, false, kt + 1 == kt1);
         // every wave passed the last k-step's barrier after its final read of slot ^ 1
         uint8_t* free_stage = smem + (slot ^ 1) * Cfg::STAGE_BYTES;
+#ifdef NGPT_BENCH_BUILD
+        const long long tick_e0 = clock64();
+#endif
         epi.partial(cur.partial(), cur.part_slot());
         epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
         if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
+#ifdef NGPT_BENCH_BUILD
+        tick_left = clock64();
+        tick_epi += tick_left - tick_e0;
+        ++tick_tiles;
+#endif
         if (keep_slot) {
             wg_barrier();          // all waves are done with the scratch
             refill(slot ^ 1);
@@ -861,6 +884,14 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     }
     wg_barrier();
     epi.end(smem, bid, G);
+#ifdef NGPT_BENCH_BUILD
+    if (bid == 0 && ml.lane == 0 && ml.wave < 16) {
+        g_phase_ticks[4 * ml.wave + 0] = clock64() - tick_start;
+        g_phase_ticks[4 * ml.wave + 1] = tick_epi;
+        g_phase_ticks[4 * ml.wave + 2] = tick_tiles;
+        g_phase_ticks[4 * ml.wave + 3] = tick_wait;
+    }
+#endif
 }
 
 }  // namespace ngpt
