@@ -62,7 +62,10 @@ int ngpt_profile_read(int slot, double* total_ms, int* launches);
  * (libngpt_fp8_bench.so, compiled with -DNGPT_BENCH_BUILD), never in libngpt_fp8.so.  key 2: ablation bits
  * for timing runs of ngpt_gemm_fp8_tn with out_kind 3 (1 = no operand loads, 2 = no MFMAs, 4 = no k-loop
  * barrier; results are then meaningless); key 4: split-K factor used by ngpt_gemm_fp8_tn with out_kind 2;
- * key 7: 1 = accept operand row strides below K (overlapping rows keep the operands cache resident in
+ * key 5: ngpt_fc_relu2_fwd (whole-line path) stores only the upper four waves' half of the output (1), does so with
+ * the lower four waves issuing every operand load (2), skips the epilogue (3), or both (4); key 6: 1 =
+ * ngpt_lmhead_ce_fwd_codes writes every tile's codes over the same two blocks of the panel (stores that stay in the
+ * L2); key 7: 1 = accept operand row strides below K (overlapping rows keep the operands cache resident in
  * timing runs).  Process-global and not synchronised: one thread, set before the timed calls. */
 int ngpt_tuning_set(int key, int value);
 

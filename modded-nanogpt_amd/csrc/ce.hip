@@ -478,6 +478,9 @@ struct EpiCEFwdT {
     int ncand;            // n_predict (+1 with prefix targets)
     int* cand;            // LDS: [MAX_CAND][CE_MAX_BN] valid target column of the job's tokens, else -1
     float sum[8];
+#ifdef NGPT_BENCH_BUILD
+    int bench_alias;      // timing aid (tuning key 6): 1 = every tile writes its codes over the panel's first blocks (they stay in L2)
+#endif
 
     __device__ void partial(bool, int) {}
     __device__ void begin(int, int, uint8_t* extra) {
@@ -515,6 +518,9 @@ struct EpiCEFwdT {
         if constexpr (CODES) {
             const int wr = co.wave_row0 >> 6, wc = co.wave_col0 >> 7;
             cd_base = codes + ((int64_t)(c0 >> 8) * nkp + (r0 >> 7) + (wr >> 1)) * kPanelBytes;
+#ifdef NGPT_BENCH_BUILD
+            if (bench_alias == 1) cd_base = codes + (wr >> 1) * kPanelBytes;
+#endif
             cd_lane = (uint32_t)((128 * wc + (lane & 31)) * 128 + 64 * (wr & 1) + 16 * (lane >> 5));
         }
         auto code_store = [&](int tm, int tn, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
@@ -1008,7 +1014,13 @@ static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwdT<CODES>& epi, hip
     if (mg < 1) mg = 1;
     {
         ProfileScope prof(PROF_CE_FWD, st);
+#ifdef NGPT_BENCH_BUILD
+        EpiCEFwdT<CODES> timed = epi;
+        timed.bench_alias = g_tuning[6];
+        kernel<<<CE_XCDS * CE_SPLITS * mg, Cfg::THREADS, LDS, st>>>(g, timed);
+#else
         kernel<<<CE_XCDS * CE_SPLITS * mg, Cfg::THREADS, LDS, st>>>(g, epi);
+#endif
     }
     return check_launch("lm_head CE forward");
 }

@@ -16,7 +16,8 @@ using SmallCfg = TileCfg<128, 128, 2, 2, 128, 2, 2>;
 
 #ifdef NGPT_BENCH_BUILD
 // Measurement build only.  Tuning keys: [2] ablation bits (honoured by the discarding epilogue only),
-// [4] split-K factor of ngpt_gemm_fp8_tn,
+// [4] split-K factor of ngpt_gemm_fp8_tn, [5] FP8 c_fc with part of its epilogue / of its loading waves left out (gemm_api.hip),
+// [6] 1 = the code-writing CE forward stores every tile's codes over the same blocks (ce.hip),
 // [7] 1 = accept operand row strides below K (overlapping rows keep the operands cache resident)
 extern int g_tuning[8];
 #endif
