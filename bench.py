@@ -585,6 +585,51 @@ def workload_ceiling(args, amd, dev) -> int:
     buf = (ctypes.c_longlong * 64)()
     assert lib.ngpt_bench_gemm_phase_ticks(buf) == 0, lib.ngpt_last_error()
     res["phase_rows"].append({"what": f"plain GEMM {R} x {C} x 768, result discarded", "ticks": list(buf[:32])})
+    # Issue rates behind the epilogue designs: single vector instructions with 1, 2 and 4 waves per SIMD, and 64-lane LDS
+    # gathers with the address patterns of the softcap table (6656 entries)
+    names = ["v_mul_f32", "v_add_f32", "v_and_b32", "v_lshrrev_b32", "v_max_f32", "v_fma_f32", "v_perm_b32", "v_and_or_b32", "v_cvt_pk_bf16_f32",
+             "v_pk_sub_u16 clamp", "v_pk_min_u16", "v_pk_lshlrev_b16", "v_mov_b32_dpp", "v_exp_f32"]
+    vsink = torch.zeros(1024, dtype=torch.int32, device=dev)
+    vticks = torch.zeros(16, dtype=torch.int64, device=dev)
+    res["valu_rows"] = []
+    n_it = 2000
+    for kind, name in enumerate(names):
+        row = {"instruction": name}
+        for threads in (256, 512, 1024):
+            for _ in range(2):
+                assert lib.ngpt_bench_valu_rate(kind, threads, n_it, vsink.data_ptr(), vticks.data_ptr(), st) == 0, lib.ngpt_last_error()
+            torch.cuda.synchronize()
+            waves = threads // 64
+            t = vticks[:waves].double()
+            # one wave per SIMD: cycles per instruction of a wave; more: the slowest wave's cycles per instruction, per wave of the SIMD
+            row[f"waves_per_simd_{waves // 4}"] = float(t.max()) / (n_it * 32) / (waves // 4)
+        res["valu_rows"].append(row)
+    res["lds_rows"] = []
+    TABN = 6656
+    gen = torch.Generator().manual_seed(1)
+    def table_index(l):       # the fused CE's table index of a logit (sign bit | clamped bf16 magnitude)
+        bits = l.bfloat16().view(torch.int16).to(torch.int32) & 0xffff
+        t_ = ((bits & 0x7fff) - 0x3980).clamp(0, 2559)
+        return t_ + (bits >> 15) * 4096
+    n_off = cus * 512 * 16
+    lane = (torch.arange(n_off) // 16) % 64
+    kk = torch.arange(n_off) % 16
+    patterns = (("consecutive lanes, consecutive entries (no bank conflict)", lane + 64 * kk),
+                ("one entry for all lanes (broadcast)", torch.full((n_off,), 17)),
+                ("uniformly random entries", torch.randint(0, TABN, (n_off,), generator=gen)),
+                ("table entries of N(0, 1) logits", table_index(torch.randn(n_off, generator=gen))),
+                ("table entries of N(0, 3) logits", table_index(torch.randn(n_off, generator=gen) * 3)))
+    gsink = torch.zeros(512, device=dev)
+    for what, idx in patterns:
+        offs = (idx.to(torch.int32) * 4).to(dev)
+        row = {"pattern": what}
+        for threads in (256, 512):
+            for _ in range(2):
+                assert lib.ngpt_bench_lds_gather(offs.data_ptr(), TABN, threads, n_it, gsink.data_ptr(), vticks.data_ptr(), st) == 0, lib.ngpt_last_error()
+            torch.cuda.synchronize()
+            waves = threads // 64
+            row[f"waves_per_cu_{waves}"] = float(vticks[:waves].double().max()) / (n_it * 16) / waves      # LDS cycles per gather and compute unit
+        res["lds_rows"].append(row)
     res["store_rows"] = [{"what": f"FP8 c_fc {Mm} x {Nn} x {Kk}, {what}", "ms": statistics.median(samples[m]), "ms_min": min(samples[m])}
                          for m, what in modes]
     print(json.dumps(res))

@@ -85,6 +85,17 @@ int ngpt_bench_kstep_rate(const void* src, int64_t src_stride, int mode, int ite
  * recompute), _gemm_ of every other GEMM of the library.  out64: 64 int64 in host memory. */
 int ngpt_bench_ce_phase_ticks(long long* out64);
 int ngpt_bench_gemm_phase_ticks(long long* out64);
+
+/* Issue rates of the machine that the epilogue designs lean on.  ngpt_bench_valu_rate: every wave of one workgroup
+ * per compute unit runs iters x 32 vector instructions of one kind (0 v_mul_f32, 1 v_add_f32, 2 v_and_b32,
+ * 3 v_lshrrev_b32, 4 v_max_f32, 5 v_fma_f32, 6 v_perm_b32, 7 v_and_or_b32, 8 v_cvt_pk_bf16_f32, 9 v_pk_sub_u16 clamp,
+ * 10 v_pk_min_u16, 11 v_pk_lshlrev_b16, 12 v_mov_b32_dpp, 13 v_exp_f32) on independent registers; threads = 256, 512
+ * or 1024 per workgroup = 1, 2 or 4 waves per SIMD; ticks (device, 16 int64) receives the shader-clock cycles of each
+ * wave of workgroup 0; sink: 1024 uint32 (device).  ngpt_bench_lds_gather: every wave issues iters x 16 64-lane
+ * ds_read_b32 with the byte offsets offs[(workgroup * threads + thread) * 16 ..+15] (device, below 4 * entries) into a
+ * table of `entries` floats; threads = 256 or 512; ticks: 8 int64; sink: 512 floats. */
+int ngpt_bench_valu_rate(int kind, int threads, int iters, void* sink, long long* ticks, void* stream);
+int ngpt_bench_lds_gather(const void* offs, int entries, int threads, int iters, void* sink, long long* ticks, void* stream);
 #endif
 
 /* ---- quantisers ---------------------------------------------------------------------------

@@ -14,6 +14,8 @@ BENCH_SIGNATURES = {
     "ngpt_bench_kstep_rate": (c_int, [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "ngpt_bench_ce_phase_ticks": (c_int, [c_void_p]),
     "ngpt_bench_gemm_phase_ticks": (c_int, [c_void_p]),
+    "ngpt_bench_valu_rate": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "ngpt_bench_lds_gather": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
 }
 
 E4M3, E5M2 = 0, 1
