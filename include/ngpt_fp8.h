@@ -256,15 +256,24 @@ int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, const float
 
 /* ---- fused lm_head + softcapped cross-entropy ---------------------------------------------
  * FusedSoftcappedCrossEntropy.forward/backward, triton_kernels.py:1208-1292, without the
- * [M, V] logits (or their gradient) ever being stored: the forward keeps per-row softmax
- * statistics from vocabulary tiles, the backward recomputes the logits tile by tile.
+ * [M, V] logits ever being stored: the forward keeps per-row softmax statistics from vocabulary
+ * tiles; the backward rebuilds the e5m2 gradient of the logits -- from recomputed logits
+ * (ngpt_lmhead_ce_bwd) or from one code byte per logit kept by the forward (the _codes pair) --
+ * and does store that gradient, once, in its workspace (M x V bytes) as the operand of dx and dW.
  *
  * Forward: x [M,K] bf16, w bf16 in `w_layout` ([V,K] or [K,V]).  Writes losses [M] fp32 and,
  * saved for backward: lse [M] fp32 (log-sum-exp of the softcapped logits), saved_sigma
  * [(NGPT_MAX_PREDICT + 1) * M] fp32 (the bf16-rounded sigmoid at every candidate target column;
  * entries of invalid targets are left untouched), x_f8 [M,K] and w_f8_vk [V,K] (e4m3, always
- * vocabulary-major).  K % 128 == 0, M % 16 == 0, V % 16 == 0. */
+ * vocabulary-major).  K % 128 == 0, M % 16 == 0, V % 16 == 0.
+ * Two kernels serve the forward.  For V % 64 == 0 and K in {256, 512, 768, 1024} a token-stationary
+ * kernel keeps 128 tokens' activations in LDS and streams the weights from a second, MFMA-fragment
+ * ordered copy that lives in the workspace (V x K bytes); ngpt_lmhead_ce_fwd_workspace_bytes
+ * includes it.  A workspace of only ngpt_lmhead_ce_fwd_min_workspace_bytes (lookup tables and
+ * partial sums) selects the generic tile kernel, as do all other shapes.  Results agree to the
+ * last bits of the sum of exponentials (different summation order); codes and fp8 copies are equal. */
 int64_t ngpt_lmhead_ce_fwd_workspace_bytes(int M, int K, int V, int w_layout);
+int64_t ngpt_lmhead_ce_fwd_min_workspace_bytes(int M, int K, int V, int w_layout);
 int ngpt_lmhead_ce_fwd(const void* x_bf16, const void* w_bf16, const int64_t* targets,
                        const float* mtp_weights, int n_predict,
                        const int64_t* prefix_targets, const float* prefix_weight,

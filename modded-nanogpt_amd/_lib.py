@@ -58,6 +58,7 @@ SIGNATURES = {
     "ngpt_ce_fwd_bwd_workspace_bytes": (_L, []),
     "ngpt_ce_fwd_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _F, _F, _F, _F, _F, _P, _L, _P]),
     "ngpt_lmhead_ce_fwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
+    "ngpt_lmhead_ce_fwd_min_workspace_bytes": (_L, [_I, _I, _I, _I]),
     "ngpt_lmhead_ce_fwd": (_I, [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _F, _F, _F, _F, _F,
                                 _P, _P, _P, _P, _P, _I, _P, _L, _P]),
     "ngpt_lmhead_ce_fwd_static_max_rows": (_I, []),

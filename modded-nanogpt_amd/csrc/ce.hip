@@ -660,6 +660,10 @@ __global__ void ce_finalize_kernel(const float* __restrict__ part, const float* 
     lse_out[m] = lse;
 }
 
+}  // namespace ngpt
+#include "ce_fwd_xs.h"
+namespace ngpt {
+
 // =====================================================================================================
 // Backward, recomputing the logits.  rowf[m] = coef * S_w[m] * exp(A - lse[m]).
 // One 256-thread block per 256 rows (one token tile of the recompute kernel).  rowf is written for the
@@ -1025,6 +1029,38 @@ static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwdT<CODES>& epi, hip
     return check_launch("lm_head CE forward");
 }
 
+// The token-stationary forward (ce_fwd_xs.h) covers V % 64 == 0, K % 256 == 0, K <= XS_MAX_K; other shapes take the tile kernel.
+static bool xs_eligible(int M, int K, int V) { return M > 0 && V % XS_UNIT == 0 && (K == 256 || K == 512 || K == 768 || K == 1024); }
+
+template <bool CODES, int NS>
+static int launch_ce_fwd_xs(XsArgs a, hipStream_t st) {
+    auto kernel = ce_fwd_xs_kernel<CODES, NS>;
+    const int LDS = XS_CAND_LDS + a.K * XS_TOK;      // dynamic part; the table is static LDS
+    static PerDeviceOnce configured;
+    if (int e = configured.run([&] { return allow_lds(kernel, XS_CAND_LDS + XS_MAX_K * XS_TOK); })) return e;
+    const int cus = num_cus();
+    if (cus < CE_XCDS) return fail(NGPT_EINVAL, "lm_head CE forward: no HIP device (or fewer than %d compute units)", CE_XCDS);
+    // workgroups per XCD = token tiles in flight (mg) x vocabulary shares (splits); the split count that needs the
+    // fewest unit-steps per workgroup wins, the smaller one on a tie (longer jobs, fewer slab loads)
+    const int per_xcd_slots = cus / CE_XCDS, tiles_m = (a.M + XS_TOK - 1) / XS_TOK, per_xcd = (tiles_m + CE_XCDS - 1) / CE_XCDS;
+    const int units = a.V / XS_UNIT;
+    int best_splits = 1, best_mg = 1;
+    int64_t best_cost = -1;
+    for (int s = 1; s <= XS_MAX_SPLITS; s *= 2) {
+        if (s > per_xcd_slots || s > units) break;
+        int mg = per_xcd_slots / s;
+        if (mg > per_xcd) mg = per_xcd;
+        const int64_t cost = (int64_t)((per_xcd + mg - 1) / mg) * ((units + s - 1) / s);
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_splits = s; best_mg = mg; }
+    }
+    a.splits = best_splits;
+    {
+        ProfileScope prof(PROF_CE_FWD, st);
+        kernel<<<CE_XCDS * best_splits * best_mg, XS_THREADS, LDS, st>>>(a);
+    }
+    return check_launch("lm_head CE forward (token-stationary)");
+}
+
 template <class Cfg, class Iter, class Epi>
 static int launch_grid_kernel(const GemmOperands& g, const Epi& epi, hipStream_t st, int slot, const char* what) {
     auto kernel = gemm_tn_kernel<Cfg, FMT_E4M3, FMT_E4M3, Epi, Iter>;
@@ -1099,9 +1135,15 @@ extern "C" int64_t ngpt_ce_fwd_bwd_workspace_bytes(void) { return 2 * TAB_BYTES;
 // ------------------------------------------------------------------------------------------------
 // forward workspace: tabE | tabD | part [CE_SPLITS][M] | (IN_OUT only) nothing extra: the transposed
 // quantiser writes w_f8_vk directly.
-extern "C" int64_t ngpt_lmhead_ce_fwd_workspace_bytes(int M, int K, int V, int w_layout) {
+static int64_t fwd_base_workspace_bytes(int M) { return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)CE_SPLITS * M * 4, 256); }
+extern "C" int64_t ngpt_lmhead_ce_fwd_min_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)K; (void)V; (void)w_layout;
-    return align_up(2 * TAB_BYTES, 256) + align_up((int64_t)CE_SPLITS * M * 4, 256);
+    return fwd_base_workspace_bytes(M);
+}
+// ... | fragment-major copy of the weights (token-stationary kernel only)
+extern "C" int64_t ngpt_lmhead_ce_fwd_workspace_bytes(int M, int K, int V, int w_layout) {
+    (void)w_layout;
+    return fwd_base_workspace_bytes(M) + (xs_eligible(M, K, V) ? align_up(xs_frag_bytes(V, K), 256) : 0);
 }
 
 namespace ngpt {
@@ -1120,14 +1162,17 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
     if (K % 128 || M % 16 || V % 16)
         return fail(NGPT_EALIGN, "%s: need K %% 128 == 0, M %% 16 == 0, V %% 16 == 0 (M=%d K=%d V=%d)", who, M, K, V);
     if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "%s: w_layout=%d", who, w_layout);
-    int64_t need = ngpt_lmhead_ce_fwd_workspace_bytes(M, K, V, w_layout);
+    int64_t need = fwd_base_workspace_bytes(M);
     if (workspace_bytes < need)
         return fail(NGPT_EWORKSPACE, "%s: workspace %lld < %lld bytes", who, (long long)workspace_bytes, (long long)need);
+    // the token-stationary kernel needs room for its copy of the weights; a workspace of the minimum size selects the tile kernel
+    const bool use_xs = xs_eligible(M, K, V) && workspace_bytes >= ngpt_lmhead_ce_fwd_workspace_bytes(M, K, V, w_layout);
     hipStream_t st = (hipStream_t)stream;
     uint8_t* ws = (uint8_t*)workspace;
     float* tabE = (float*)ws;
     float* tabD = tabE + TAB_ENTRIES;
     float* part = (float*)(ws + align_up(2 * TAB_BYTES, 256));
+    uint8_t* w_frag = ws + fwd_base_workspace_bytes(M);
 
     Softcap sc = make_softcap(A, B, C);
     ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc, sigma_codes != nullptr);
@@ -1151,7 +1196,31 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
         epi.scale = x_s * w_s;
         epi.ncand = prefix_targets ? n_predict + 1 : n_predict;
     };
-    if (sigma_codes) {
+    if (use_xs) {
+        xs_frag_from_f8_kernel<<<std::min((V / XS_UNIT) * (K / 128), 8 * num_cus()), 256, 0, st>>>((const uint8_t*)w_f8_vk, V, K, w_frag);
+        if (int e = check_launch("xs_frag_from_f8_kernel")) return e;
+        XsArgs a{};
+        a.w_frag = w_frag;
+        a.x_f8 = (const uint8_t*)x_f8;
+        a.M = M; a.V = V; a.K = K;
+        a.codes = (uint8_t*)sigma_codes;
+        a.nkp = (int)(round256(V) / 128);
+        a.gtabE = tabE;
+        a.part = part;
+        a.saved_sigma = saved_sigma;
+        a.ca = ca;
+        a.sc = sc;
+        a.scale = x_s * w_s;
+        a.ncand = prefix_targets ? n_predict + 1 : n_predict;
+        int e = NGPT_EINVAL;
+        switch (K / 64) {   // the contraction loop is unrolled completely: one instantiation per supported K
+            case 4: e = sigma_codes ? launch_ce_fwd_xs<true, 4>(a, st) : launch_ce_fwd_xs<false, 4>(a, st); break;
+            case 8: e = sigma_codes ? launch_ce_fwd_xs<true, 8>(a, st) : launch_ce_fwd_xs<false, 8>(a, st); break;
+            case 12: e = sigma_codes ? launch_ce_fwd_xs<true, 12>(a, st) : launch_ce_fwd_xs<false, 12>(a, st); break;
+            case 16: e = sigma_codes ? launch_ce_fwd_xs<true, 16>(a, st) : launch_ce_fwd_xs<false, 16>(a, st); break;
+        }
+        if (e) return e;
+    } else if (sigma_codes) {
         EpiCEFwdT<true> epi{};
         fill(epi);
         epi.codes = (uint8_t*)sigma_codes;
@@ -1216,7 +1285,7 @@ extern "C" int ngpt_lmhead_ce_fwd_static(const void* x_bf16, const void* w_bf16,
     if (int e = static_scratch(&ws)) return e;
     return lmhead_ce_fwd_impl("ngpt_lmhead_ce_fwd_static", x_bf16, w_bf16, targets, mtp_weights, n_predict, prefix_targets,
                               prefix_weight, M, K, V, x_s, w_s, A, B, C, losses, lse, saved_sigma, x_f8, w_f8_vk, w_layout,
-                              ws, kStaticBytes, stream);
+                              ws, fwd_base_workspace_bytes(M), stream);      // the minimum size: always the tile kernel
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -422,6 +422,65 @@ def test_fused_lmhead_ce(amd, oracle, layout, M, K, V, n_predict, prefix):
     assert_close_gemm(dw, dw_ref)
 
 
+@pytest.mark.parametrize("codes", [False, True])
+@pytest.mark.parametrize("M,K,V,n_predict,prefix", [
+    (80, 256, 640, 1, False),           # fewer tokens than one token tile
+    (640, 256, 2432, 1, False),         # five token tiles, the last 256-row code block half used; 38 vocabulary units
+    (384, 768, 5120, 3, True),          # multi-token prediction + prefix targets
+    (1024, 512, 4096, 4, True),
+    (2048, 1024, 8192, 1, False),       # the longest contraction the token slab has room for
+])
+def test_lmhead_ce_forward_kernels_agree(amd, oracle, M, K, V, n_predict, prefix, codes):
+    """Two kernels serve the fused forward: the token-stationary one (activations resident in LDS, weights streamed
+    from a fragment-ordered copy in the workspace) and the tile kernel, which a workspace of the minimum size selects.
+    Same logits bit for bit, hence equal codes, sigmas and fp8 copies; the sums of exponentials are taken in a
+    different order, so lse and the losses agree to rounding."""
+    lib = amd._lib.load()
+    x, w, t, sc, mtp, pt, pw = _fused_case(oracle, M, K, V, seed=M + V + K, n_predict=n_predict, prefix=prefix)
+    t[M // 2] = -3
+    xd, wd, td, mtpd = dev(x), dev(w), dev(t), dev(mtp)
+    ptd = dev(pt) if pt is not None else None
+    pwd = dev(pw) if pw is not None else None
+    stream = torch.cuda.current_stream().cuda_stream
+    ptr = lambda a: None if a is None else a.data_ptr()
+    Vp, Mp = -(-V // 256) * 256, -(-M // 256) * 256
+
+    def run(nbytes):
+        o = dict(losses=torch.full((M,), float("nan"), device="cuda"), lse=torch.full((M,), float("nan"), device="cuda"),
+                 sig=torch.zeros((5, M), device="cuda"), x_f8=torch.zeros((M, K), dtype=torch.uint8, device="cuda"),
+                 w_f8=torch.zeros((V, K), dtype=torch.uint8, device="cuda"),
+                 codes=torch.zeros(lib.ngpt_lmhead_ce_codes_bytes(M, V), dtype=torch.uint8, device="cuda"))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        head = (ptr(xd), ptr(wd), ptr(td), ptr(mtpd), n_predict, ptr(ptd), ptr(pwd), M, K, V, sc["x_s"], sc["w_s"], 23.0, 5.0, 7.5,
+                ptr(o["losses"]), ptr(o["lse"]), ptr(o["sig"]), ptr(o["x_f8"]), ptr(o["w_f8"]))
+        if codes:
+            rc = lib.ngpt_lmhead_ce_fwd_codes(*head, ptr(o["codes"]), 0, ptr(ws), nbytes, stream)
+        else:
+            rc = lib.ngpt_lmhead_ce_fwd(*head, 0, ptr(ws), nbytes, stream)
+        assert rc == 0, lib.ngpt_last_error()
+        torch.cuda.synchronize()
+        return o
+
+    full, least = lib.ngpt_lmhead_ce_fwd_workspace_bytes(M, K, V, 0), lib.ngpt_lmhead_ce_fwd_min_workspace_bytes(M, K, V, 0)
+    assert full == least + V * K                  # this shape is one the token-stationary kernel takes
+    a, b = run(full), run(least)
+    for name in ("sig", "x_f8", "w_f8"):
+        assert torch.equal(a[name], b[name]), name
+    assert torch.isfinite(a["lse"]).all() and (a["lse"] - b["lse"]).abs().max().item() <= 1e-5
+    assert (a["losses"] - b["losses"]).abs().max().item() <= 1e-5
+    if codes:     # blocks [token tile][vocabulary / 128] of 256 tokens x 128 codes; tokens past M and entries past V are not defined
+        ca, cb = a["codes"].view(Mp // 256, Vp // 128, 256, 128), b["codes"].view(Mp // 256, Vp // 128, 256, 128)
+        tok = (torch.arange(Mp, device="cuda").view(Mp // 256, 1, 256, 1) < M)
+        voc = (torch.arange(Vp // 128, device="cuda").view(1, -1, 1, 1) * 128 + torch.arange(128, device="cuda").view(1, 1, 1, 128)) < V
+        keep = tok & voc
+        assert torch.equal(ca[keep.expand_as(ca)], cb[keep.expand_as(cb)])
+        assert int((ca[keep.expand_as(ca)] != 0).sum()) > 0.99 * M * V
+    # and against the oracle
+    l_ref, ctx = oracle.lm_head_ce_fwd(x, t, mtp, pt, pw, w, sc["x_s"], sc["w_s"], sc["grad_s"], sc["grad_scale"], w_layout="out_in")
+    assert (a["lse"].cpu() - ctx["lse"]).abs().max() < LOSS_TOL
+    assert abs(float(a["losses"].mean().cpu() - l_ref.mean())) <= LOSS_TOL
+
+
 @pytest.mark.parametrize("grad_scale", [3.0e5, 3.0e7])
 def test_fused_lmhead_ce_gradient_saturates(amd, oracle, grad_scale):
     """Row factors large enough for the e5m2 gradient to clamp at +-57344 (the recompute kernel then takes
