@@ -15,7 +15,9 @@ per-step HIP-event times beside it) and
                 average launch duration, against the published peak; `traffic` = HBM bytes per launch from the
                 rocprofv3 counter runs recorded in profiles/hbm_traffic.json (counters cannot be read in-process),
   cpu_baseline  the CPU oracle (PyTorch eager restatement) on a bounded sample of the same workload.
-Other workloads: mm_cfg1 (configuration 1), mlp_fwd (2), mlp_fwd_bwd (one layer of 4), mlp_cfg4 (4: twelve layers),
+The default line also carries `tail47_ms` (the same step with 47 vocabulary columns below the sigma-code window, as the
+padding ids of a trained model are) and `secondary`: configurations 1, 2 (bf16 and FP8 down projection), 4 and 5 timed briefly.
+Other workloads: mm_cfg1 (configuration 1), mlp_fwd (2), mlp_fwd_fp8down, mlp_fwd_bwd (one layer of 4), mlp_cfg4 (4: twelve layers),
 cfg5 (5), mm_lmhead, ce_logits, and `ceiling`: what an fp8 GEMM reaches on this machine (matrix pipe alone and the
 k-step skeleton on zero / random operands, the shipped kernel without its epilogue, the vendor library).
 """
@@ -34,8 +36,8 @@ import time
 import torch
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-PEAK_FP8_TFLOPS = 5033.0      # MI355X dense FP8 MFMA (published)
-PEAK_BF16_TFLOPS = 2516.6     # dense BF16
+PEAK_FP8_TFLOPS = 5000.0      # MI355X dense FP8 MFMA, the published figure every fp8 fraction below is taken against
+PEAK_BF16_TFLOPS = 2500.0     # dense BF16 (published)
 PEAK_HBM_GBS = 8000.0
 M, K, V = 49152, 768, 50304
 SLOT_NAMES = ["lm_head_ce_fwd", "dlogits_recompute", "dx_gemm", "dw_gemm", "fp8_gemm", "fc_relu2", "dpre", "bf16_gemm",
@@ -262,7 +264,7 @@ def emit(args, lib, desc, tokens, flops, ms, median_ms, kernels, work, traffic_k
     result["roofline"] = roofline_of(kernels, work, traffic, src)
     if cpu is not None:
         result["cpu_baseline"] = cpu
-    print(json.dumps(result))
+    return result
 
 
 # ---------------------------------------------------------------------------------------------- workloads
@@ -314,12 +316,16 @@ def workload_lmhead_ce(args, amd, lib, dev):
         _, o_ms, o_med, _ = run_timed(lib, other, max(5, args.steps // 5), 3)
         extra["other_mode"] = {"ce_backward": "recompute" if codes_mode else "codes", "ms_per_step": o_ms,
                                "median_ms_per_step": o_med, "tokens_per_s": M / (o_ms * 1e-3)}
+    if not args.tail_columns and not args.no_tail:
+        # the same step on logits as a trained model has them in the padding ids: 47 vocabulary columns below the code window
+        tail = argparse.Namespace(**{**vars(args), "tail_columns": 47, "no_other_mode": True, "no_cpu_baseline": True, "no_tail": True,
+                                     "steps": max(5, args.steps // 5), "warmup": 3})
+        extra["tail47_ms"] = workload_lmhead_ce(tail, amd, lib, dev)["ms_per_step"]
     cpu = None if args.no_cpu_baseline else cpu_baseline(x, w, t, sc)
-    emit(args, lib, "config 3: FP8 lm_head + fused softcapped cross-entropy, forward+backward, M=49152 K=768 V=50304, "
+    return emit(args, lib, "config 3: FP8 lm_head + fused softcapped cross-entropy, forward+backward, M=49152 K=768 V=50304, "
                     "(out,in) weight, n_predict=1; " + mode_desc, M, 6.0 * M * K * V, ms, median_ms, kernels, work,
          "lmhead_ce" if codes_mode else "lmhead_ce_recompute", extra=extra, cpu=cpu,
          metric="lm_head+CE fwd+bwd tokens/s at M=49152 (FP8 TFLOP/s and fraction of dense FP8 peak alongside)")
-    return 0
 
 
 def mlp_work(Mm, D, H, backward, layers=1):
@@ -331,8 +337,8 @@ def mlp_work(Mm, D, H, backward, layers=1):
     return work
 
 
-def secondary(args, amd, lib, dev) -> int:
-    """Other workloads of the path, same JSON shape."""
+def secondary(args, amd, lib, dev):
+    """Other workloads of the path, same JSON shape (None for an unknown name)."""
     g = torch.Generator().manual_seed(0)
     wl = args.workload
     cpu, work, traffic_key, dtype, extra = None, {}, wl, "fp8", None
@@ -356,33 +362,51 @@ def secondary(args, amd, lib, dev) -> int:
             return torch.ops.nanogpt.mm_backward(gd, x_f8, w_f8, x_s, w_s, grad_s)
         flops, desc, tokens = 6.0 * Mm * Nn * Kk, "nanogpt::mm forward + mm_backward at the lm_head shape, M=16384 N=50304 K=768", Mm
         work = {"fp8_gemm": (flops, "mfma-fp8")}
-    elif wl in ("mlp_fwd", "mlp_fwd_bwd", "mlp_cfg4"):
+    elif wl in ("mlp_fwd", "mlp_fwd_fp8down", "mlp_fwd_bwd", "mlp_cfg4"):
         Mm, D, H = 49152, 768, 3072
         L = 12 if wl == "mlp_cfg4" else 1
-        bwd = wl != "mlp_fwd"
+        bwd = wl in ("mlp_fwd_bwd", "mlp_cfg4")
+        fp8down = wl == "mlp_fwd_fp8down"
         x, w_fc_c, w_pt_c, dy_c = make_mlp(0, Mm, D, H, L)
         xr = x.to(dev).requires_grad_(bwd)
         w_fc = [w.to(dev).requires_grad_(bwd) for w in w_fc_c]
         w_pt = [w.to(dev).requires_grad_(bwd) for w in w_pt_c]
         dy = dy_c.to(dev)
         w_f8, scales = torch.ops.nanogpt.quant_up_weights(torch.stack([w.detach() for w in w_fc]))
+        down = None
+        if fp8down:
+            # the delayed-scaling state of the FP8 down projection (reference train_gpt.py:1423-1434, 1670-1675): e4m3 copy of
+            # W_proj stored [D, H] with its scale, the activation scale from a first pass's amax with the reference's headroom
+            w2_scale = (w_pt[0].detach().float().abs().max() / 448).reshape(1)
+            w2_dh = torch.empty((1, D, H), dtype=torch.float8_e4m3fn, device=dev)
+            nxt, part = torch.empty(1, device=dev), torch.zeros((1, (H // 64) * (D // 64)), device=dev)
+            amd.fused.quantize_transpose_mlp_down_weights(w_pt[0].detach()[None], w2_dh, nxt, w2_scale, part)
+            normed, x_f8, dequant = torch.ops.nanogpt.mlp_input_quant(xr, scales[0:1])
+            act_scale = (torch.ops.nanogpt.fc_relu2_fwd(x_f8, w_f8[0], dequant).float().max() * 1.25 / 448).reshape(1)
+            down = (w2_dh[0].T, w2_scale, act_scale, torch.zeros(1024, device=dev))
 
         def step():
             xr.grad = None
             for l in range(L):     # the layers run back to back on one stream, nothing synchronises in between
                 w_fc[l].grad = w_pt[l].grad = None
                 normed, x_f8, dequant = torch.ops.nanogpt.mlp_input_quant(xr, scales[l:l + 1])
-                out = amd.ReLUSqrdMLP(normed[None], w_fc[l], w_pt[l], w_f8[l], dequant, x_f8[None])
+                if down is not None:
+                    out = amd.ReLUSqrdMLP(normed[None], w_fc[l], w_pt[l], w_f8[l], dequant, x_f8[None], *down)
+                else:
+                    out = amd.ReLUSqrdMLP(normed[None], w_fc[l], w_pt[l], w_f8[l], dequant, x_f8[None])
                 if bwd:
                     out.backward(dy)
             return out
         flops = (12.0 if bwd else 4.0) * Mm * D * H * L
         desc = {"mlp_fwd": "config 2: norm + quantise + FP8 c_fc with ReLU^2 + bf16 c_proj, forward",
+                "mlp_fwd_fp8down": "config 2 with the FP8 down projection: norm + quantise + FP8 c_fc with ReLU^2 and e4m3 copy + FP8 c_proj, forward",
                 "mlp_fwd_bwd": "config 4 (one layer): norm + quantise + FP8 c_fc with ReLU^2 + bf16 c_proj, forward+backward",
                 "mlp_cfg4": "config 4: 12 layers (own weights) of norm + quantise + FP8 c_fc with ReLU^2 + bf16 c_proj, forward+backward"}[wl] \
             + ", M=49152 D=768 H=3072"
         tokens = Mm
         work = mlp_work(Mm, D, H, bwd, L)
+        if fp8down:
+            work["fp8_gemm"] = work.pop("bf16_gemm")[0], "mfma-fp8"
         if not args.no_cpu_baseline:
             cpu = cpu_baseline_mlp(x, w_fc_c[0], w_pt_c[0], dy_c, bwd)
             if L > 1:
@@ -434,8 +458,7 @@ def secondary(args, amd, lib, dev) -> int:
         flops, desc, tokens = 0.0, "nanogpt::ce_fwd_bwd on materialised logits, M=49152 V=50304 (bf16 in, e5m2 gradient out)", Mm
         dtype = "bf16 in, fp32 arithmetic, e5m2 out"
     else:
-        print(f"bench.py: unknown workload {wl}", file=sys.stderr)
-        return 2
+        return None
     if args.calibrate_copy:
         calibrate_copy(dev)
     out, ms, median_ms, kernels = run_timed(lib, step, args.steps, args.warmup)
@@ -444,8 +467,25 @@ def secondary(args, amd, lib, dev) -> int:
         hbm_bytes = tokens * 50304 * 3 + tokens * 12
         kernels = {"ce_rows": {"launches_per_step": 1.0, "avg_ms": median_ms, "ms_per_step": median_ms}}
         work = {"ce_rows": (hbm_bytes, "hbm")}
-    emit(args, lib, desc, tokens, flops, ms, median_ms, kernels, work, traffic_key, dtype=dtype, extra=extra, cpu=cpu)
-    return 0
+    return emit(args, lib, desc, tokens, flops, ms, median_ms, kernels, work, traffic_key, dtype=dtype, extra=extra, cpu=cpu)
+
+
+SECONDARY_IN_DEFAULT_LINE = (("cfg1", "mm_cfg1"), ("cfg2", "mlp_fwd"), ("cfg2_fp8_down", "mlp_fwd_fp8down"), ("cfg4", "mlp_cfg4"), ("cfg5", "cfg5"))
+
+
+def secondary_summary(args, amd, lib, dev):
+    """The other benchmark configurations, timed briefly (no CPU baseline), for the default line's "secondary" entry."""
+    out = {}
+    for key, wl in SECONDARY_IN_DEFAULT_LINE:
+        sub = argparse.Namespace(**{**vars(args), "workload": wl, "no_cpu_baseline": True, "calibrate_copy": False,
+                                    "steps": 20 if wl != "mlp_cfg4" else 10, "warmup": 3})
+        r = secondary(sub, amd, lib, dev)
+        roof = r.get("roofline") or {}
+        out[key] = {"workload": r["config"]["workload"], "ms": r["ms_per_step"], "tflops": r.get("tflops"),
+                    "tokens_per_s": r["value"], "kernel": roof.get("kernel"), "roofline_frac": roof.get("frac"),
+                    "roofline_peak": roof.get("peak"), "roofline_unit": roof.get("unit")}
+        torch.cuda.empty_cache()
+    return out
 
 
 def workload_ceiling(args, amd, dev) -> int:
@@ -651,6 +691,8 @@ def main() -> int:
                     help="headline workload: this many of the last vocabulary entries get logits far below the sigma-code window "
                          "in every row (and grad_scale = 64, so that they matter): measures the fallback of the codes backward")
     ap.add_argument("--no-other-mode", action="store_true", help="headline workload: do not also time the other --ce-backward mode")
+    ap.add_argument("--no-tail", action="store_true", help="headline workload: do not also time the step with 47 vocabulary columns below the code window")
+    ap.add_argument("--no-secondary", action="store_true", help="headline workload: leave out the brief runs of configurations 1, 2, 4 and 5")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy, the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -668,8 +710,16 @@ def main() -> int:
     if args.workload == "ceiling":
         return workload_ceiling(args, amd, dev)
     if args.workload != "lmhead_ce":
-        return secondary(args, amd, lib, dev)
-    return workload_lmhead_ce(args, amd, lib, dev)
+        result = secondary(args, amd, lib, dev)
+        if result is None:
+            print(f"bench.py: unknown workload {args.workload}", file=sys.stderr)
+            return 2
+    else:
+        result = workload_lmhead_ce(args, amd, lib, dev)
+        if not args.no_secondary and not args.tail_columns:
+            result["secondary"] = secondary_summary(args, amd, lib, dev)
+    print(json.dumps(result))
+    return 0
 
 
 if __name__ == "__main__":

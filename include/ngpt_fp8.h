@@ -189,6 +189,17 @@ int ngpt_gemm_bf16(const void* A, int a_layout, int64_t lda, const void* B, int 
                    int R, int C, int K, void* out_bf16, int64_t ldc, void* workspace, int64_t workspace_bytes,
                    void* stream);
 
+/* ---- fp8 GEMM scaled by two device-resident per-tensor scales --------------------------------
+ * out[r, c] = bf16(sum_k A[r, k] * B[c, k] * (*scale_a * *scale_b)), operands fp8 with the contraction contiguous:
+ * torch._scaled_mm(post_f8, W2_f8, scale_a=activation_scale, scale_b=W2_scale, out_dtype=bf16), the FP8 down
+ * projection of FusedLinearReLUSquareFunction.forward, triton_kernels.py:706-713.  scale_a / scale_b are
+ * 1-element fp32 device buffers read by the kernel (no host synchronisation).  K % 128 == 0, C % 4 == 0.
+ * workspace: ngpt_gemm_fp8_scaled_workspace_bytes(R, C, K) bytes (tiles cut along a long contraction meet in fp32). */
+int64_t ngpt_gemm_fp8_scaled_workspace_bytes(int R, int C, int K);
+int ngpt_gemm_fp8_scaled(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
+                         const float* scale_a, const float* scale_b, void* out_bf16, int64_t ldc,
+                         void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- delayed-scaling bookkeeping of the FP8 down projection, tied-embedding gradient add -----
  * scales[l] = max(max_i partial_amax[l * partial_stride + i], 1e-12) * headroom / 448:
  * reduce_mlp_activation_scales(_kernel), triton_kernels.py:502-519, 732-745. */

@@ -37,6 +37,8 @@ SIGNATURES = {
     "ngpt_transpose_u8": (_I, [_P, _I, _I, _P, _P]),
     "ngpt_transpose_copy": (_I, [_P, _I, _I, _P, _I, _P]),
     "ngpt_gemm_fp8_tn": (_I, [_P, _I, _L, _P, _I, _L, _I, _I, _I, _F, _P, _L, _I, _P]),
+    "ngpt_gemm_fp8_scaled_workspace_bytes": (_L, [_I, _I, _I]),
+    "ngpt_gemm_fp8_scaled": (_I, [_P, _I, _L, _P, _I, _L, _I, _I, _I, _P, _P, _P, _L, _P, _L, _P]),
     "ngpt_mm_fwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
     "ngpt_mm_fwd": (_I, [_P, _P, _I, _I, _I, _F, _F, _P, _P, _P, _I, _P, _L, _P]),
     "ngpt_mm_bwd_workspace_bytes": (_L, [_I, _I, _I, _I]),

@@ -929,7 +929,8 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
 int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
                float scale, void* out, int64_t ldc, int out_kind, hipStream_t st, int splits);
 int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
-                       float scale, void* out_bf16, int64_t ldc, float* part32, int a_rows_pad, hipStream_t st);
+                       float scale, void* out_bf16, int64_t ldc, float* part32, int a_rows_pad, hipStream_t st,
+                       const float* dscale_a = nullptr, const float* dscale_b = nullptr);
 int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
                       float scale, float* out, int64_t ldc, bool accumulate, float* part32, hipStream_t st);
 int64_t balanced_part_bytes(int R, int C, int K);

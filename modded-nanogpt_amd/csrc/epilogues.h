@@ -91,11 +91,21 @@ struct EpiStoreBf16 {
     float* part32;       // required when the walk splits tiles: one BM x BN fp32 tile per partial job
     bool is_partial;
     int part_slot;
+    // optional per-tensor scales that live in device memory (1-element fp32 buffers, both or neither): the result is
+    // scaled by scale * (*dscale_a * *dscale_b), the product taken on the device, no host synchronisation
+    const float* dscale_a;
+    const float* dscale_b;
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
     __device__ void partial(bool p, int slot) { is_partial = p; part_slot = slot; }
-    __device__ void begin(int, int, uint8_t*) {}
+    __device__ void begin(int, int, uint8_t*) {
+        if (dscale_a) {   // wave-uniform, written by an earlier kernel: scalar loads through the constant address space
+            const float a = ((const __attribute__((address_space(4))) float*)(uintptr_t)dscale_a)[0];
+            const float b = ((const __attribute__((address_space(4))) float*)(uintptr_t)dscale_b)[0];
+            scale *= a * b;
+        }
+    }
     __device__ void end(uint8_t*, int, int) {}
     template <class Cfg>
     __device__ void job_begin(int) {}

@@ -166,14 +166,15 @@ int64_t balanced_part_bytes(int R, int C, int K) {
 // part32: balanced_part_bytes(R, C, K) bytes of scratch for the split tiles.
 // fa may carry FMT_TRANSPOSED (A = panel of the transpose, a_rows_pad = R rounded up to 256).
 int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int layout, int R, int C, int K,
-                       float scale, void* out_bf16, int64_t ldc, float* part32, int a_rows_pad, hipStream_t st) {
+                       float scale, void* out_bf16, int64_t ldc, float* part32, int a_rows_pad, hipStream_t st,
+                       const float* dscale_a = nullptr, const float* dscale_b = nullptr) {
     if (R <= 0 || C <= 0 || K <= 0 || K % 128 || C % 4 || ldc % 4)
         return fail(NGPT_EALIGN, "gemm_balanced_bf16: R=%d C=%d K=%d ldc=%lld", R, C, K, (long long)ldc);
     BalancePlan p = plan_balance(R, C, K);
     if (p.splits > 1 && (!part32 || p.rem * p.splits > kMaxGrid)) return fail(NGPT_EINVAL, "gemm_balanced_bf16: split tiles need the fp32 scratch tiles");
     ProfileScope prof(g_gemm_slot, st);
     GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full, a_rows_pad};
-    EpiStoreBf16 epi{(uint16_t*)out_bf16, ldc, scale, R, C, part32, false, 0};
+    EpiStoreBf16 epi{(uint16_t*)out_bf16, ldc, scale, R, C, part32, false, 0, dscale_a, dscale_b};
     if (int e = launch_gemm<MainCfg>(g, fa, fb, epi, st)) return e;
     if (p.splits > 1) rem_tiles_kernel<uint16_t><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(part32, p.splits, (uint16_t*)out_bf16, ldc, R, C, p.full);
     return check_launch("gemm_balanced_bf16");
@@ -402,6 +403,28 @@ extern "C" int ngpt_fc_relu2_bwd_dpre(const void* dy_bf16, const void* w2_bf16, 
     EpiDpre epi{(uint16_t*)dpre_bf16, (const uint16_t*)post_bf16, H, H, M};
     ProfileScope prof(PROF_DPRE, (hipStream_t)stream);
     return launch_gemm_fmt<MainCfg, FMT_BF16, FMT_BF16>(g, epi, (hipStream_t)stream, 0);
+}
+
+// ------------------------------------------------------------------------------------------ fp8 GEMM with device-side scales
+// torch._scaled_mm(post_f8, W2_f8, scale_a = activation_scale, scale_b = W2_scale, out_dtype = bf16): the FP8 down
+// projection of FusedLinearReLUSquareFunction.forward (triton_kernels.py:706-713).  Both scales are 1-element fp32
+// device buffers; the epilogue multiplies by their product, so nothing of size [R, C] but the bf16 result is written.
+extern "C" int64_t ngpt_gemm_fp8_scaled_workspace_bytes(int R, int C, int K) { return balanced_part_bytes(R, C, K); }
+
+extern "C" int ngpt_gemm_fp8_scaled(const void* A, int fa, int64_t lda, const void* B, int fb, int64_t ldb, int R, int C, int K,
+                                    const float* scale_a, const float* scale_b, void* out_bf16, int64_t ldc,
+                                    void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!A || !B || !out_bf16 || !scale_a || !scale_b || !workspace) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_scaled: null pointer");
+    if ((fa != NGPT_FMT_E4M3 && fa != NGPT_FMT_E5M2) || (fb != NGPT_FMT_E4M3 && fb != NGPT_FMT_E5M2))
+        return fail(NGPT_EINVAL, "ngpt_gemm_fp8_scaled: fa=%d fb=%d", fa, fb);
+    if (int e = check_gemm_dims("ngpt_gemm_fp8_scaled", R, C, K, lda, ldb)) return e;
+    if (C % 4 || ldc % 4 || ldc < C) return fail(NGPT_EALIGN, "ngpt_gemm_fp8_scaled: C=%d ldc=%lld must be multiples of 4, ldc >= C", C, (long long)ldc);
+    if (workspace_bytes < ngpt_gemm_fp8_scaled_workspace_bytes(R, C, K))
+        return fail(NGPT_EWORKSPACE, "ngpt_gemm_fp8_scaled: workspace %lld < %lld bytes", (long long)workspace_bytes,
+                    (long long)ngpt_gemm_fp8_scaled_workspace_bytes(R, C, K));
+    GemmSlot slot(PROF_GEMM);
+    return gemm_balanced_bf16(A, fa, lda, B, fb, ldb, 0, R, C, K, 1.0f, out_bf16, ldc, (float*)workspace, 0, (hipStream_t)stream,
+                              scale_a, scale_b);
 }
 
 // ------------------------------------------------------------------------------------------ plain bf16 GEMM

@@ -131,11 +131,11 @@ class FusedLinearReLUSquareFunction(torch.autograd.Function):
         if W2_f8 is not None:
             # W2_f8 is the (H, D) view of a (D, H) row-major e4m3 buffer: the contraction index H
             # is contiguous on both sides, which is what the TN GEMM reads.  The two scales are
-            # 1-element device tensors; their product is taken on the device, no host sync.
+            # 1-element device tensors; the GEMM's epilogue multiplies by their product, no host sync.
             w2_dh = W2_f8.T
             assert w2_dh.is_contiguous()
-            x3 = ops.gemm_fp8_tn_op(post_f8, w2_dh, 1.0, True)
-            x3 = (x3 * (activation_scale * W2_scale)).to(torch.bfloat16)
+            x3 = ops.gemm_fp8_scaled(post_f8, w2_dh, activation_scale.reshape(-1).to(torch.float32),
+                                     W2_scale.reshape(-1).to(torch.float32))
         else:
             x3 = ops.gemm_bf16(post, W2, False, True)          # post @ W2, W2 [H, D] read with the contraction as its rows
         # the backward is all bf16 and needs post and W2 themselves, not the e4m3 copies

@@ -607,6 +607,32 @@ def gemm_fp8_tn(a: Tensor, b: Tensor, scale: float, out_dtype=torch.bfloat16, ou
     return out
 
 
+@torch.library.custom_op("nanogpt::gemm_fp8_scaled", mutates_args=())
+def gemm_fp8_scaled(a: Tensor, b: Tensor, scale_a: Tensor, scale_b: Tensor) -> Tensor:
+    """bf16 [R, C] = (a [R, K] fp8) @ (b [C, K] fp8).T * (scale_a * scale_b) with both scales 1-element fp32 device
+    tensors read by the kernel: `torch._scaled_mm(post_f8, W2_f8, scale_a=activation_scale, scale_b=W2_scale,
+    out_dtype=bf16)`, the FP8 down projection (reference triton_kernels.py:706-713), in one launch."""
+    _gpu(a, b, scale_a, scale_b)
+    fmt = {E4M3: _lib.E4M3, E5M2: _lib.E5M2}
+    R, K = a.shape
+    Cn = b.shape[0]
+    assert b.shape[1] == K and a.stride(1) == 1 and b.stride(1) == 1
+    assert scale_a.dtype == torch.float32 and scale_b.dtype == torch.float32 and scale_a.numel() >= 1 and scale_b.numel() >= 1
+    lib = _lib.load()
+    out = torch.empty((R, Cn), dtype=torch.bfloat16, device=a.device)
+    ws = _workspace(lib.ngpt_gemm_fp8_scaled_workspace_bytes(R, Cn, K), a.device)
+    _lib.check(lib.ngpt_gemm_fp8_scaled(_p(a), fmt[a.dtype], a.stride(0), _p(b), fmt[b.dtype], b.stride(0), R, Cn, K,
+                                        _p(scale_a), _p(scale_b), _p(out), Cn, _p(ws), ws.numel(), _stream(a)),
+               "ngpt_gemm_fp8_scaled")
+    return out
+
+
+@gemm_fp8_scaled.register_fake
+def _(a, b, scale_a, scale_b):
+    assert a.ndim == 2 and b.ndim == 2 and a.shape[1] == b.shape[1]
+    return a.new_empty((a.shape[0], b.shape[0]), dtype=torch.bfloat16)
+
+
 @torch.library.custom_op("nanogpt::gemm_fp8_tn", mutates_args=())
 def gemm_fp8_tn_op(a: Tensor, b: Tensor, scale: float, out_f32: bool) -> Tensor:
     """`gemm_fp8_tn` as a registered operator, for callers that run under `torch.compile(fullgraph=True)`

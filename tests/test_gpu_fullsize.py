@@ -27,20 +27,42 @@ def _rel(got, ref):
     return ((got.float() - ref.float()).norm() / ref.float().norm().clamp_min(1e-30)).item()
 
 
-def _run_gpu(x, w, t, sc):
+def _run_gpu(x, w, t, sc, mode="recompute"):
+    """Forward + backward through the operators; `mode` = where the backward takes the gradient of the logits from:
+    "recompute" (second logits GEMM) or "codes" (one code byte per logit kept by the forward, the default of the
+    autograd function and what bench.py times)."""
     d = "cuda"
     M = x.shape[0]
     mtp = torch.tensor([1.0], device=d)
     pt = torch.full((M,), -1, dtype=torch.int64, device=d)
     pw = torch.zeros(1, device=d)
     xd, wd, td = x.to(d), w.to(d), t.to(d)
-    losses, lse, sig, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(
-        xd, wd, td, mtp, pt, pw, sc["x_s"], sc["w_s"], sc["A"], sc["B"], sc["C"], False)
-    dx, dw = torch.ops.nanogpt.lmhead_ce_bwd(
-        x_f8, w_f8, td, mtp, pt, pw, lse, sig, sc["x_s"], sc["w_s"], sc["grad_s"], sc["grad_scale"],
-        sc["A"], sc["B"], sc["C"], False)
+    fwd_args = (xd, wd, td, mtp, pt, pw, sc["x_s"], sc["w_s"], sc["A"], sc["B"], sc["C"], False)
+    tail = (sc["x_s"], sc["w_s"], sc["grad_s"], sc["grad_scale"], sc["A"], sc["B"], sc["C"], False)
+    if mode == "codes":
+        losses, lse, sig, x_f8, w_f8, codes = torch.ops.nanogpt.lmhead_ce_fwd_codes(*fwd_args)
+        dx, dw = torch.ops.nanogpt.lmhead_ce_bwd_codes(x_f8, w_f8, td, mtp, pt, pw, lse, sig, codes, *tail)
+    else:
+        losses, lse, sig, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(*fwd_args)
+        dx, dw = torch.ops.nanogpt.lmhead_ce_bwd(x_f8, w_f8, td, mtp, pt, pw, lse, sig, *tail)
     torch.cuda.synchronize()
     return losses, lse, x_f8, w_f8, dx, dw
+
+
+def _check_fp8_copies_and_lse(oracle, x, w, sc, lse, x_f8, w_f8):
+    """The fp8 copies equal the oracle's quantiser on every byte, and EVERY row's lse equals an fp32 reference taken on
+    the GPU in row chunks from those verified copies (logits as bf16(acc * x_s * w_s), the oracle's softcap, logsumexp
+    in fp32 -- reference train_gpt.py:1689-1692), so nothing that later checks build on rests on the kernel's own statistics."""
+    assert torch.equal(x_f8.view(torch.uint8).cpu(), oracle.quant_e4m3(x, sc["x_s"]).view(torch.uint8))
+    assert torch.equal(w_f8.view(torch.uint8).cpu(), oracle.quant_e4m3(w, sc["w_s"]).view(torch.uint8))
+    wf = w_f8.float()
+    scale = torch.tensor(sc["x_s"], dtype=torch.float32) * torch.tensor(sc["w_s"], dtype=torch.float32)
+    worst = 0.0
+    for r0 in range(0, x_f8.shape[0], 2048):
+        logits = ((x_f8[r0:r0 + 2048].float() @ wf.T) * scale.item()).bfloat16()
+        z = sc["A"] * oracle.softcap_sigma(logits, sc["B"], sc["C"])
+        worst = max(worst, (torch.logsumexp(z, dim=1) - lse[r0:r0 + 2048]).abs().max().item())
+    assert worst <= LOSS_TOL, worst
 
 
 def _check_rows(oracle, x, w, t, sc, rows, losses, dx):
@@ -60,11 +82,13 @@ def _check_dw_columns(oracle, t, sc, cols, lse, x_f8, w_f8, dw):
     assert _rel(dw.cpu()[cols], dw_ref) <= GEMM_TOL
 
 
-def test_config3_full_size(amd, oracle):
+@pytest.mark.parametrize("mode", ["codes", "recompute"])
+def test_config3_full_size(amd, oracle, mode):
     x, w, t, sc = oracle.make_cfg3(seed=0)
     M, V = x.shape[0], w.shape[0]
-    losses, lse, x_f8, w_f8, dx, dw = _run_gpu(x, w, t, sc)
+    losses, lse, x_f8, w_f8, dx, dw = _run_gpu(x, w, t, sc, mode)
     assert torch.isfinite(losses).all() and torch.isfinite(dx.float()).all() and torch.isfinite(dw).all()
+    _check_fp8_copies_and_lse(oracle, x, w, sc, lse, x_f8, w_f8)
     # row subset (first / middle / last tiles, tile edges) against the oracle
     rows = torch.cat([torch.arange(0, M, 997), torch.arange(M - 64, M), torch.arange(255, M, 8192)]).unique()
     _check_rows(oracle, x, w, t, sc, rows, losses, dx)
@@ -75,8 +99,8 @@ def test_config3_full_size(amd, oracle):
     _check_dw_columns(oracle, t, sc, cols, lse, x_f8, w_f8, dw)
     # additivity over the token halves
     h = M // 2
-    la, _, _, _, dxa, dwa = _run_gpu(x[:h], w, t[:h], sc)
-    lb, _, _, _, dxb, dwb = _run_gpu(x[h:], w, t[h:], sc)
+    la, _, _, _, dxa, dwa = _run_gpu(x[:h], w, t[:h], sc, mode)
+    lb, _, _, _, dxb, dwb = _run_gpu(x[h:], w, t[h:], sc, mode)
     assert (torch.cat([la, lb]) - losses).abs().max().item() <= 1e-5
     assert _rel(torch.cat([dxa, dxb]), dx) <= 1e-3
     assert _rel(dwa + dwb, dw) <= 1e-4
@@ -90,7 +114,8 @@ def test_config5_shape(amd, oracle):
     w = (torch.randn(V, K, generator=g) / math.sqrt(K)).bfloat16()
     t = torch.randint(0, 50257, (M,), generator=g)
     sc = dict(x_s=100 / 448, w_s=1.6 / 448, grad_s=0.75 / 448, grad_scale=1.0, A=23.0, B=5.0, C=7.5)
-    losses, lse, x_f8, w_f8, dx, dw = _run_gpu(x, w, t, sc)
+    losses, lse, x_f8, w_f8, dx, dw = _run_gpu(x, w, t, sc, "codes")
+    _check_fp8_copies_and_lse(oracle, x, w, sc, lse, x_f8, w_f8)
     rows = torch.cat([torch.arange(0, M, 2039), torch.arange(M - 32, M)]).unique()
     _check_rows(oracle, x, w, t, sc, rows, losses, dx)
     cols = torch.cat([t[:8], torch.arange(V - 4, V)]).unique()
