@@ -19,7 +19,8 @@ The default line also carries `tail47_ms` (the same step with 47 vocabulary colu
 padding ids of a trained model are) and `secondary`: configurations 1, 2 (bf16 and FP8 down projection), 4 and 5 timed briefly.
 Other workloads: mm_cfg1 (configuration 1), mlp_fwd (2), mlp_fwd_fp8down, mlp_fwd_bwd (one layer of 4), mlp_cfg4 (4: twelve layers),
 cfg5 (5), mm_lmhead, ce_logits, and `ceiling`: what an fp8 GEMM reaches on this machine (matrix pipe alone and the
-k-step skeleton on zero / random operands, the shipped kernel without its epilogue, the vendor library).
+k-step skeleton on zero / random operands, the shipped tile kernel without its epilogue, the vendor library; needs the
+measurement build of the library, `python -m modded_nanogpt_amd.build`).
 """
 from __future__ import annotations
 
@@ -305,7 +306,7 @@ def workload_lmhead_ce(args, amd, lib, dev):
     work = {n: (gemm, "mfma-fp8") for n in ("lm_head_ce_fwd", "dlogits_recompute", "dx_gemm", "dw_gemm")}
     mode_desc = "the backward recomputes the logits (four GEMM passes)"
     if codes_mode:              # the second slot then is the code -> e5m2 conversion, a memory-bound pass over 2 x M x V bytes
-        kernels["dlogits_from_codes"] = kernels.pop("dlogits_recompute")
+        kernels["dlogits_from_codes"] = kernels.pop("dlogits_recompute", {"launches_per_step": 0.0, "avg_ms": 0.0, "ms_per_step": 0.0})
         del work["dlogits_recompute"]
         work["dlogits_from_codes"] = (2.0 * M * V, "hbm")
         mode_desc = "the forward keeps one sigma code byte per logit for the backward (three GEMM passes)"
@@ -567,111 +568,6 @@ def workload_ceiling(args, amd, dev) -> int:
         except Exception as e:    # a shape the library refuses is reported, not fatal
             res["rows"].append({"what": f"vendor library torch._scaled_mm {Mm} x {Nn} x {Kk}", "error": str(e)[:200]})
         del a, b
-    # What the output of a store-heavy epilogue costs, and whether it matters which waves carry it: the FP8 c_fc
-    # (49152 x 3072 x 768, ReLU^2, whole-line stores) complete, with half of its output stored by waves that also
-    # issue operand loads, with the same half stored by waves that issue none (the memory counter retires in issue
-    # order, so only such waves never wait for their stores), and with nothing stored.
-    Mm, Nn, Kk = 49152, 3072, 768
-    xq = torch.randn(Mm, Kk, device=dev).to(E4)
-    wq = (torch.randn(Nn, Kk, device=dev) * 0.05).to(E4)
-    post = torch.zeros(Mm, Nn, dtype=torch.bfloat16, device=dev)
-    modes = ((0, "complete"), (1, "half of the output, stored by 4 of 8 waves; all 8 waves issue operand loads"),
-             (2, "half of the output, stored by the 4 waves that issue no operand load"),
-             (3, "epilogue skipped; all 8 waves issue operand loads"), (4, "epilogue skipped; 4 waves issue operand loads"))
-    samples = {m: [] for m, _ in modes}
-    for rep in range(7):
-        for m, _ in modes:
-            lib.ngpt_tuning_set(5, m)
-            call = lambda: lib.ngpt_fc_relu2_fwd(xq.data_ptr(), wq.data_ptr(), one.data_ptr(), Mm, Nn, Kk, post.data_ptr(), None, None, None, 0, st)
-            for _ in range(3):
-                assert call() == 0, lib.ngpt_last_error()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(30):
-                call()
-            e1.record()
-            torch.cuda.synchronize()
-            samples[m].append(e0.elapsed_time(e1) / 30)
-    lib.ngpt_tuning_set(5, 0)
-    # Where the time of the fused CE forward goes, against the plain GEMM of the same shape: cycles of workgroup 0's waves
-    # inside the epilogue calls and outside them (per tile and per k-step), from the kernels' own cycle counters.
-    res["phase_rows"] = []
-    x, w, t, sc = make_cfg3(seed=0)
-    xd, wd, td = x.to(dev), w.to(dev), t.to(dev)
-    mtp = torch.tensor([1.0], device=dev)
-    pt = torch.full((x.shape[0],), -1, dtype=torch.int64, device=dev)
-    pw = torch.zeros(1, device=dev)
-    fwd_args = (xd, wd, td, mtp, pt, pw, sc["x_s"], sc["w_s"], sc["A"], sc["B"], sc["C"], False)
-    product_lib, amd._lib._lib = amd._lib._lib, lib          # the operators call through the measurement build here
-    try:
-        for what, op, alias in (("fused CE forward writing sigma codes", torch.ops.nanogpt.lmhead_ce_fwd_codes, 0),
-                                ("... with the code stores of every tile aliased onto two blocks (they stay in L2)", torch.ops.nanogpt.lmhead_ce_fwd_codes, 1),
-                                ("fused CE forward", torch.ops.nanogpt.lmhead_ce_fwd, 0)):
-            lib.ngpt_tuning_set(6, alias)
-            for _ in range(3):
-                op(*fwd_args)
-            buf = (ctypes.c_longlong * 64)()
-            assert lib.ngpt_bench_ce_phase_ticks(buf) == 0, lib.ngpt_last_error()
-            res["phase_rows"].append({"what": what, "ticks": list(buf[:32])})
-    finally:
-        lib.ngpt_tuning_set(6, 0)
-        amd._lib._lib = product_lib
-    a = torch.randint(0, 120, (R, 768), dtype=torch.uint8, device=dev).view(E4)
-    b = torch.randint(0, 120, (C, 768), dtype=torch.uint8, device=dev).view(E4)
-    out = torch.zeros(16, device=dev)
-    for _ in range(3):
-        assert lib.ngpt_gemm_fp8_tn(a.data_ptr(), 0, 768, b.data_ptr(), 0, 768, R, C, 768, 1.0, out.data_ptr(), C, 3, st) == 0, lib.ngpt_last_error()
-    buf = (ctypes.c_longlong * 64)()
-    assert lib.ngpt_bench_gemm_phase_ticks(buf) == 0, lib.ngpt_last_error()
-    res["phase_rows"].append({"what": f"plain GEMM {R} x {C} x 768, result discarded", "ticks": list(buf[:32])})
-    # Issue rates behind the epilogue designs: single vector instructions with 1, 2 and 4 waves per SIMD, and 64-lane LDS
-    # gathers with the address patterns of the softcap table (6656 entries)
-    names = ["v_mul_f32", "v_add_f32", "v_and_b32", "v_lshrrev_b32", "v_max_f32", "v_fma_f32", "v_perm_b32", "v_and_or_b32", "v_cvt_pk_bf16_f32",
-             "v_pk_sub_u16 clamp", "v_pk_min_u16", "v_pk_lshlrev_b16", "v_mov_b32_dpp", "v_exp_f32"]
-    vsink = torch.zeros(1024, dtype=torch.int32, device=dev)
-    vticks = torch.zeros(16, dtype=torch.int64, device=dev)
-    res["valu_rows"] = []
-    n_it = 2000
-    for kind, name in enumerate(names):
-        row = {"instruction": name}
-        for threads in (256, 512, 1024):
-            for _ in range(2):
-                assert lib.ngpt_bench_valu_rate(kind, threads, n_it, vsink.data_ptr(), vticks.data_ptr(), st) == 0, lib.ngpt_last_error()
-            torch.cuda.synchronize()
-            waves = threads // 64
-            t = vticks[:waves].double()
-            # one wave per SIMD: cycles per instruction of a wave; more: the slowest wave's cycles per instruction, per wave of the SIMD
-            row[f"waves_per_simd_{waves // 4}"] = float(t.max()) / (n_it * 32) / (waves // 4)
-        res["valu_rows"].append(row)
-    res["lds_rows"] = []
-    TABN = 6656
-    gen = torch.Generator().manual_seed(1)
-    def table_index(l):       # the fused CE's table index of a logit (sign bit | clamped bf16 magnitude)
-        bits = l.bfloat16().view(torch.int16).to(torch.int32) & 0xffff
-        t_ = ((bits & 0x7fff) - 0x3980).clamp(0, 2559)
-        return t_ + (bits >> 15) * 4096
-    n_off = cus * 512 * 16
-    lane = (torch.arange(n_off) // 16) % 64
-    kk = torch.arange(n_off) % 16
-    patterns = (("consecutive lanes, consecutive entries (no bank conflict)", lane + 64 * kk),
-                ("one entry for all lanes (broadcast)", torch.full((n_off,), 17)),
-                ("uniformly random entries", torch.randint(0, TABN, (n_off,), generator=gen)),
-                ("table entries of N(0, 1) logits", table_index(torch.randn(n_off, generator=gen))),
-                ("table entries of N(0, 3) logits", table_index(torch.randn(n_off, generator=gen) * 3)))
-    gsink = torch.zeros(512, device=dev)
-    for what, idx in patterns:
-        offs = (idx.to(torch.int32) * 4).to(dev)
-        row = {"pattern": what}
-        for threads in (256, 512):
-            for _ in range(2):
-                assert lib.ngpt_bench_lds_gather(offs.data_ptr(), TABN, threads, n_it, gsink.data_ptr(), vticks.data_ptr(), st) == 0, lib.ngpt_last_error()
-            torch.cuda.synchronize()
-            waves = threads // 64
-            row[f"waves_per_cu_{waves}"] = float(vticks[:waves].double().max()) / (n_it * 16) / waves      # LDS cycles per gather and compute unit
-        res["lds_rows"].append(row)
-    res["store_rows"] = [{"what": f"FP8 c_fc {Mm} x {Nn} x {Kk}, {what}", "ms": statistics.median(samples[m]), "ms_min": min(samples[m])}
-                         for m, what in modes]
     print(json.dumps(res))
     return 0
 

@@ -58,44 +58,17 @@ int ngpt_profile_enable(int on);
 int ngpt_profile_read(int slot, double* total_ms, int* launches);
 
 #ifdef NGPT_BENCH_BUILD
-/* Timing aid, no counterpart in the reference; exists only in the measurement build of the library
- * (libngpt_fp8_bench.so, compiled with -DNGPT_BENCH_BUILD), never in libngpt_fp8.so.  key 2: ablation bits
- * for timing runs of ngpt_gemm_fp8_tn with out_kind 3 (1 = no operand loads, 2 = no MFMAs, 4 = no k-loop
- * barrier; results are then meaningless); key 4: split-K factor used by ngpt_gemm_fp8_tn with out_kind 2;
- * key 5: ngpt_fc_relu2_fwd (whole-line path) stores only the upper four waves' half of the output (1), does so with
- * the lower four waves issuing every operand load (2), skips the epilogue (3), or both (4); key 6: 1 =
- * ngpt_lmhead_ce_fwd_codes writes every tile's codes over the same two blocks of the panel (stores that stay in the
- * L2); key 7: 1 = accept operand row strides below K (overlapping rows keep the operands cache resident in
- * timing runs).  Process-global and not synchronised: one thread, set before the timed calls. */
-int ngpt_tuning_set(int key, int value);
-
-/* Microbenchmark of the fp8 GEMM's k-step skeleton (same tile shape and instructions as the shipped kernel, no
+/* Measurement aids, no counterpart in the reference; they exist only in the measurement build of the library
+ * (libngpt_fp8_bench.so, compiled with -DNGPT_BENCH_BUILD), never in libngpt_fp8.so.  That build also accepts
+ * out_kind 3 in ngpt_gemm_fp8_tn: the contraction loop alone, result discarded.
+ *
+ * Microbenchmark of the fp8 GEMM's k-step skeleton (same tile shape and instructions as the tile kernel, no
  * epilogue): one launch of `grid` workgroups x `iters` k-steps of 256 x 256 x 128.  mode bits: 1 = operand fragments
  * re-read from LDS every sub-step, 2 = a workgroup barrier per k-step, 4 = 64 KiB of operands per k-step through
  * direct-to-LDS loads; 0 = the matrix pipe alone.  src: fp8 bytes, 64 KiB + 8 x 64 KiB per workgroup, src_stride
  * bytes apart; sink: 512 floats; ticks [grid][2] int64 = shader-clock cycles and 100 MHz wall ticks per workgroup. */
 int ngpt_bench_kstep_rate(const void* src, int64_t src_stride, int mode, int iters, int grid, float* sink,
                           long long* ticks, void* stream);
-
-/* Where the time of a GEMM-shaped kernel goes: every such kernel of the measurement build counts shader-clock
- * cycles in its workgroup 0, per wave w < 16: out64[4 w + 0] whole kernel, [4 w + 1] inside the epilogue calls of
- * its tiles, [4 w + 2] number of tiles, [4 w + 3] from leaving an epilogue to passing the barrier of the next tile's
- * first k-step (three quarters of that k-step's MFMAs plus the wait for slower waves).  These two calls wait for the
- * device and return the counts of the last launch: _ce_ of the fused lm_head + CE kernels (forward, dlogits
- * recompute), _gemm_ of every other GEMM of the library.  out64: 64 int64 in host memory. */
-int ngpt_bench_ce_phase_ticks(long long* out64);
-int ngpt_bench_gemm_phase_ticks(long long* out64);
-
-/* Issue rates of the machine that the epilogue designs lean on.  ngpt_bench_valu_rate: every wave of one workgroup
- * per compute unit runs iters x 32 vector instructions of one kind (0 v_mul_f32, 1 v_add_f32, 2 v_and_b32,
- * 3 v_lshrrev_b32, 4 v_max_f32, 5 v_fma_f32, 6 v_perm_b32, 7 v_and_or_b32, 8 v_cvt_pk_bf16_f32, 9 v_pk_sub_u16 clamp,
- * 10 v_pk_min_u16, 11 v_pk_lshlrev_b16, 12 v_mov_b32_dpp, 13 v_exp_f32) on independent registers; threads = 256, 512
- * or 1024 per workgroup = 1, 2 or 4 waves per SIMD; ticks (device, 16 int64) receives the shader-clock cycles of each
- * wave of workgroup 0; sink: 1024 uint32 (device).  ngpt_bench_lds_gather: every wave issues iters x 16 64-lane
- * ds_read_b32 with the byte offsets offs[(workgroup * threads + thread) * 16 ..+15] (device, below 4 * entries) into a
- * table of `entries` floats; threads = 256 or 512; ticks: 8 int64; sink: 512 floats. */
-int ngpt_bench_valu_rate(int kind, int threads, int iters, void* sink, long long* ticks, void* stream);
-int ngpt_bench_lds_gather(const void* offs, int entries, int threads, int iters, void* sink, long long* ticks, void* stream);
 #endif
 
 /* ---- quantisers ---------------------------------------------------------------------------

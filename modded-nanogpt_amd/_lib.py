@@ -10,12 +10,7 @@ LIB_PATH = pathlib.Path(__file__).resolve().parent / "lib" / "libngpt_fp8.so"
 # the same sources compiled with -DNGPT_BENCH_BUILD: adds the timing aids that measurements use and nothing else needs
 BENCH_LIB_PATH = LIB_PATH.with_name("libngpt_fp8_bench.so")
 BENCH_SIGNATURES = {
-    "ngpt_tuning_set": (c_int, [c_int, c_int]),
     "ngpt_bench_kstep_rate": (c_int, [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
-    "ngpt_bench_ce_phase_ticks": (c_int, [c_void_p]),
-    "ngpt_bench_gemm_phase_ticks": (c_int, [c_void_p]),
-    "ngpt_bench_valu_rate": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
-    "ngpt_bench_lds_gather": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
 }
 
 E4M3, E5M2 = 0, 1

@@ -59,4 +59,7 @@ def build(verbose: bool = True, bench: bool = False) -> pathlib.Path:
 
 if __name__ == "__main__":
     print(build())
-    print(build(bench=True))
+    try:
+        print(build(bench=True))
+    except RuntimeError as e:      # only `bench.py --workload ceiling` needs it
+        print("warning: the measurement build failed:", str(e)[:500], file=sys.stderr)

@@ -20,6 +20,7 @@
 #include <atomic>
 #include <cmath>
 #include <cstring>
+#include <numeric>
 
 namespace ngpt {
 
@@ -478,9 +479,6 @@ struct EpiCEFwdT {
     int ncand;            // n_predict (+1 with prefix targets)
     int* cand;            // LDS: [MAX_CAND][CE_MAX_BN] valid target column of the job's tokens, else -1
     float sum[8];
-#ifdef NGPT_BENCH_BUILD
-    int bench_alias;      // timing aid (tuning key 6): 1 = every tile writes its codes over the panel's first blocks (they stay in L2)
-#endif
 
     __device__ void partial(bool, int) {}
     __device__ void begin(int, int, uint8_t* extra) {
@@ -518,9 +516,6 @@ struct EpiCEFwdT {
         if constexpr (CODES) {
             const int wr = co.wave_row0 >> 6, wc = co.wave_col0 >> 7;
             cd_base = codes + ((int64_t)(c0 >> 8) * nkp + (r0 >> 7) + (wr >> 1)) * kPanelBytes;
-#ifdef NGPT_BENCH_BUILD
-            if (bench_alias == 1) cd_base = codes + (wr >> 1) * kPanelBytes;
-#endif
             cd_lane = (uint32_t)((128 * wc + (lane & 31)) * 128 + 64 * (wr & 1) + 16 * (lane >> 5));
         }
         auto code_store = [&](int tm, int tn, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
@@ -1019,13 +1014,7 @@ static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwdT<CODES>& epi, hip
     if (mg < 1) mg = 1;
     {
         ProfileScope prof(PROF_CE_FWD, st);
-#ifdef NGPT_BENCH_BUILD
-        EpiCEFwdT<CODES> timed = epi;
-        timed.bench_alias = g_tuning[6];
-        kernel<<<CE_XCDS * CE_SPLITS * mg, Cfg::THREADS, LDS, st>>>(g, timed);
-#else
         kernel<<<CE_XCDS * CE_SPLITS * mg, Cfg::THREADS, LDS, st>>>(g, epi);
-#endif
     }
     return check_launch("lm_head CE forward");
 }
@@ -1186,7 +1175,7 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
         if (int e = ngpt_quant_fp8_2d(w_bf16, K, V, w_s, NGPT_FMT_E4M3, nullptr, w_f8_vk, stream)) return e;
     }
 
-    GemmOperands g{(const uint8_t*)w_f8_vk, (const uint8_t*)x_f8, K, K, V, M, K, 1, 0};
+    GemmOperands g{(const uint8_t*)w_f8_vk, (const uint8_t*)x_f8, K, K, V, M, K, 1};
     const CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
     auto fill = [&](auto& epi) {
         epi.gtabE = tabE;
@@ -1368,7 +1357,7 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
         const int Mt = (int)round256(Mc), nkt = Mt / 128;
         if (int e = panel_transpose<2>((const uint8_t*)x_f8, K, m0, Mc, K, nkt, x_t, st)) return e;
         // 1. recompute the pass's logits and turn them into the e5m2 dlogits panel
-        GemmOperands g{(const uint8_t*)x_f8 + (int64_t)m0 * K, (const uint8_t*)w_f8_vk, K, K, Mc, V, K, 1, 0};
+        GemmOperands g{(const uint8_t*)x_f8 + (int64_t)m0 * K, (const uint8_t*)w_f8_vk, K, K, Mc, V, K, 1};
         EpiDlStore epi{};
         epi.gtabD = tabD;
         epi.rowf = rowf + m0;
@@ -1384,9 +1373,12 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
             ProfileScope prof(PROF_CE_DLOGITS, st);
             const int nvt = (int)(Vp / 256), nflags = 2 + (Mt / 256) * nvt;
             fill_f32_kernel<<<(nflags + 255) / 256, 256, 0, st>>>((float*)count, nflags, 0.0f);
-            // a sample of the tiles decides between the two ways (stride coprime to the tiles per row, so that the
-            // sample covers all vocabulary columns); the recompute of 45 % of the tiles costs what the conversion does
-            const int nbx = V / 128, ntiles = (Mt / 256) * nvt, stride = ntiles >= 64 * 127 ? 127 : 1, nsample = (ntiles + stride - 1) / stride;
+            // a sample of a few hundred tiles decides between the two ways, its stride coprime to the tiles per row so that
+            // the sample walks through all vocabulary columns; the recompute of 45 % of the tiles costs what the conversion does
+            const int nbx = V / 128, ntiles = (Mt / 256) * nvt;
+            int stride = std::max(1, ntiles / 300);
+            while (stride > 1 && std::gcd(stride, nvt) != 1) ++stride;
+            const int nsample = (ntiles + stride - 1) / stride;
             const int limit = nsample * 45 / 100;
             ce_codes_probe_kernel<<<nsample, 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, nbx, nvt, ntiles, stride, rowf, dcode, hits);
             ce_codes_to_dl_kernel<<<dim3(nbx, nkt), 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, rowf, dcode,
@@ -1434,16 +1426,6 @@ extern "C" int ngpt_lmhead_ce_bwd(const void* x_f8, const void* w_f8_vk, const i
                               w_layout, workspace, workspace_bytes, stream);
 }
 
-#ifdef NGPT_BENCH_BUILD
-// Measurement build: cycle counts of the last GEMM-shaped kernel launched from this file (g_phase_ticks in gemm_tn.h:
-// 16 waves x 4 numbers of workgroup 0), after a device synchronisation.
-extern "C" int ngpt_bench_ce_phase_ticks(long long* out64) {
-    if (!out64) return fail(NGPT_EINVAL, "ngpt_bench_ce_phase_ticks: null pointer");
-    if (hipDeviceSynchronize() != hipSuccess) return fail(NGPT_EINVAL, "ngpt_bench_ce_phase_ticks: device error");
-    if (hipMemcpyFromSymbol(out64, HIP_SYMBOL(g_phase_ticks), 64 * sizeof(long long)) != hipSuccess) return fail(NGPT_EINVAL, "ngpt_bench_ce_phase_ticks: copy failed");
-    return NGPT_OK;
-}
-#endif
 
 extern "C" int ngpt_lmhead_ce_fwd_codes(const void* x_bf16, const void* w_bf16, const int64_t* targets,
                                         const float* mtp_weights, int n_predict,

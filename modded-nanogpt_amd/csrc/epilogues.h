@@ -234,11 +234,9 @@ struct EpiDpre {
 };
 
 #ifdef NGPT_BENCH_BUILD
-// Mainloop-only timing aid (measurement build of the library only): keeps the accumulators alive but writes
+// Contraction-loop-only timing aid (measurement build of the library only): keeps the accumulators alive but writes
 // (practically) nothing.
-template <bool ABLATE>
-struct EpiDiscardT {
-    static constexpr bool ABLATABLE = ABLATE;
+struct EpiDiscard {
     float* out;   // >= 4 floats; workgroup 0 leaves its shader-clock and 100 MHz wall-clock tick counts in out[2], out[3]
     static constexpr int EXTRA_LDS = 0;
     static constexpr bool NEEDS_SCRATCH = false;
@@ -271,9 +269,6 @@ struct EpiDiscardT {
         if (s == 1.2345678e30f) out[0] = s;
     }
 };
-
-using EpiDiscard = EpiDiscardT<false>;
-using EpiDiscardAblate = EpiDiscardT<true>;    // honours GemmOperands::ablate, at the price of its branches
 #endif  // NGPT_BENCH_BUILD
 
 // out[r, c] (+)= acc * scale in fp32.  The += form (ACCUMULATE) uses floating-point atomics on an output the caller
@@ -457,21 +452,5 @@ struct EpiRelu2T {
     }
 };
 
-#ifdef NGPT_BENCH_BUILD
-// Timing aid: EpiRelu2Lines in which only waves store_from .. NWAVES - 1 run the epilogue for their part of the tile
-// (the rest of the output is never written).  With TileCfg::LOADERS = 4 and store_from = 4 the storing waves are the
-// ones that issue no operand load: what the output costs when it does not sit in a loading wave's memory counter.
-struct EpiRelu2LinesHalf : EpiRelu2Lines {
-    int store_from;
-    template <class Cfg>
-    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co, uint8_t* scratch, int lane) {
-        if ((int)(threadIdx.x >> 6) < store_from) {
-            stored_all = false;   // this wave issued no store: no relaxed wait
-            return;
-        }
-        EpiRelu2Lines::template tile<Cfg>(acc, r0, c0, co, scratch, lane);
-    }
-};
-#endif
 
 }  // namespace ngpt

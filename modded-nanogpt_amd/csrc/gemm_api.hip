@@ -78,17 +78,10 @@ int num_cus() {
     return n;
 }
 
-#ifdef NGPT_BENCH_BUILD
-int g_tuning[8] = {0, 2, 0, 0, 1, 0, 0, 0};
-static bool relaxed_strides() { return g_tuning[7] != 0; }
-#else
-static bool relaxed_strides() { return false; }
-#endif
-
 static int check_gemm_dims(const char* who, int R, int C, int K, int64_t lda, int64_t ldb) {
     if (R <= 0 || C <= 0 || K <= 0) return fail(NGPT_EINVAL, "%s: empty problem R=%d C=%d K=%d", who, R, C, K);
     if (K % 128) return fail(NGPT_EALIGN, "%s: contraction length %d must be a multiple of 128", who, K);
-    if (lda % 16 || ldb % 16 || ((lda < K || ldb < K) && !relaxed_strides()))
+    if (lda % 16 || ldb % 16 || lda < K || ldb < K)
         return fail(NGPT_EALIGN, "%s: operand row strides (%lld, %lld) must be multiples of 16 and >= K",
                     who, (long long)lda, (long long)ldb);
     return NGPT_OK;
@@ -101,7 +94,7 @@ thread_local int g_gemm_slot = PROF_GEMM;
 // and in the last round tiles % G workgroups work while the others idle (dx of the lm_head backward:
 // 576 tiles on 256 CUs = 2.25 rounds, paid as 3).  Instead the first floor(tiles / G) * G tiles run as
 // whole tiles and each of the remaining ones is cut along the contraction into as many jobs as fill
-// one more round; those partial results meet in fp32 through atomics.
+// one more round; every part goes to its own fp32 scratch tile and a summing pass adds a tile's parts up in a fixed order.
 struct BalancePlan {
     int tiles, full, rem, splits;
 };
@@ -173,7 +166,7 @@ int gemm_balanced_bf16(const void* A, int fa, int64_t lda, const void* B, int fb
     BalancePlan p = plan_balance(R, C, K);
     if (p.splits > 1 && (!part32 || p.rem * p.splits > kMaxGrid)) return fail(NGPT_EINVAL, "gemm_balanced_bf16: split tiles need the fp32 scratch tiles");
     ProfileScope prof(g_gemm_slot, st);
-    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full, a_rows_pad};
+    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, layout, p.full, a_rows_pad};
     EpiStoreBf16 epi{(uint16_t*)out_bf16, ldc, scale, R, C, part32, false, 0, dscale_a, dscale_b};
     if (int e = launch_gemm<MainCfg>(g, fa, fb, epi, st)) return e;
     if (p.splits > 1) rem_tiles_kernel<uint16_t><<<dim3(p.rem, kRemSlices), 256, 0, st>>>(part32, p.splits, (uint16_t*)out_bf16, ldc, R, C, p.full);
@@ -188,7 +181,7 @@ int gemm_balanced_f32(const void* A, int fa, int64_t lda, const void* B, int fb,
         return fail(NGPT_EALIGN, "gemm_balanced_f32: R=%d C=%d K=%d ldc=%lld", R, C, K, (long long)ldc);
     BalancePlan p = plan_balance(R, C, K);
     ProfileScope prof(g_gemm_slot, st);
-    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, 0, layout, p.full};
+    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, p.splits, layout, p.full};
     if (accumulate) {
         EpiStoreF32<true> epi{out, ldc, scale, R, C, nullptr, false, 0};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
@@ -208,12 +201,7 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
     if (splits < 1) splits = 1;
     if (splits > K / 128) splits = K / 128;
     if (splits > 1 && out_kind != 2) return fail(NGPT_EINVAL, "gemm_fp8_tn: split-K needs the accumulating fp32 output");
-#ifdef NGPT_BENCH_BUILD
-    const int ablate = g_tuning[2];
-#else
-    const int ablate = 0;
-#endif
-    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, splits, ablate};
+    GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, lda, ldb, R, C, K, splits};
     ProfileScope prof(g_gemm_slot, st);
     if (out_kind == 0) {
         EpiStoreBf16 epi{(uint16_t*)out, ldc, scale, R, C, nullptr, false, 0};
@@ -224,10 +212,6 @@ int gemm_store(const void* A, int fa, int64_t lda, const void* B, int fb, int64_
     }
     if (out_kind == 3) {
 #ifdef NGPT_BENCH_BUILD
-        if (g.ablate) {
-            EpiDiscardAblate epi{(float*)out, 0, 0};
-            return launch_gemm<MainCfg>(g, fa, fb, epi, st);
-        }
         EpiDiscard epi{(float*)out, 0, 0};
         return launch_gemm<MainCfg>(g, fa, fb, epi, st);
 #else
@@ -249,25 +233,6 @@ using namespace ngpt;
 extern "C" int ngpt_abi_version(void) { return 1; }
 extern "C" const char* ngpt_last_error(void) { return last_error_buf(); }
 extern "C" int ngpt_num_cus(void) { return num_cus(); }
-
-#ifdef NGPT_BENCH_BUILD
-// Measurement build: cycle counts of the last GEMM-shaped kernel launched from this file (g_phase_ticks in gemm_tn.h:
-// 16 waves x 4 numbers of workgroup 0), after a device synchronisation.
-extern "C" int ngpt_bench_gemm_phase_ticks(long long* out64) {
-    if (!out64) return fail(NGPT_EINVAL, "ngpt_bench_gemm_phase_ticks: null pointer");
-    if (hipDeviceSynchronize() != hipSuccess) return fail(NGPT_EINVAL, "ngpt_bench_gemm_phase_ticks: device error");
-    if (hipMemcpyFromSymbol(out64, HIP_SYMBOL(g_phase_ticks), 64 * sizeof(long long)) != hipSuccess) return fail(NGPT_EINVAL, "ngpt_bench_gemm_phase_ticks: copy failed");
-    return NGPT_OK;
-}
-#endif
-
-#ifdef NGPT_BENCH_BUILD
-extern "C" int ngpt_tuning_set(int key, int value) {
-    if (key < 0 || key >= 8) return fail(NGPT_EINVAL, "ngpt_tuning_set: key=%d", key);
-    g_tuning[key] = value;
-    return NGPT_OK;
-}
-#endif
 
 extern "C" int ngpt_profile_enable(int on) {
     std::lock_guard<std::mutex> lk(g_prof_mu);
@@ -305,11 +270,7 @@ extern "C" int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const voi
     if ((fmt_a | fmt_b) & ~1) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: fmt_a=%d fmt_b=%d", fmt_a, fmt_b);
     if (out_kind < 0 || out_kind > 3) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: out_kind=%d", out_kind);
     if (ldc < C) return fail(NGPT_EINVAL, "ngpt_gemm_fp8_tn: ldc=%lld < C=%d", (long long)ldc, C);
-#ifdef NGPT_BENCH_BUILD
-    const int splits = g_tuning[4];
-#else
     const int splits = 1;
-#endif
     return gemm_store(A, fmt_a, lda, B, fmt_b, ldb, R, C, K, scale, out, ldc, out_kind, (hipStream_t)stream, splits);
 }
 
@@ -399,7 +360,7 @@ extern "C" int ngpt_fc_relu2_bwd_dpre(const void* dy_bf16, const void* w2_bf16, 
     if (D % 64 || H % 8) return fail(NGPT_EALIGN, "ngpt_fc_relu2_bwd_dpre: need D %% 64 == 0 and H %% 8 == 0 (D=%d H=%d)", D, H);
     // bf16 operands: the loader works in bytes, so the contraction length and row strides are 2 * D.
     // Transposed product (tile rows = hidden units, tile columns = tokens), see EpiDpre.
-    GemmOperands g{(const uint8_t*)w2_bf16, (const uint8_t*)dy_bf16, 2 * (int64_t)D, 2 * (int64_t)D, H, M, 2 * D, 1, 0};
+    GemmOperands g{(const uint8_t*)w2_bf16, (const uint8_t*)dy_bf16, 2 * (int64_t)D, 2 * (int64_t)D, H, M, 2 * D, 1};
     EpiDpre epi{(uint16_t*)dpre_bf16, (const uint16_t*)post_bf16, H, H, M};
     ProfileScope prof(PROF_DPRE, (hipStream_t)stream);
     return launch_gemm_fmt<MainCfg, FMT_BF16, FMT_BF16>(g, epi, (hipStream_t)stream, 0);
@@ -448,13 +409,6 @@ extern "C" int ngpt_gemm_bf16(const void* A, int a_layout, int64_t lda, const vo
     // the loader works in bytes: contraction length and row strides are 2 x the element counts
     const int fa = a_layout == NGPT_K_CONTIGUOUS ? FMT_BF16 : (FMT_BF16 | FMT_TRANSPOSED);
     const int fb = b_layout == NGPT_K_CONTIGUOUS ? FMT_BF16 : (FMT_BF16 | FMT_TRANSPOSED);
-#ifdef NGPT_BENCH_BUILD
-    if (g_tuning[3]) {   // timing aid: the contraction loop alone (whole tiles, result discarded), honouring the ablation bits
-        GemmOperands g{(const uint8_t*)A, (const uint8_t*)B, 2 * lda, 2 * ldb, R, C, 2 * K, 1, g_tuning[2]};
-        EpiDiscardAblate epi{(float*)workspace, 0, 0};
-        return launch_gemm<MainCfg>(g, fa, fb, epi, (hipStream_t)stream);
-    }
-#endif
     GemmSlot slot(PROF_GEMM_BF16);
     return gemm_balanced_bf16(A, fa, 2 * lda, B, fb, 2 * ldb, 0, R, C, 2 * K, 1.0f, out_bf16, ldc, (float*)workspace, 0,
                               (hipStream_t)stream);
@@ -467,7 +421,7 @@ extern "C" int ngpt_linear_relu2_bf16(const void* x_bf16, const void* w_bf16, in
     if (!x_bf16 || !w_bf16 || !post_bf16) return fail(NGPT_EINVAL, "ngpt_linear_relu2_bf16: null pointer");
     if (M <= 0 || N <= 0 || K <= 0) return fail(NGPT_EINVAL, "ngpt_linear_relu2_bf16: empty problem M=%d N=%d K=%d", M, N, K);
     if (K % 64 || N % 8) return fail(NGPT_EALIGN, "ngpt_linear_relu2_bf16: need K %% 64 == 0 and N %% 8 == 0 (N=%d K=%d)", N, K);
-    GemmOperands gt{(const uint8_t*)w_bf16, (const uint8_t*)x_bf16, 2 * (int64_t)K, 2 * (int64_t)K, N, M, 2 * K, 1, 0};
+    GemmOperands gt{(const uint8_t*)w_bf16, (const uint8_t*)x_bf16, 2 * (int64_t)K, 2 * (int64_t)K, N, M, 2 * K, 1};
     EpiRelu2Lines epi{(uint16_t*)post_bf16, N, nullptr, N, M};
     ProfileScope prof(PROF_FC_RELU2, (hipStream_t)stream);
     return launch_gemm_fmt<MainCfg, FMT_BF16, FMT_BF16>(gt, epi, (hipStream_t)stream, 0);
@@ -482,7 +436,7 @@ extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float
         return fail(NGPT_EINVAL, "ngpt_fc_relu2_fwd: post_f8 needs act_scale and partial_amax");
     if (int e = check_gemm_dims("ngpt_fc_relu2_fwd", M, N, K, K, K)) return e;
     if (N % 16) return fail(NGPT_EALIGN, "ngpt_fc_relu2_fwd: N=%d must be a multiple of 16", N);
-    GemmOperands g{(const uint8_t*)x_f8, (const uint8_t*)w_f8, K, K, M, N, K, 1, 0};
+    GemmOperands g{(const uint8_t*)x_f8, (const uint8_t*)w_f8, K, K, M, N, K, 1};
     ProfileScope prof(PROF_FC_RELU2, (hipStream_t)stream);
     auto fill = [&](auto& epi) {
         epi.post = (uint16_t*)post_bf16;
@@ -504,14 +458,7 @@ extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float
     }
     if (N % 8 == 0) {
         // without the e4m3 copy: transposed product (tile rows = hidden units, tile columns = tokens), whole-line stores
-        GemmOperands gt{(const uint8_t*)w_f8, (const uint8_t*)x_f8, K, K, N, M, K, 1, 0};
-#ifdef NGPT_BENCH_BUILD
-        if (g_tuning[5]) {   // timing aid: half of the output stored, by waves that load (1) or by waves that do not (2)
-            EpiRelu2LinesHalf half{{(uint16_t*)post_bf16, N, dequant, N, M}, g_tuning[5] >= 3 ? 8 : 4};
-            if (g_tuning[5] == 2 || g_tuning[5] == 4) return launch_gemm_fmt<TileCfg<256, 256, 4, 2, 128, 2, 1, 4>, FMT_E4M3, FMT_E4M3>(gt, half, (hipStream_t)stream, 0);
-            return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(gt, half, (hipStream_t)stream, 0);
-        }
-#endif
+        GemmOperands gt{(const uint8_t*)w_f8, (const uint8_t*)x_f8, K, K, N, M, K, 1};
         EpiRelu2Lines epi{(uint16_t*)post_bf16, N, dequant, N, M};
         return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(gt, epi, (hipStream_t)stream, 0);
     }

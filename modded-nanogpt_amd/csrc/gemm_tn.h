@@ -52,7 +52,6 @@ struct GemmOperands {
     int64_t lda, ldb;   // ignored for a blocked operand
     int R, C, K;        // K % 128 == 0
     int splits;         // split-K: the contraction of a split tile is cut into this many jobs (>= 1); needs an accumulating epilogue if > 1
-    int ablate;         // timing aid, measurement build only (no epilogue of the default build honours it): bit 0 = issue no operand loads after the first, bit 1 = no MFMA work, bit 2 = no k-loop barrier
     int layout;         // kBlockedA | kBlockedB | kRowsPermuted
     int full_tiles;     // the first full_tiles tiles (in walk order) are never split; 0 = `splits` applies to every tile
     int a_rows_pad;     // transposed A only: R rounded up to 256
@@ -65,18 +64,13 @@ struct GemmOperands {
     int probe_limit;
 };
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1, int LOADERS_ = 0>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1>
 struct TileCfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, NSTAGES = NSTAGES_;
     static constexpr int WGS_PER_CU = WGS_PER_CU_;                 // co-resident workgroups the register budget allows
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int NWAVES = WAVES_M * WAVES_N;
     static constexpr int THREADS = NWAVES * 64;
-    // Waves that issue the operand loads (the first LOADERS of the workgroup; 0 = all of them).  With fewer loaders
-    // than waves the other waves never wait on the memory counter in the k-loop: the stores of their epilogue drain
-    // while the next tile is computed (the counter retires in issue order, so a wave that loads cannot do that).
-    static constexpr int LOADERS = LOADERS_ ? LOADERS_ : NWAVES;
-    static constexpr bool SPLIT_DUTIES = LOADERS != NWAVES;
     static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;   // wave tile
     static constexpr int TM = WTM / 32, TN = WTN / 32;             // MFMA tiles per wave
     static constexpr int KSUB = BK / 64;                           // 64-byte MFMA contraction steps per k-step
@@ -86,15 +80,13 @@ struct TileCfg {
     static constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int SMEM_BYTES = NSTAGES * STAGE_BYTES;
-    static constexpr int A_LOADS = BM / ROWS_PER_LOAD / LOADERS;   // wave-level loads per k-step and loading wave
-    static constexpr int B_LOADS = BN / ROWS_PER_LOAD / LOADERS;
+    static constexpr int A_LOADS = BM / ROWS_PER_LOAD / NWAVES;    // wave-level loads per k-step and wave
+    static constexpr int B_LOADS = BN / ROWS_PER_LOAD / NWAVES;
     static constexpr int LOADS = A_LOADS + B_LOADS;
     static constexpr int WAVE_SCRATCH = STAGE_BYTES / NWAVES;      // epilogue staging per wave
     static_assert(BK == 64 || BK == 128, "BK is 64 or 128 bytes");
     static_assert(NSTAGES >= 2 && NSTAGES <= 4, "2..4 LDS stages");
-    static_assert(LOADERS <= NWAVES && BM % (ROWS_PER_LOAD * LOADERS) == 0 && BN % (ROWS_PER_LOAD * LOADERS) == 0 &&
-                      BM % (ROWS_PER_LOAD * NWAVES) == 0 && BN % (ROWS_PER_LOAD * NWAVES) == 0,
-                  "tile rows must split over waves");
+    static_assert(BM % (ROWS_PER_LOAD * NWAVES) == 0 && BN % (ROWS_PER_LOAD * NWAVES) == 0, "tile rows must split over waves");
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be made of 32x32 MFMA tiles");
     // LDS swizzle: chunk q of row r is stored at chunk position q ^ swz(r)
     static __device__ __forceinline__ int swz(int r) { return (r / RPB) % CPR; }
@@ -150,7 +142,7 @@ struct LaneOffsets {
     // lanes that a transposing read serves together hit 32 distinct 8-byte bank pairs (see frag offsets below).
     // `lim` = columns of this operand left from the tile's origin (a multiple of 8): chunks past it are clamped.
     static __device__ uint32_t tr16_off(int load, int wave, int lane, int64_t ld, int lim) {
-        const int m = 2 * (wave + load * Cfg::LOADERS) + (lane >> 5);
+        const int m = 2 * (wave + load * Cfg::NWAVES) + (lane >> 5);
         int chunk = (lane & 31) ^ (4 * (m & 3));
         chunk = min(chunk, lim / 8 - 1);
         return (uint32_t)((int64_t)m * ld + chunk * 16);
@@ -166,12 +158,12 @@ struct LaneOffsets {
             if (a_transposed) {
                 // 1 KiB piece `c32` of the k-step's 32: half (token block) c32 / 16, contraction rows 8 * (c32 % 16) ..+7;
                 // the 16-byte chunk q of contraction row r lands at chunk position q ^ (r & 7)
-                const int c32 = wave + i * Cfg::LOADERS;
+                const int c32 = wave + i * Cfg::NWAVES;
                 const int r = 8 * (c32 & 15) + lrow;
                 a_off[i] = (uint32_t)((c32 >> 4) * kPanelBytes + r * 128 + ((lchunk ^ (r & 7)) << 4));
                 continue;
             }
-            int R = (wave + i * Cfg::LOADERS) * Cfg::ROWS_PER_LOAD + lrow;
+            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
             int q = lchunk ^ Cfg::swz(R);
             if (g.layout & kBlockedA) { a_off[i] = (uint32_t)(R * 128 + q * 16); continue; }   // padded: no clamp
             int rr = min(R, g.R - 1 - r0);                       // clamp rows past the end
@@ -183,7 +175,7 @@ struct LaneOffsets {
 #pragma unroll
         for (int i = 0; i < Cfg::B_LOADS; ++i) {
             if (b_tr16) { b_off[i] = tr16_off(i, wave, lane, g.ldb, g.C - c0); continue; }
-            int R = (wave + i * Cfg::LOADERS) * Cfg::ROWS_PER_LOAD + lrow;
+            int R = (wave + i * Cfg::NWAVES) * Cfg::ROWS_PER_LOAD + lrow;
             int q = lchunk ^ Cfg::swz(R);
             if (g.layout & kBlockedB) { b_off[i] = (uint32_t)(R * 128 + q * 16); continue; }
             int rr = min(R, g.C - 1 - c0);
@@ -312,20 +304,16 @@ struct TileMainloop {
             a_next += a_step;
         }
         b_next += b_step;
-        if (!loader()) return;
 #pragma unroll
         for (int i = 0; i < Cfg::A_LOADS; ++i)
-            global_to_lds16(ab + lo.a_off[i], s + (wave + i * Cfg::LOADERS) * 1024);
+            global_to_lds16(ab + lo.a_off[i], s + (wave + i * Cfg::NWAVES) * 1024);
     }
-    __device__ __forceinline__ bool loader() const { return !Cfg::SPLIT_DUTIES || wave < Cfg::LOADERS; }
     __device__ void issue_loads_b(uint8_t* smem) {
         if (b_pending == nullptr) return;
         uint8_t* s = smem + pending_stage * Cfg::STAGE_BYTES;
-        if (loader()) {
 #pragma unroll
-            for (int i = 0; i < Cfg::B_LOADS; ++i)
-                global_to_lds16(b_pending + lo.b_off[i], s + Cfg::A_BYTES + (wave + i * Cfg::LOADERS) * 1024);
-        }
+        for (int i = 0; i < Cfg::B_LOADS; ++i)
+            global_to_lds16(b_pending + lo.b_off[i], s + Cfg::A_BYTES + (wave + i * Cfg::NWAVES) * 1024);
         b_pending = nullptr;
     }
 
@@ -699,12 +687,6 @@ struct StepCursor {
     }
 };
 
-// Epilogues that declare `static constexpr bool ABLATABLE = true` honour GemmOperands::ablate (timing aid).
-template <class E, class = void>
-struct EpiAblatable : std::false_type {};
-template <class E>
-struct EpiAblatable<E, std::void_t<decltype(E::ABLATABLE)>> : std::bool_constant<E::ABLATABLE> {};
-
 // Epilogues that declare `static constexpr int TILE_STORES = n` promise that every wave issues exactly n
 // vector-memory instructions in each tile() call (and none in job_end).  The memory counter retires in
 // issue order and the operand loads of a tile's first k-step are issued before the previous tile's
@@ -736,13 +718,6 @@ struct EpiDropsFragments : std::false_type {};
 template <class E>
 struct EpiDropsFragments<E, std::void_t<decltype(E::DROPS_FRAGMENTS)>> : std::bool_constant<E::DROPS_FRAGMENTS> {};
 
-#ifdef NGPT_BENCH_BUILD
-// Measurement build: shader-clock cycles that wave w (< 16) of workgroup 0 spent in the last launch of a kernel of this
-// translation unit: [4 w + 0] whole kernel, [4 w + 1] inside the epilogue calls of its tiles, [4 w + 2] number of tiles,
-// [4 w + 3] between leaving an epilogue and passing the barrier of the next tile's first k-step (three quarters of that
-// k-step's MFMAs plus the wait for the slower waves).
-static __device__ long long g_phase_ticks[64];
-#endif
 
 template <class Cfg, int AFMT, int BFMT, class Epi, class Iter = GridIter>
 __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(GemmOperands g, Epi epi) {
@@ -750,13 +725,8 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     static_assert(Epi::EXTRA_LDS % 1024 == 0, "epilogue LDS must keep the stages 1 KiB aligned");
     static_assert(Cfg::NSTAGES == 2, "the k-loop below alternates between two LDS slots");
     uint8_t* const smem = smem_all + Epi::EXTRA_LDS;      // operand slots
-    const int ablate = EpiAblatable<Epi>::value ? __builtin_amdgcn_readfirstlane(g.ablate) : 0;
     TileMainloop<Cfg, AFMT, BFMT> ml;
     ml.init();
-#ifdef NGPT_BENCH_BUILD
-    const long long tick_start = clock64();
-    long long tick_epi = 0, tick_tiles = 0, tick_wait = 0, tick_left = 0;
-#endif
     const int bid = blockIdx.x, G = gridDim.x;
     const int nk = g.K / Cfg::BK;
     AccCoords<Cfg> coords(ml.wr, ml.wc, ml.lane, (g.layout & kRowsPermuted) != 0);
@@ -776,7 +746,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
                 ml.issue_loads_b(smem);
                 ml.set_tile(g, pre.it.tr() * Cfg::BM, pre.it.tc() * Cfg::BN, pre.kt);
             }
-            if (!(ablate & 1) || ahead == 0) ml.issue_loads(smem, into_slot);
+            ml.issue_loads(smem, into_slot);
             pre.advance();
             ++ahead;
         }
@@ -787,21 +757,11 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     ml.issue_loads_b(smem);
     epi.begin(bid, G, smem_all);
     // operands of the first k-step
-    if (ml.loader()) {
-        if (ahead == 2) wait_vmem_le<Cfg::LOADS>();
-        else wait_vmem_le<0>();
-    }
+    if (ahead == 2) wait_vmem_le<Cfg::LOADS>();
+    else wait_vmem_le<0>();
     wg_barrier();
 
-    v16f acc[Cfg::TM][Cfg::TN];
-    if (ablate) {   // the first k-step of a job overwrites the accumulators, unless the MFMAs are ablated
-#pragma unroll
-        for (int i = 0; i < Cfg::TM; ++i)
-#pragma unroll
-            for (int j = 0; j < Cfg::TN; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-    }
+    v16f acc[Cfg::TM][Cfg::TN];     // the first k-step of a job overwrites them
     v8i fa[Cfg::TM], fb = {};      // first fragments of the upcoming k-step, when `have`
 #pragma unroll
     for (int t = 0; t < Cfg::TM; ++t) fa[t] = (v8i){};
@@ -826,14 +786,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
             auto sync = [&]() {
                 // only the wait differs between the relaxed and the plain first k-step: a scalar branch around it
                 // instead of a second copy of the k-step
-                // (split duties: a loading wave stores nothing, the others wait for no load -- the barrier tells them)
-                if (Cfg::SPLIT_DUTIES) { if (ml.loader()) wait_vmem_le<0>(); }
-                else if (decltype(first)::value && EpiTileStores<Epi>::value > 0 && relaxed) wait_vmem_le<EpiTileStores<Epi>::value>();
+                if (decltype(first)::value && EpiTileStores<Epi>::value > 0 && relaxed) wait_vmem_le<EpiTileStores<Epi>::value>();
                 else wait_vmem_le<0>();
-                if (!(ablate & 4)) wg_barrier();
-#ifdef NGPT_BENCH_BUILD
-                if (decltype(first)::value && tick_left) { tick_wait += clock64() - tick_left; tick_left = 0; }
-#endif
+                wg_barrier();
             };
             auto refill_here = [&]() {
                 if (!(last_kt && keep_slot)) refill(slot);
@@ -841,15 +796,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
                 // k-step counts on every operand load having been issued before the epilogue's stores
                 if (last_kt) ml.issue_loads_b(smem);
             };
-            if (!(ablate & 2)) {
-                ml.template compute<decltype(first)::value, decltype(first)::value && EpiDropsFragments<Epi>::value>(
-                    smem, slot, slot ^ 1, have, more, acc, fa, fb, sync, refill_here);
-            } else {
-                ml.issue_loads_b(smem);
-                sync();
-                refill_here();
-            }
-            have = more && (TileMainloop<Cfg, AFMT, BFMT>::kAsmFrags16 || (AFMT & 3) != FMT_BF16) && !(ablate & 2);
+            ml.template compute<decltype(first)::value, decltype(first)::value && EpiDropsFragments<Epi>::value>(
+                smem, slot, slot ^ 1, have, more, acc, fa, fb, sync, refill_here);
+            have = more && (TileMainloop<Cfg, AFMT, BFMT>::kAsmFrags16 || (AFMT & 3) != FMT_BF16);
             --ahead;
             slot ^= 1;
         };
@@ -863,17 +812,9 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
         for (int kt = kt0 + 1; kt < kt1; ++kt) kstep(std::false_type{}, false, kt + 1 == kt1);
         // every wave passed the last k-step's barrier after its final read of slot ^ 1
         uint8_t* free_stage = smem + (slot ^ 1) * Cfg::STAGE_BYTES;
-#ifdef NGPT_BENCH_BUILD
-        const long long tick_e0 = clock64();
-#endif
         epi.partial(cur.partial(), cur.part_slot());
         epi.template tile<Cfg>(acc, r0, c0, coords, free_stage + ml.wave * Cfg::WAVE_SCRATCH, ml.lane);
         if (cur.job_end()) epi.template job_end<Cfg>(c0, cur.job_id(), coords, free_stage);
-#ifdef NGPT_BENCH_BUILD
-        tick_left = clock64();
-        tick_epi += tick_left - tick_e0;
-        ++tick_tiles;
-#endif
         if (keep_slot) {
             wg_barrier();          // all waves are done with the scratch
             refill(slot ^ 1);
@@ -884,14 +825,6 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     }
     wg_barrier();
     epi.end(smem, bid, G);
-#ifdef NGPT_BENCH_BUILD
-    if (bid == 0 && ml.lane == 0 && ml.wave < 16) {
-        g_phase_ticks[4 * ml.wave + 0] = clock64() - tick_start;
-        g_phase_ticks[4 * ml.wave + 1] = tick_epi;
-        g_phase_ticks[4 * ml.wave + 2] = tick_tiles;
-        g_phase_ticks[4 * ml.wave + 3] = tick_wait;
-    }
-#endif
 }
 
 }  // namespace ngpt

@@ -14,13 +14,6 @@ using SmallCfg = TileCfg<128, 128, 2, 2, 128, 2, 2>;
 // (Measured slower on MI355X for the shapes of this path: four 32 KiB stages of 64-byte k-steps, and a
 // 256 x 128 tile with two 4-wave workgroups per CU.  The kernel stays generic over TileCfg.)
 
-#ifdef NGPT_BENCH_BUILD
-// Measurement build only.  Tuning keys: [2] ablation bits (honoured by the discarding epilogue only),
-// [4] split-K factor of ngpt_gemm_fp8_tn, [5] FP8 c_fc with part of its epilogue / of its loading waves left out (gemm_api.hip),
-// [6] 1 = the code-writing CE forward stores every tile's codes over the same blocks (ce.hip),
-// [7] 1 = accept operand row strides below K (overlapping rows keep the operands cache resident)
-extern int g_tuning[8];
-#endif
 
 // hipFuncSetAttribute applies to the device that is current when it is called: one flag per kernel
 // instantiation and device.  Racing first calls both set the attribute, which is harmless.
@@ -55,12 +48,7 @@ int launch_gemm_fmt(const GemmOperands& g, const Epi& epi, hipStream_t st, int m
 }
 
 struct EpiStoreBf16;
-#ifdef NGPT_BENCH_BUILD
-template <bool ABLATE> struct EpiDiscardT;
-template <class Epi> constexpr bool kBf16Epi = std::is_same<Epi, EpiStoreBf16>::value || std::is_same<Epi, EpiDiscardT<true>>::value;
-#else
 template <class Epi> constexpr bool kBf16Epi = std::is_same<Epi, EpiStoreBf16>::value;
-#endif
 
 template <class Cfg, class Epi>
 int launch_gemm_cfg(const GemmOperands& g, int fa, int fb, const Epi& epi, hipStream_t st, int max_grid = 0) {

@@ -23,7 +23,10 @@ E4M3 = torch.float8_e4m3fn
 #                byte per logit as well, the e5m2 gradient itself; the logits are never stored), and the backward
 #                rebuilds the gradient from it: three GEMM passes per step;
 #   "recompute"  nothing of size [tokens, vocabulary] is kept and the backward runs the logits GEMM again: four passes.
-# Both give bit-identical gradients.  Set before the forward runs (module attribute or NGPT_CE_BACKWARD).
+# Given the same row statistics (lse, saved sigmas) both produce the same e5m2 gradient bytes, hence bit-identical dx / dW;
+# through this function the two forwards sum the exponentials of a row in different orders and with table entries that
+# differ in their last mantissa bits (the code-carrying ones), so lse and with it the gradients agree to about 1e-5 relative.
+# Set before the forward runs (module attribute or NGPT_CE_BACKWARD).
 CE_BACKWARD = os.environ.get("NGPT_CE_BACKWARD", "codes")
 assert CE_BACKWARD in ("codes", "recompute"), f"NGPT_CE_BACKWARD={CE_BACKWARD!r}: expected 'codes' or 'recompute'"
 
@@ -113,6 +116,14 @@ class FusedLinearReLUSquareFunction(torch.autograd.Function):
                 activation_scale=None, partial_amax=None):
         # saved for the backward: post = relu(x @ W1.T)^2 (the pre-activation never reaches memory)
         x_flat = x.view((-1, x.shape[-1]))
+        # There is no PyTorch fallback behind these kernels; say what they need before anything is launched.  The
+        # products of the backward contract over the tokens, so the token count is bound by the contraction step too.
+        tokens, model_dim, hidden_dim = x_flat.shape[0], x_flat.shape[1], W1.shape[0]
+        assert model_dim % 64 == 0 and hidden_dim % 64 == 0, (
+            f"FusedLinearReLUSquareFunction: model_dim={model_dim} and hidden_dim={hidden_dim} must be multiples of 64")
+        assert tokens % 8 == 0 and (tokens % 64 == 0 or not (x.requires_grad or W1.requires_grad or W2.requires_grad)), (
+            f"FusedLinearReLUSquareFunction: {tokens} tokens; the forward needs a multiple of 8, the backward (which "
+            "contracts over the tokens) a multiple of 64")
         post_f8 = None
         if W1_f8 is not None:
             assert x_f8 is not None and dequant_scale is not None

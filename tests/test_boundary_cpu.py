@@ -43,10 +43,10 @@ def test_header_symbols_are_exported_and_bound(amd):
 
 
 def test_timing_aids_are_in_the_measurement_build_only(amd):
-    """ngpt_tuning_set and the discarding epilogue flip process-global state and give meaningless results: the shipped
-    library must not export them; the measurement build (same sources, -DNGPT_BENCH_BUILD) has them on top."""
+    """The k-step microbenchmark and the discarding epilogue are measurement aids: the shipped library must not export
+    or accept them; the measurement build (same sources, -DNGPT_BENCH_BUILD) has them on top."""
     aids = declared_symbols(bench_only=True)
-    assert aids == sorted(amd._lib.BENCH_SIGNATURES) and "ngpt_tuning_set" in aids
+    assert aids == sorted(amd._lib.BENCH_SIGNATURES) and "ngpt_bench_kstep_rate" in aids
     lib = ctypes.CDLL(str(amd._lib.LIB_PATH))
     for n in aids:
         assert not hasattr(lib, n), f"{n} must not be exported by the default library"
@@ -84,8 +84,25 @@ def test_argument_errors_do_not_need_a_gpu(amd):
     assert lib.ngpt_mm_bwd(1, 1, 1, 128, 128, 128, 1.0, 1.0, 1.0, 1, 1, 0, 1, 16, None) == -3   # workspace
     assert lib.ngpt_ce_fwd_bwd(1, 1, 1, None, None, 1, 1, 4, 64, 9, 23.0, 5.0, 7.5, 1.0, 1.0, 1, 1 << 20, None) == -4
     assert lib.ngpt_mm_bwd_workspace_bytes(1024, 3072, 768, 0) >= 2 * 1024 * 3072 + 768 * 1024 + 768 * 3072
+    # the bf16 products of the MLP: contraction a multiple of 64, rows / columns multiples of 8 -- refused, never sent elsewhere
+    assert lib.ngpt_gemm_bf16(1, 1, 768, 1, 1, 768, 768, 768, 1000, 1, 768, 1, 1 << 30, None) == -2
+    assert b"K % 64" in lib.ngpt_last_error()
+    assert lib.ngpt_gemm_bf16(1, 0, 64, 1, 0, 64, 12, 768, 64, 1, 768, 1, 1 << 30, None) == -2
+    assert lib.ngpt_linear_relu2_bf16(1, 1, 64, 100, 64, 1, None) == -2
+    assert lib.ngpt_gemm_fp8_scaled(1, 0, 128, 1, 0, 128, 64, 64, 128, None, None, 1, 64, 1, 1 << 20, None) == -1      # scales are required
     with pytest.raises(amd._lib.NgptError):
         amd._lib.check(-2, "probe")
+
+
+def test_mlp_function_states_its_alignment_limits(amd):
+    """FusedLinearReLUSquareFunction has no PyTorch fallback: shapes its kernels cannot take are refused with a message
+    that names the limit, before any tensor is touched."""
+    x = torch.zeros(1, 100, 768, dtype=torch.bfloat16, requires_grad=True)
+    w1, w2 = torch.zeros(3072, 768, dtype=torch.bfloat16), torch.zeros(3072, 768, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="multiple of 8"):
+        amd.ReLUSqrdMLP(x, w1, w2)
+    with pytest.raises(AssertionError, match="multiples of 64"):
+        amd.ReLUSqrdMLP(torch.zeros(1, 128, 100, dtype=torch.bfloat16), torch.zeros(3072, 100, dtype=torch.bfloat16), w2)
 
 
 def test_operator_schemas_match_the_reference(amd):

@@ -278,7 +278,8 @@ def test_config4_mlp_backward_full_size(amd, oracle, M, D, H):
 def test_config4_twelve_layers_back_to_back(amd):
     """Benchmark configuration 4 as worded: twelve layers with their own weights, forward + backward, enqueued back
     to back on one stream without a synchronisation in between.  Every layer's outputs and gradients must be what
-    the same layer gives when it runs alone (split tiles meet through fp32 atomics, whose order is free)."""
+    the same layer gives when it runs alone (the parts of split tiles are summed in a fixed order, so nothing may differ
+    beyond what a run of the same kernels on the same data differs by)."""
     g = torch.Generator().manual_seed(12)
     M, D, H, L = 49152, 768, 3072, 12
     d = "cuda"
