@@ -24,6 +24,7 @@
 
 namespace ngpt {
 
+constexpr int kCodeGroupBytes = 256 * 16;   // code panel block: [8 groups of 16 codes][256 tokens][16 bytes]
 constexpr int TAB_LO = 0x3980;            // bf16 bits of 2^-12
 constexpr int TAB_N = 0x4380 - 0x3980;    // 2560 entries per sign, up to 2^8
 constexpr int TAB_NEG = 4096;             // negative logits start here, so the sign is one index bit
@@ -459,9 +460,11 @@ __device__ __forceinline__ uint32_t pack_codes4(float w0, float w1, float w2, fl
 }
 
 // CODES: the table entries carry sigma codes (ce_table_kernel with embed_codes) and every tile also writes its
-// 256 x 256 codes into the token-major code panel: blocks [token tile][vocabulary / 128] of 256 rows (tokens) x 128
-// bytes, a lane's 16 accumulator registers (16 vocabulary rows of one token, in register order, i.e. dw_pos order
-// inside every 32-group) as one 16-byte store.
+// 256 x 256 codes into the code panel: blocks [token tile][vocabulary / 128] of 256 tokens x 128 codes, a lane's 16
+// accumulator registers (16 vocabulary rows of one token, in register order, i.e. dw_pos order inside every
+// 32-group) as one 16-byte store.  Inside a block the 16-byte pieces are ordered [8 groups of 16 codes][256 tokens]:
+// the 32 lanes of a store instruction that hold consecutive tokens then write 512 contiguous bytes instead of 16
+// bytes in each of 32 lines, which is what the vector memory unit is fast at.
 template <bool CODES>
 struct EpiCEFwdT {
     static constexpr int EXTRA_LDS = CE_FWD_EXTRA_LDS;
@@ -516,10 +519,10 @@ struct EpiCEFwdT {
         if constexpr (CODES) {
             const int wr = co.wave_row0 >> 6, wc = co.wave_col0 >> 7;
             cd_base = codes + ((int64_t)(c0 >> 8) * nkp + (r0 >> 7) + (wr >> 1)) * kPanelBytes;
-            cd_lane = (uint32_t)((128 * wc + (lane & 31)) * 128 + 64 * (wr & 1) + 16 * (lane >> 5));
+            cd_lane = (uint32_t)((4 * (wr & 1) + (lane >> 5)) * kCodeGroupBytes + (128 * wc + (lane & 31)) * 16);
         }
         auto code_store = [&](int tm, int tn, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
-            *(v4i*)(cd_base + (cd_lane + tn * 4096 + tm * 32)) = (v4i){(int)w0, (int)w1, (int)w2, (int)w3};
+            *(v4i*)(cd_base + (cd_lane + tn * 512 + tm * 2 * kCodeGroupBytes)) = (v4i){(int)w0, (int)w1, (int)w2, (int)w3};
         };
         if (r0 + Cfg::BM <= V) {
             // Batches of 8 accumulator registers, software-pipelined by hand: while the 8 table reads of batch b are in
@@ -818,7 +821,7 @@ __global__ void ce_dl_fix_kernel(const float* __restrict__ lse, const float* __r
     }
 }
 
-// Backward from the forward's sigma codes: the code panel (token-major, see EpiCEFwdT) of one pass becomes that
+// Backward from the forward's sigma codes: the code panel (see EpiCEFwdT) of one pass becomes that
 // pass's dlogits panel (vocabulary-major, tokens of a k-step in dw_pos order), dl = e5m2_sat(rowf[token] * dcode[code]):
 // the same product and conversion as EpiDlStore, so the two agree bit for bit.  One workgroup moves 128 tokens x 128
 // vocabulary entries: 16 KiB of one code block in, converted on the way into LDS, transposed as in
@@ -849,18 +852,18 @@ __global__ __launch_bounds__(256) void ce_codes_probe_kernel(const uint8_t* __re
     v4i c[2][8];
     float rf[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) rf[j] = rowf[tok0 + ((tid + 256 * j) >> 3)];
+    for (int j = 0; j < 8; ++j) rf[j] = rowf[tok0 + tid];       // piece tid + 256 j of a block: group j of token tid
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
         const int kv = min(2 * vt + q, nbx - 1);     // the last tile of an odd count holds one block: read it twice
-        const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes;    // 256 tokens x 128 codes
+        const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes;    // [8 groups][256 tokens] x 16 codes
 #pragma unroll
         for (int j = 0; j < 8; ++j) c[q][j] = *(const v4i*)(src + (tid + 256 * j) * 16);
     }
     bool below = false;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        const bool inside = tok0 + ((tid + 256 * j) >> 3) < M;
+        const bool inside = tok0 + tid < M;
 #pragma unroll
         for (int q = 0; q < 2; ++q)
 #pragma unroll
@@ -884,12 +887,12 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
     __syncthreads();
     auto word_at = [&](int r, int w) -> uint32_t& { return tile[r * kStride + (w ^ (((r >> 4) & 7) << 2))]; };
     const int tok0 = m0 + a * 128;
-    const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes + ((tok0 >> 7) & 1) * (kPanelBytes / 2);
+    const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes + (tok0 & 128) * 16;
     bool below = false;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int i = tid + 256 * j, r = i >> 3, ch = i & 7;     // 16 codes of token tok0 + r
-        const v4i c = *(const v4i*)(src + r * 128 + ch * 16);
+        const int i = tid + 256 * j, r = i & 127, ch = i >> 7;   // 16 codes (group ch) of token tok0 + r
+        const v4i c = *(const v4i*)(src + ch * kCodeGroupBytes + r * 16);
         const float rf = rowf[tok0 + r];                          // zero past the last token
 #pragma unroll
         for (int k = 0; k < 4; ++k) {

@@ -195,8 +195,8 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
             uint8_t* cd_base = nullptr;
             uint32_t cd_lane = 0;
             if constexpr (CODES) {
-                cd_base = p.codes + ((int64_t)(c0 >> 8) * p.nkp + (u >> 1)) * kPanelBytes + 64 * (u & 1);
-                cd_lane = (uint32_t)(((c0 & 255) + j) * 128 + 16 * h);
+                cd_base = p.codes + ((int64_t)(c0 >> 8) * p.nkp + (u >> 1)) * kPanelBytes + 4 * (u & 1) * kCodeGroupBytes;
+                cd_lane = (uint32_t)(h * kCodeGroupBytes + ((c0 & 255) + j) * 16);
             }
             {
                 constexpr int NB = 16;
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
                         cw[2 * (b & 1)] = pack_codes4(cur[0], cur[1], cur[2], cur[3]);
                         cw[2 * (b & 1) + 1] = pack_codes4(cur[4], cur[5], cur[6], cur[7]);
                         if (b & 1)      // (tn, tm) = (b / 4, b / 2 % 2)
-                            *(v4i*)(cd_base + (cd_lane + (b >> 2) * 4096 + ((b >> 1) & 1) * 32)) =
+                            *(v4i*)(cd_base + (cd_lane + (b >> 2) * 512 + ((b >> 1) & 1) * 2 * kCodeGroupBytes)) =
                                 (v4i){(int)cw[0], (int)cw[1], (int)cw[2], (int)cw[3]};
                     }
                     __builtin_amdgcn_sched_barrier(0);

@@ -437,9 +437,10 @@ def test_lmhead_ce_forward_kernels_agree(amd, oracle, M, K, V, n_predict, prefix
     assert torch.isfinite(a["lse"]).all() and (a["lse"] - b["lse"]).abs().max().item() <= 1e-5
     assert (a["losses"] - b["losses"]).abs().max().item() <= 1e-5
     if codes:     # blocks [token tile][vocabulary / 128] of 256 tokens x 128 codes; tokens past M and entries past V are not defined
-        ca, cb = a["codes"].view(Mp // 256, Vp // 128, 256, 128), b["codes"].view(Mp // 256, Vp // 128, 256, 128)
-        tok = (torch.arange(Mp, device="cuda").view(Mp // 256, 1, 256, 1) < M)
-        voc = (torch.arange(Vp // 128, device="cuda").view(1, -1, 1, 1) * 128 + torch.arange(128, device="cuda").view(1, 1, 1, 128)) < V
+        ca, cb = a["codes"].view(Mp // 256, Vp // 128, 8, 256, 16), b["codes"].view(Mp // 256, Vp // 128, 8, 256, 16)
+        # inside a block: [8 groups of 16 codes][256 tokens][16 codes]
+        tok = (torch.arange(Mp, device="cuda").view(Mp // 256, 1, 1, 256, 1) < M)
+        voc = (torch.arange(Vp // 16, device="cuda").view(1, Vp // 128, 8, 1, 1) * 16 + torch.arange(16, device="cuda").view(1, 1, 1, 1, 16)) < V
         keep = tok & voc
         assert torch.equal(ca[keep.expand_as(ca)], cb[keep.expand_as(cb)])
         assert int((ca[keep.expand_as(ca)] != 0).sum()) > 0.99 * M * V
@@ -512,9 +513,10 @@ def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, pr
     assert torch.equal(u8(x_f8), u8(x_f8c)) and torch.equal(u8(w_f8), u8(w_f8c)) and torch.equal(sig0, sig1)
     assert (lse0 - lse1).abs().max().item() <= 2e-5 and (l0 - l1).abs().max().item() <= 1e-4
     assert codes.numel() == -(-M // 256) * 256 * (-(-V // 256) * 256)
-    # code panel: blocks [token tile][vocabulary / 128] of 256 tokens x 128 bytes; count zero codes inside the matrix
-    blocks = codes.view(-(-M // 256), -(-V // 256) * 2, 256, 128)[:, : V // 128]
-    valid = blocks.permute(0, 2, 1, 3).reshape(-1, V)[:M]
+    # code panel: blocks [token tile][vocabulary / 128] of [8 groups of 16 codes][256 tokens][16 bytes]; count zero
+    # codes inside the matrix
+    blocks = codes.view(-(-M // 256), -(-V // 256) * 2, 8, 256, 16)[:, : V // 128]
+    valid = blocks.permute(0, 3, 1, 2, 4).reshape(-1, V)[:M]
     assert bool((valid == 0).any()) == (below_window != 0)
     bwd = (x_f8, w_f8, dev(t), dev(mtp), ptd, pwd, lse1, sig1)
     tail = (sc["x_s"], sc["w_s"], sc["grad_s"], grad_scale, 23.0, 5.0, 7.5, in_out)
