@@ -248,7 +248,7 @@ int ngpt_ce_fwd_bwd(const void* logits_bf16, const int64_t* targets, const float
  * Forward: x [M,K] bf16, w bf16 in `w_layout` ([V,K] or [K,V]).  Writes losses [M] fp32 and,
  * saved for backward: lse [M] fp32 (log-sum-exp of the softcapped logits), saved_sigma
  * [(NGPT_MAX_PREDICT + 1) * M] fp32 (the bf16-rounded sigmoid at every candidate target column;
- * entries of invalid targets are left untouched), x_f8 [M,K] and w_f8_vk [V,K] (e4m3, always
+ * entries of invalid targets are zero), x_f8 [M,K] and w_f8_vk [V,K] (e4m3, always
  * vocabulary-major).  K % 128 == 0, M % 16 == 0, V % 16 == 0.
  * Two kernels serve the forward.  For V % 64 == 0 and K in {256, 512, 768, 1024} a token-stationary
  * kernel keeps 128 tokens' activations in LDS and streams the weights from a second, MFMA-fragment

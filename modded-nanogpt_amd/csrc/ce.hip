@@ -92,16 +92,21 @@ __device__ __forceinline__ float softcap_E(float sigma, const Softcap& sc) { ret
 // embed_codes: every tabE entry carries the sigma code of its logit in the low 8 bits of its fp32 pattern, and the
 // upper 24 bits are chosen so that the pattern read as a float is as close to exp(z - A) as those 8 bits allow
 // (relative error at most 2^-16, either sign): one table read then serves the sum of exponentials and the code.
-__global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc, bool embed_codes) {
-    int i = blockIdx.x * blockDim.x + threadIdx.x;
+// tabE may be null (the backward from codes keeps its code table in that place).
+__device__ __forceinline__ void ce_table_entry(int i, float* tabE, float* tabD, const Softcap& sc, bool embed_codes) {
     if (i >= TAB_ENTRIES) return;
     int t = i % TAB_NEG, neg = i / TAB_NEG;
-    if (t >= TAB_N) { tabE[i] = 0.0f; tabD[i] = 0.0f; return; }   // unused gap
+    if (t >= TAB_N) {   // unused gap
+        if (tabE) tabE[i] = 0.0f;
+        tabD[i] = 0.0f;
+        return;
+    }
     uint32_t bits = t == 0 ? 0u : (uint32_t)(TAB_LO + t);
     float l = bf16_bits_to_f32(bits | (neg ? 0x8000u : 0u));
     float s = softcap_sigma(l, sc);
     float e = softcap_E(s, sc);
     tabD[i] = e * s * (1.0f - s);
+    if (!tabE) return;
     if (embed_codes) {
         const uint32_t code = sigma_code(s), hi = __float_as_uint(e) & ~0xffu;
         float best = __uint_as_float(hi | code);
@@ -114,22 +119,26 @@ __global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc, bool embed
     }
     tabE[i] = e;
 }
+constexpr int TAB_BLOCKS = (TAB_ENTRIES + 255) / 256;
+__global__ void ce_table_kernel(float* tabE, float* tabD, Softcap sc, bool embed_codes) {
+    ce_table_entry(blockIdx.x * blockDim.x + threadIdx.x, tabE, tabD, sc, embed_codes);
+}
 
 // dcode[c] = D of the sigma with code c (the expression of ce_table_kernel's tabD), dcode[0] = 0; dcode[256] = D of
 // the largest sigma below the window, which bounds D of every sigma there if D grows with sigma up to it, and
 // infinity if it does not (D = exp(A sigma - A) sigma (1 - sigma) grows on (0, 1/2) whatever A > 0 is).
-__global__ void ce_dcode_kernel(float* dcode, Softcap sc) {
-    const int c = threadIdx.x;
+__device__ __forceinline__ float ce_d_below_window(const Softcap& sc) {
+    const float s = bf16_bits_to_f32((uint32_t)(SIGC_LOW - 1));
+    return s < 0.5f ? softcap_E(s, sc) * s * (1.0f - s) : __builtin_inff();
+}
+__device__ __forceinline__ void ce_dcode_entry(int c, float* dcode, const Softcap& sc) {   // c = 0 .. 255
     float d = 0.0f;
     if (c >= 1) {
         const float s = bf16_bits_to_f32((uint32_t)(SIGC_LOW + c - 1));
         d = softcap_E(s, sc) * s * (1.0f - s);
     }
     dcode[c] = d;
-    if (c == 0) {
-        const float s = bf16_bits_to_f32((uint32_t)(SIGC_LOW - 1));
-        dcode[256] = s < 0.5f ? softcap_E(s, sc) * s * (1.0f - s) : __builtin_inff();
-    }
+    if (c == 0) dcode[256] = ce_d_below_window(sc);
 }
 
 __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
@@ -668,14 +677,16 @@ namespace ngpt {
 // whole block, zero past M (zero codes in the panel's padding without any masking in the epilogue);
 // big[block] says whether any |rowf| of the block is large enough for rowf * D to leave the e5m2 range:
 // D = E * sigma * (1 - sigma) <= 1/4, so |rowf| <= 4 * 57344 needs no clamp.
-__global__ void ce_rowf_kernel(const float* __restrict__ lse, CandArgs ca, Softcap sc, float coef,
-                               float* __restrict__ rowf, int* __restrict__ big) {
-    int m = blockIdx.x * blockDim.x + threadIdx.x;
-    float f = 0.0f;
-    if (m < ca.M) f = coef * (row_weight_sum(ca, m) * expf(sc.A - lse[m]));
+__device__ __forceinline__ float ce_row_factor(const float* __restrict__ lse, const CandArgs& ca, const Softcap& sc, float coef, int m) {
+    return m < ca.M ? coef * (row_weight_sum(ca, m) * expf(sc.A - lse[m])) : 0.0f;
+}
+__device__ __forceinline__ void ce_rowf_block(int block, const float* __restrict__ lse, const CandArgs& ca, const Softcap& sc, float coef,
+                                              float* __restrict__ rowf, int* __restrict__ big) {
+    const int m = block * 256 + threadIdx.x;
+    const float f = ce_row_factor(lse, ca, sc, coef, m);
     rowf[m] = f;
     int b = __syncthreads_or(!(fabsf(f) <= 4.0f * 57344.0f));   // NaN counts as big
-    if (threadIdx.x == 0) big[blockIdx.x] = b;
+    if (threadIdx.x == 0) big[block] = b;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -836,40 +847,86 @@ __device__ __forceinline__ bool code_needs_logit(uint32_t w, float rf, float d_b
     return (((w - 0x01010101u) & ~w & 0x80808080u) != 0u) & !(fabsf(rf) * d_below < 0x1p-17f);
 }
 
-// Looks at every `stride`-th 256 x 256 tile of the pass's codes and counts those that the conversion would put on the
-// list.  If more than a given share of the sample is, the conversion below is skipped and the whole panel recomputed
-// from the logits (CondGridIter): conversion plus the recompute of that many tiles would cost more than the recompute
-// alone.  A step with codes then never costs much more than one without.
-__global__ __launch_bounds__(256) void ce_codes_probe_kernel(const uint8_t* __restrict__ codes, int nkp, int m0, int M, int nbx, int nvt, int ntiles,
-                                                            int stride, const float* __restrict__ rowf, const float* __restrict__ dcode,
-                                                            int* __restrict__ hits) {
-    const int idx = blockIdx.x * stride, tid = threadIdx.x;
-    if (idx >= ntiles) return;
-    const int vt = idx % nvt, tt = idx / nvt;
-    const float d_below = dcode[256];
-    const int tok0 = m0 + tt * 256;
-    // all loads first (branch-free), then the tests: the kernel is a handful of round trips to memory long
-    v4i c[2][8];
-    float rf[8];
+// Everything the backward needs before its first large kernel, in one launch of 256-thread workgroups; block ranges, in
+// this order (a range may be empty): the table of the gradient factor; the code table; the row factors of all rows;
+// zeros for the pass's tile list state; W^T as a panel; the pass's x^T as a panel; the probe of the pass's codes.
+//
+// The probe looks at every `stride`-th 256 x 256 tile of the pass's codes and counts those that the conversion would
+// put on the list.  If more than a given share of the sample is, the conversion is skipped and the whole panel
+// recomputed from the logits (TileListIter walks the whole grid then): conversion plus the recompute of that many tiles
+// would cost more than the recompute alone, so a step with codes never costs much more than one without.  Workgroup j
+// of the probe takes the sampled tiles j, j + kProbeBlocks, .. and writes its own count to hits[j]: nothing to zero
+// beforehand, and the readers add the kProbeBlocks counts up (probe_total).  It computes the row factors itself, with
+// the expression of ce_rowf_block, since those are written by the same launch.
+struct BwdPrepArgs {
+    float *tabD, *dcode;
+    Softcap sc;
+    const float* lse;
+    CandArgs ca;
+    float coef;
+    float* rowf;
+    int* big;
+    int* zero;
+    int nzero;
+    const uint8_t *w_f8, *x_f8;
+    int K, V, nkv, m0, Mc, nkt;
+    uint8_t *w_t, *x_t;
+    const uint8_t* codes;
+    int nkp, nbx, nvt, stride, nsample;
+    int* hits;
+    int b_tab, b_dcode, b_rowf, b_zero, b_wt, b_xt;      // workgroups of each range; the probe takes the rest
+};
+
+__device__ __forceinline__ void ce_codes_probe_block(const BwdPrepArgs& p, int b) {
+    const int tid = threadIdx.x;
+    const float d_below = ce_d_below_window(p.sc);
+    int found = 0;
+    for (int sample = b; sample < p.nsample; sample += kProbeBlocks) {
+        const int idx = sample * p.stride, vt = idx % p.nvt, tt = idx / p.nvt;
+        const int tok0 = p.m0 + tt * 256;
+        // all loads first (branch-free), then the tests: a sample is one round trip to memory long
+        const float rf = ce_row_factor(p.lse, p.ca, p.sc, p.coef, tok0 + tid);     // piece tid + 256 j of a block: group j of token tid
+        v4i c[2][8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) rf[j] = rowf[tok0 + tid];       // piece tid + 256 j of a block: group j of token tid
+        for (int q = 0; q < 2; ++q) {
+            const int kv = min(2 * vt + q, p.nbx - 1);     // the last tile of an odd count holds one block: read it twice
+            const uint8_t* src = p.codes + ((int64_t)(tok0 >> 8) * p.nkp + kv) * kPanelBytes;    // [8 groups][256 tokens] x 16 codes
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        const int kv = min(2 * vt + q, nbx - 1);     // the last tile of an odd count holds one block: read it twice
-        const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes;    // [8 groups][256 tokens] x 16 codes
+            for (int j = 0; j < 8; ++j) c[q][j] = *(const v4i*)(src + (tid + 256 * j) * 16);
+        }
+        bool below = false;
+        const bool inside = tok0 + tid < p.ca.M;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) c[q][j] = *(const v4i*)(src + (tid + 256 * j) * 16);
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) below |= inside & code_needs_logit((uint32_t)c[q][j][k], rf, d_below);
+        found += __syncthreads_or(below) ? 1 : 0;
     }
-    bool below = false;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const bool inside = tok0 + tid < M;
-#pragma unroll
-        for (int q = 0; q < 2; ++q)
-#pragma unroll
-            for (int k = 0; k < 4; ++k) below |= inside & code_needs_logit((uint32_t)c[q][j][k], rf[j], d_below);
+    if (tid == 0) p.hits[b] = found;
+}
+
+__global__ __launch_bounds__(256) void ce_bwd_prep_kernel(BwdPrepArgs p) {
+    int b = blockIdx.x;
+    const int tid = threadIdx.x;
+    if (b < p.b_tab) { ce_table_entry(b * 256 + tid, nullptr, p.tabD, p.sc, false); return; }
+    b -= p.b_tab;
+    if (b < p.b_dcode) { ce_dcode_entry(tid, p.dcode, p.sc); return; }
+    b -= p.b_dcode;
+    if (b < p.b_rowf) { ce_rowf_block(b, p.lse, p.ca, p.sc, p.coef, p.rowf, p.big); return; }
+    b -= p.b_rowf;
+    if (b < p.b_zero) {
+        if (b * 256 + tid < p.nzero) p.zero[b * 256 + tid] = 0;
+        return;
     }
-    if (__syncthreads_or(below) && tid == 0) atomicAdd(hits, 1);
+    b -= p.b_zero;
+    const int ncg = (p.K + 127) / 128;      // column groups of both transposes: their columns are the K features
+    if (b < p.b_wt) { panel_transpose_block<0, kPanelRaw>(p.w_f8, p.K, 0, p.V, p.K, p.nkv, 1.0f, p.w_t, b % ncg, b / ncg); return; }
+    b -= p.b_wt;
+    if (b < p.b_xt) { panel_transpose_block<2, kPanelRaw>(p.x_f8, p.K, p.m0, p.Mc, p.K, p.nkt, 1.0f, p.x_t, b % ncg, b / ncg); return; }
+    b -= p.b_xt;
+    ce_codes_probe_block(p, b);
 }
 
 __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __restrict__ codes, int nkp, int m0, int M,
@@ -880,7 +937,7 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
     constexpr int kStride = 33;
     __shared__ uint32_t tile[128 * kStride];
     __shared__ float dtab[256];
-    if (*probe_hits > probe_limit) return;      // the whole panel is recomputed instead (see ce_codes_probe_kernel)
+    if (probe_total(probe_hits) > probe_limit) return;      // the whole panel is recomputed instead (see ce_bwd_prep_kernel)
     const int kv = blockIdx.x, a = blockIdx.y, tid = threadIdx.x;
     dtab[tid] = dcode[tid];
     const float d_below = dcode[256];
@@ -1140,6 +1197,50 @@ extern "C" int64_t ngpt_lmhead_ce_fwd_workspace_bytes(int M, int K, int V, int w
 }
 
 namespace ngpt {
+// Everything the forward's GEMM kernel starts from, in one launch.  Block ranges: [0, bx) the e4m3 copy of the
+// activations; then bw blocks for the e4m3 copy of (out, in) weights, which also goes to the token-stationary kernel's
+// fragment order if w_frag is given (each 8-byte piece of a row is 8 bytes of one 16-byte fragment entry, see
+// xs_frag_from_f8_kernel); then the lookup tables; then the zeros of the partial sums (an empty vocabulary split must
+// read as zero) and of the saved sigmas (entries of candidates without a target are never written by the kernel).
+struct FwdPrepArgs {
+    const v4i* x; v2i* x_f8; int64_t nx8; float x_s;
+    const v4i* w; v2i* w_f8; int64_t nw8; float w_s; uint8_t* w_frag; int K8;
+    int bx, bw;
+    float *tabE, *tabD; Softcap sc; bool embed_codes;
+    float* zero0; int64_t n0; float* zero1; int64_t n1;
+};
+__global__ __launch_bounds__(256) void ce_fwd_prep_kernel(FwdPrepArgs p) {
+    int b = blockIdx.x;
+    const int tid = threadIdx.x;
+    if (b < p.bx) {
+        const QuantScale qs(p.x_s);
+        for (int64_t i = (int64_t)b * 256 + tid; i < p.nx8; i += (int64_t)p.bx * 256) p.x_f8[i] = quant8<FMT_E4M3>(p.x[i], qs);
+        return;
+    }
+    b -= p.bx;
+    if (b < p.bw) {
+        const QuantScale qs(p.w_s);
+        for (int64_t i = (int64_t)b * 256 + tid; i < p.nw8; i += (int64_t)p.bw * 256) {
+            const v2i q = quant8<FMT_E4M3>(p.w[i], qs);
+            p.w_f8[i] = q;
+            if (p.w_frag) {
+                const int row = (int)(i / p.K8), c8 = (int)(i - (int64_t)row * p.K8);     // 8-byte piece c8 of the row
+                const int u = row >> 6, tm = (row >> 5) & 1, ri = row & 31, ks = c8 >> 3, hh = (c8 >> 2) & 1, part = (c8 >> 1) & 1;
+                *(v2i*)(p.w_frag + (((int64_t)u * (p.K8 >> 3) + ks) * 4 + tm * 2 + part) * 1024 + (hh * 32 + ri) * 16 + (c8 & 1) * 8) = q;
+            }
+        }
+        return;
+    }
+    b -= p.bw;
+    if (b < TAB_BLOCKS) {
+        ce_table_entry(b * 256 + tid, p.tabE, p.tabD, p.sc, p.embed_codes);
+        return;
+    }
+    const int64_t i = (int64_t)(b - TAB_BLOCKS) * 256 + tid;
+    if (i < p.n0) p.zero0[i] = 0.0f;
+    else if (i - p.n0 < p.n1) p.zero1[i - p.n0] = 0.0f;
+}
+
 // Forward of the fused lm_head + CE on a workspace that the caller (ngpt_lmhead_ce_fwd) or the library itself
 // (ngpt_lmhead_ce_fwd_static) provides; `who` names the entry point in error messages.
 static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w_bf16, const int64_t* targets,
@@ -1168,14 +1269,29 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
     uint8_t* w_frag = ws + fwd_base_workspace_bytes(M);
 
     Softcap sc = make_softcap(A, B, C);
-    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc, sigma_codes != nullptr);
-    // a vocabulary split can be empty for a tiny V; its partial sums must read as zero
-    fill_f32_kernel<<<(CE_SPLITS * M + 255) / 256, 256, 0, st>>>(part, (int64_t)CE_SPLITS * M, 0.0f);
-    if (w_layout == NGPT_W_OUT_IN) {
-        if (int e = quant_e4m3_pair(x_bf16, x_f8, (int64_t)M * K, x_s, w_bf16, w_f8_vk, (int64_t)V * K, w_s, st)) return e;
-    } else {
-        if (int e = ngpt_quant_fp8(x_bf16, x_f8, (int64_t)M * K, x_s, NGPT_FMT_E4M3, stream)) return e;
-        if (int e = ngpt_quant_fp8_2d(w_bf16, K, V, w_s, NGPT_FMT_E4M3, nullptr, w_f8_vk, stream)) return e;
+    {
+        FwdPrepArgs a{};
+        a.x = (const v4i*)x_bf16; a.x_f8 = (v2i*)x_f8; a.nx8 = (int64_t)M * K / 8; a.x_s = x_s;
+        const bool w_here = w_layout == NGPT_W_OUT_IN;     // (in, out) weights go through the transposing quantiser below
+        a.w = (const v4i*)w_bf16; a.w_f8 = (v2i*)w_f8_vk; a.nw8 = w_here ? (int64_t)V * K / 8 : 0; a.w_s = w_s;
+        a.w_frag = (w_here && use_xs) ? w_frag : nullptr;
+        a.K8 = K / 8;
+        // quantiser blocks in proportion to the sizes
+        const int64_t cap = (int64_t)num_cus() * 16;
+        int64_t bx = (a.nx8 + 255) / 256, bw = (a.nw8 + 255) / 256;
+        if (bx + bw > cap) {
+            bx = std::max<int64_t>(1, bx * cap / (bx + bw));
+            bw = a.nw8 ? std::max<int64_t>(1, cap - bx) : 0;
+        }
+        a.bx = (int)bx; a.bw = (int)bw;
+        a.tabE = tabE; a.tabD = tabD; a.sc = sc; a.embed_codes = sigma_codes != nullptr;
+        a.zero0 = part; a.n0 = (int64_t)CE_SPLITS * M;
+        a.zero1 = saved_sigma; a.n1 = (int64_t)MAX_CAND * M;
+        const int64_t fill_blocks = (a.n0 + a.n1 + 255) / 256;
+        ce_fwd_prep_kernel<<<(int)(bx + bw + TAB_BLOCKS + fill_blocks), 256, 0, st>>>(a);
+        if (int e = check_launch("ce_fwd_prep_kernel")) return e;
+        if (!w_here)
+            if (int e = ngpt_quant_fp8_2d(w_bf16, K, V, w_s, NGPT_FMT_E4M3, nullptr, w_f8_vk, stream)) return e;
     }
 
     GemmOperands g{(const uint8_t*)w_f8_vk, (const uint8_t*)x_f8, K, K, V, M, K, 1};
@@ -1190,8 +1306,10 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
         epi.ncand = prefix_targets ? n_predict + 1 : n_predict;
     };
     if (use_xs) {
-        xs_frag_from_f8_kernel<<<std::min((V / XS_UNIT) * (K / 128), 8 * num_cus()), 256, 0, st>>>((const uint8_t*)w_f8_vk, V, K, w_frag);
-        if (int e = check_launch("xs_frag_from_f8_kernel")) return e;
+        if (w_layout != NGPT_W_OUT_IN) {
+            xs_frag_from_f8_kernel<<<std::min((V / XS_UNIT) * (K / 128), 8 * num_cus()), 256, 0, st>>>((const uint8_t*)w_f8_vk, V, K, w_frag);
+            if (int e = check_launch("xs_frag_from_f8_kernel")) return e;
+        }
         XsArgs a{};
         a.w_frag = w_frag;
         a.x_f8 = (const uint8_t*)x_f8;
@@ -1287,8 +1405,8 @@ extern "C" int ngpt_lmhead_ce_fwd_static(const void* x_bf16, const void* w_bf16,
 static int64_t bwd_part_bytes(int64_t Mc, int64_t Mt, int K, int V) {
     return std::max(balanced_part_bytes((int)Mc, K, V), std::max(balanced_part_bytes(V, K, (int)Mt), balanced_part_bytes(K, V, (int)Mt)));
 }
-// codes backward: count | probe hits | flags [tiles] | list [tiles] of the 256 x 256 tiles of one pass's logits
-static int64_t flag_bytes(int64_t Mt, int64_t Vp) { return align_up((2 + 2 * (Mt / 256) * (Vp / 256)) * 4, 256); }
+// codes backward: probe counts [kProbeBlocks] | count | flags [tiles] | list [tiles] of the 256 x 256 tiles of one pass's logits
+static int64_t flag_bytes(int64_t Mt, int64_t Vp) { return align_up((kProbeBlocks + 1 + 2 * (Mt / 256) * (Vp / 256)) * 4, 256); }
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
     int64_t Mc = bwd_chunk_rows(M), Mt = round256(Mc), Kp = round256(K), Vp = round256(V);
@@ -1335,9 +1453,9 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
     ws += Vp * Mt_max;
     float* parts = (float*)ws;
     ws += bwd_part_bytes(Mc_max, Mt_max, K, V);
-    int* count = (int*)ws;                   // number of listed tiles
-    int* hits = count + 1;                   // sampled code blocks that would list a tile
-    int* flags = count + 2;                  // per 256 x 256 tile of the pass's logits: a sigma of it lies below the code window and matters
+    int* hits = (int*)ws;                    // sampled tiles that would be listed, one count per workgroup of the probe
+    int* count = hits + kProbeBlocks;        // number of listed tiles
+    int* flags = count + 1;                  // per 256 x 256 tile of the pass's logits: a sigma of it lies below the code window and matters
     int* list = flags + (Mt_max / 256) * (Vp / 256);
     static_assert(BWD_CHUNK_ROWS / 256 < 65536, "a list entry holds the token tile in its upper 16 bits");
     if (Vp / 256 >= 65536) return fail(NGPT_ERANGE, "%s: V=%d", who, V);
@@ -1345,20 +1463,41 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
     Softcap sc = make_softcap(A, B, C);
     const float coef = make_coef(A, C, grad_s, grad_scale);
     CandArgs ca{targets, prefix_targets, mtp_weights, prefix_weight, n_predict, M, V};
-    ce_table_kernel<<<(TAB_ENTRIES + 255) / 256, 256, 0, st>>>(tabE, tabD, sc, false);
     float* dcode = tabE;                     // the backward does not read tabE: its first 257 entries serve as the code table
-    if (sigma_codes) ce_dcode_kernel<<<1, 256, 0, st>>>(dcode, sc);
-    ce_rowf_kernel<<<(M + 255) / 256, 256, 0, st>>>(lse, ca, sc, coef, rowf, big);
-    if (int e = check_launch("ce_rowf_kernel")) return e;
     const int nkv = V / 128;
-    if (int e = panel_transpose<0>((const uint8_t*)w_f8_vk, K, 0, V, K, nkv, w_t, st)) return e;
     const bool several = M > Mc_max;       // dw then accumulates over the passes
     if (several) fill_f32_kernel<<<(int)(((int64_t)V * K + 255) / 256), 256, 0, st>>>((float*)dw_f32, (int64_t)V * K, 0.0f);
 
     for (int m0 = 0; m0 < M; m0 += Mc_max) {
         const int Mc = (M - m0 < Mc_max) ? (M - m0) : Mc_max;
         const int Mt = (int)round256(Mc), nkt = Mt / 128;
-        if (int e = panel_transpose<2>((const uint8_t*)x_f8, K, m0, Mc, K, nkt, x_t, st)) return e;
+        const int nvt = (int)(Vp / 256), nbx = V / 128, ntiles = (Mt / 256) * nvt;
+        // a sample of a few hundred tiles decides between conversion and recompute, its stride coprime to the tiles per row
+        // so that the sample walks through all vocabulary columns; the recompute of 45 % of the tiles costs what the conversion does
+        int stride = std::max(1, ntiles / 300);
+        while (stride > 1 && std::gcd(stride, nvt) != 1) ++stride;
+        const int nsample = (ntiles + stride - 1) / stride;
+        const int limit = nsample * 45 / 100;
+        {   // tables, row factors and W^T with the first pass; x^T, the tile list's zeros and the probe with every pass
+            BwdPrepArgs a{};
+            a.tabD = tabD; a.dcode = dcode; a.sc = sc; a.lse = lse; a.ca = ca; a.coef = coef; a.rowf = rowf; a.big = big;
+            a.zero = count; a.nzero = 1 + ntiles;
+            a.w_f8 = (const uint8_t*)w_f8_vk; a.x_f8 = (const uint8_t*)x_f8;
+            a.K = K; a.V = V; a.nkv = nkv; a.m0 = m0; a.Mc = Mc; a.nkt = nkt; a.w_t = w_t; a.x_t = x_t;
+            a.codes = (const uint8_t*)sigma_codes; a.nkp = (int)(Vp / 128); a.nbx = nbx; a.nvt = nvt; a.stride = stride; a.nsample = nsample;
+            a.hits = hits;
+            const int ncg = (K + 127) / 128;
+            const bool first = m0 == 0;
+            a.b_tab = first ? TAB_BLOCKS : 0;
+            a.b_dcode = (first && sigma_codes) ? 1 : 0;
+            a.b_rowf = first ? (M + 255) / 256 : 0;
+            a.b_zero = sigma_codes ? (a.nzero + 255) / 256 : 0;
+            a.b_wt = first ? ncg * nkv : 0;
+            a.b_xt = ncg * nkt;
+            const int b_probe = sigma_codes ? kProbeBlocks : 0;
+            ce_bwd_prep_kernel<<<a.b_tab + a.b_dcode + a.b_rowf + a.b_zero + a.b_wt + a.b_xt + b_probe, 256, 0, st>>>(a);
+            if (int e = check_launch("ce_bwd_prep_kernel")) return e;
+        }
         // 1. recompute the pass's logits and turn them into the e5m2 dlogits panel
         GemmOperands g{(const uint8_t*)x_f8 + (int64_t)m0 * K, (const uint8_t*)w_f8_vk, K, K, Mc, V, K, 1};
         EpiDlStore epi{};
@@ -1374,16 +1513,6 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
             // 1'. the pass's dlogits panel from the forward's sigma codes; tiles with a sigma below the code window
             //     that matters (none, normally) are then redone from the logits
             ProfileScope prof(PROF_CE_DLOGITS, st);
-            const int nvt = (int)(Vp / 256), nflags = 2 + (Mt / 256) * nvt;
-            fill_f32_kernel<<<(nflags + 255) / 256, 256, 0, st>>>((float*)count, nflags, 0.0f);
-            // a sample of a few hundred tiles decides between the two ways, its stride coprime to the tiles per row so that
-            // the sample walks through all vocabulary columns; the recompute of 45 % of the tiles costs what the conversion does
-            const int nbx = V / 128, ntiles = (Mt / 256) * nvt;
-            int stride = std::max(1, ntiles / 300);
-            while (stride > 1 && std::gcd(stride, nvt) != 1) ++stride;
-            const int nsample = (ntiles + stride - 1) / stride;
-            const int limit = nsample * 45 / 100;
-            ce_codes_probe_kernel<<<nsample, 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, nbx, nvt, ntiles, stride, rowf, dcode, hits);
             ce_codes_to_dl_kernel<<<dim3(nbx, nkt), 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, rowf, dcode,
                                                                   nkt, dw_panel, nvt, flags, list, count, hits, limit);
             if (int e = check_launch("ce_codes_to_dl_kernel")) return e;
@@ -1392,7 +1521,6 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
             g.probe_hits = hits;
             g.probe_limit = limit;
             if (int e = launch_grid_kernel<MainCfg, TileListIter>(g, epi, st, -1, "lm_head CE backward (dlogits of the listed tiles)")) return e;
-            if (int e = launch_grid_kernel<MainCfg, CondGridIter>(g, epi, st, -1, "lm_head CE backward (dlogits, all tiles)")) return e;
         } else if (int e = launch_grid_kernel<MainCfg, GridIter>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
         ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, nkt, dw_panel);

@@ -55,14 +55,23 @@ struct GemmOperands {
     int layout;         // kBlockedA | kBlockedB | kRowsPermuted
     int full_tiles;     // the first full_tiles tiles (in walk order) are never split; 0 = `splits` applies to every tile
     int a_rows_pad;     // transposed A only: R rounded up to 256
-    // TileListIter only: the kernel works on the tiles tile_list[0 .. *tile_count) instead of on all of them
+    // TileListIter only: the kernel works on the tiles tile_list[0 .. *tile_count) instead of on all of them, unless the
+    // counts probe_hits[0 .. kProbeBlocks) that an earlier kernel wrote add up to more than probe_limit: then on all of them
     const int* tile_list;
     const int* tile_count;
-    // TileListIter / CondGridIter: a counter written by an earlier kernel decides which of the two walks does the work:
-    // the listed tiles while *probe_hits <= probe_limit, the whole grid otherwise (the other walk finds no job)
     const int* probe_hits;
     int probe_limit;
 };
+
+// Sum of the per-workgroup counts of a probe (written by an earlier kernel, hence read as scalar loads).
+constexpr int kProbeBlocks = 64;
+__device__ __forceinline__ int probe_total(const int* hits) {
+    const __attribute__((address_space(4))) int* h = (const __attribute__((address_space(4))) int*)(uintptr_t)hits;
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < kProbeBlocks; ++i) s += h[i];
+    return s;
+}
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BK_ = 128, int NSTAGES_ = 2, int WGS_PER_CU_ = 1>
 struct TileCfg {
@@ -624,31 +633,24 @@ struct GridIter {
 
 // GridIter over a list of tiles: tile_list[i] = (tile row << 16) | tile column, i < *tile_count (both written by an
 // earlier kernel and read through the constant address space, i.e. as scalar loads that stay out of the vector memory
-// counter).  The base class walks a 1 x count grid; its column index is the position in the list.
+// counter); the base class then walks a 1 x count grid and its column index is the position in the list.  If the probe
+// counts say so (GemmOperands::probe_hits) the walk covers the whole grid instead.
 struct TileListIter : GridIter {
     const int* list;
-    static __device__ bool whole_grid(const GemmOperands& g) {
-        return ((const __attribute__((address_space(4))) int*)(uintptr_t)g.probe_hits)[0] > g.probe_limit;
-    }
+    bool whole;
+    static __device__ bool whole_grid(const GemmOperands& g) { return probe_total(g.probe_hits) > g.probe_limit; }
     static __device__ GemmOperands listed(GemmOperands g, int BM, int BN) {
-        g.R = BM;
-        g.C = whole_grid(g) ? 0 : ((const __attribute__((address_space(4))) int*)(uintptr_t)g.tile_count)[0] * BN;
+        if (!whole_grid(g)) {
+            g.R = BM;
+            g.C = ((const __attribute__((address_space(4))) int*)(uintptr_t)g.tile_count)[0] * BN;
+        }
         return g;
     }
     __device__ TileListIter(const GemmOperands& g, int BM, int BN, int bid_, int G_)
-        : GridIter(listed(g, BM, BN), BM, BN, bid_, G_), list(g.tile_list) {}
+        : GridIter(listed(g, BM, BN), BM, BN, bid_, G_), list(g.tile_list), whole(whole_grid(g)) {}
     __device__ int entry() const { return ((const __attribute__((address_space(4))) int*)(uintptr_t)list)[tc_]; }
-    __device__ int tr() const { return entry() >> 16; }
-    __device__ int tc() const { return entry() & 0xffff; }
-};
-
-// GridIter that walks the whole grid if the probe counter says so and nothing otherwise (see GemmOperands::probe_hits).
-struct CondGridIter : GridIter {
-    static __device__ GemmOperands cond(GemmOperands g) {
-        if (!TileListIter::whole_grid(g)) g.R = 0;
-        return g;
-    }
-    __device__ CondGridIter(const GemmOperands& g, int BM, int BN, int bid_, int G_) : GridIter(cond(g), BM, BN, bid_, G_) {}
+    __device__ int tr() const { return whole ? tr_ : entry() >> 16; }
+    __device__ int tc() const { return whole ? tc_ : entry() & 0xffff; }
 };
 
 // The generic persistent kernel.  `Iter` walks the tiles of this workgroup (see GridIter).  `Epi` supplies
@@ -733,7 +735,7 @@ __global__ __launch_bounds__(Cfg::THREADS, Cfg::WGS_PER_CU) void gemm_tn_kernel(
     Iter cur(g, Cfg::BM, Cfg::BN, bid, G);
     // a walk over listed tiles usually has no job at all: leave before the epilogue's set-up (other walks go on, their
     // epilogues may have something to write for a workgroup without work)
-    if constexpr (std::is_same<Iter, TileListIter>::value || std::is_same<Iter, CondGridIter>::value) { if (!cur.valid()) return; }
+    if constexpr (std::is_same<Iter, TileListIter>::value) { if (!cur.valid()) return; }
 
     // `pre` walks the (job, k-step) sequence of this workgroup ahead of the MFMAs; `ahead` counts the
     // k-steps whose operand loads have been issued and not yet consumed (at most one per slot).

@@ -41,13 +41,13 @@ __device__ __forceinline__ void transpose4x4_bytes(uint32_t (&r)[4]) {
 // the transposing reads below conflict-free.  A thread then owns 4 columns x 16 rows: four 4 x 4 byte
 // blocks, transposed in registers, are the four words of one 16-byte piece of each column's panel row;
 // the 8 threads that share a column group are adjacent lanes, so they write whole 128-byte rows.
+// The work of one workgroup of 256 threads: column group cg, k-step kt (also called by kernels that do several jobs in one launch).
 template <int PERM, int QFMT>
-__global__ __launch_bounds__(256) void panel_transpose_kernel(const uint8_t* __restrict__ in, int64_t ld, int row0, int nrows, int cols,
-                                                              int nk, float scale, uint8_t* __restrict__ out) {
+__device__ __forceinline__ void panel_transpose_block(const uint8_t* __restrict__ in, int64_t ld, int row0, int nrows, int cols,
+                                                      int nk, float scale, uint8_t* __restrict__ out, int cg, int kt) {
     constexpr int kStride = 33;
     __shared__ uint32_t tile[128 * kStride];
-    // neighbouring workgroups take neighbouring column groups of the same rows: together they read whole rows
-    const int cg = blockIdx.x, kt = blockIdx.y, tid = threadIdx.x;
+    const int tid = threadIdx.x;
     auto word_at = [&](int r, int w) -> uint32_t& { return tile[r * kStride + (w ^ (((r >> 4) & 7) << 2))]; };
     if (QFMT == kPanelRaw) {
 #pragma unroll
@@ -90,6 +90,13 @@ __global__ __launch_bounds__(256) void panel_transpose_kernel(const uint8_t* __r
         if (col < cols)
             *(v4i*)(out + panel_offset(col, kt * 128, nk) + sub * 16) = (v4i){(int)w[0][c], (int)w[1][c], (int)w[2][c], (int)w[3][c]};
     }
+}
+
+template <int PERM, int QFMT>
+__global__ __launch_bounds__(256) void panel_transpose_kernel(const uint8_t* __restrict__ in, int64_t ld, int row0, int nrows, int cols,
+                                                              int nk, float scale, uint8_t* __restrict__ out) {
+    // neighbouring workgroups take neighbouring column groups of the same rows: together they read whole rows
+    panel_transpose_block<PERM, QFMT>(in, ld, row0, nrows, cols, nk, scale, out, blockIdx.x, blockIdx.y);
 }
 
 template <int PERM, int QFMT = kPanelRaw>

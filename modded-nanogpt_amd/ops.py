@@ -235,7 +235,7 @@ def lmhead_ce_fwd(x: Tensor, w: Tensor, targets: Tensor, mtp_weights: Tensor, pr
     dev = x.device
     losses = torch.empty(M, dtype=torch.float32, device=dev)
     lse = torch.empty(M, dtype=torch.float32, device=dev)
-    saved_sigma = torch.zeros((MAX_PREDICT + 1, M), dtype=torch.float32, device=dev)
+    saved_sigma = torch.empty((MAX_PREDICT + 1, M), dtype=torch.float32, device=dev)     # zeroed by the library
     x_f8 = torch.empty((M, K), dtype=E4M3, device=dev)
     w_f8 = torch.empty((V, K), dtype=E4M3, device=dev)
     layout = _lib.W_IN_OUT if w_in_out else _lib.W_OUT_IN
@@ -308,7 +308,7 @@ def lmhead_ce_fwd_codes(x: Tensor, w: Tensor, targets: Tensor, mtp_weights: Tens
     dev = x.device
     losses = torch.empty(M, dtype=torch.float32, device=dev)
     lse = torch.empty(M, dtype=torch.float32, device=dev)
-    saved_sigma = torch.zeros((MAX_PREDICT + 1, M), dtype=torch.float32, device=dev)
+    saved_sigma = torch.empty((MAX_PREDICT + 1, M), dtype=torch.float32, device=dev)     # zeroed by the library
     x_f8 = torch.empty((M, K), dtype=E4M3, device=dev)
     w_f8 = torch.empty((V, K), dtype=E4M3, device=dev)
     codes = torch.empty(lib.ngpt_lmhead_ce_codes_bytes(M, V), dtype=torch.uint8, device=dev)
