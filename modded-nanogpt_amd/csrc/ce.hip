@@ -849,7 +849,8 @@ __device__ __forceinline__ bool code_needs_logit(uint32_t w, float rf, float d_b
 
 // Everything the backward needs before its first large kernel, in one launch of 256-thread workgroups; block ranges, in
 // this order (a range may be empty): the table of the gradient factor; the code table; the row factors of all rows;
-// zeros for the pass's tile list state; W^T as a panel; the pass's x^T as a panel; the probe of the pass's codes.
+// zeros for the pass's tile list state; W^T as a panel; the pass's x^T as a panel; the weights in the token-stationary
+// kernel's fragment order; the probe of the pass's codes.
 //
 // The probe looks at every `stride`-th 256 x 256 tile of the pass's codes and counts those that the conversion would
 // put on the list.  If more than a given share of the sample is, the conversion is skipped and the whole panel
@@ -874,7 +875,8 @@ struct BwdPrepArgs {
     const uint8_t* codes;
     int nkp, nbx, nvt, stride, nsample;
     int* hits;
-    int b_tab, b_dcode, b_rowf, b_zero, b_wt, b_xt;      // workgroups of each range; the probe takes the rest
+    uint8_t* w_frag;
+    int b_tab, b_dcode, b_rowf, b_zero, b_wt, b_xt, b_frag;      // workgroups of each range; the probe takes the rest
 };
 
 __device__ __forceinline__ void ce_codes_probe_block(const BwdPrepArgs& p, int b) {
@@ -926,6 +928,8 @@ __global__ __launch_bounds__(256) void ce_bwd_prep_kernel(BwdPrepArgs p) {
     b -= p.b_wt;
     if (b < p.b_xt) { panel_transpose_block<2, kPanelRaw>(p.x_f8, p.K, p.m0, p.Mc, p.K, p.nkt, 1.0f, p.x_t, b % ncg, b / ncg); return; }
     b -= p.b_xt;
+    if (b < p.b_frag) { xs_frag_from_f8(p.w_f8, p.V, p.K, p.w_frag, b, p.b_frag); return; }
+    b -= p.b_frag;
     ce_codes_probe_block(p, b);
 }
 
@@ -1082,9 +1086,9 @@ static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwdT<CODES>& epi, hip
 // The token-stationary forward (ce_fwd_xs.h) covers V % 64 == 0, K % 256 == 0, K <= XS_MAX_K; other shapes take the tile kernel.
 static bool xs_eligible(int M, int K, int V) { return M > 0 && V % XS_UNIT == 0 && (K == 256 || K == 512 || K == 768 || K == 1024); }
 
-template <bool CODES, int NS>
+template <int MODE, int NS>
 static int launch_ce_fwd_xs(XsArgs a, hipStream_t st) {
-    auto kernel = ce_fwd_xs_kernel<CODES, NS>;
+    auto kernel = ce_fwd_xs_kernel<MODE, NS>;
     const int LDS = XS_CAND_LDS + a.K * XS_TOK;      // dynamic part; the table is static LDS
     static PerDeviceOnce configured;
     if (int e = configured.run([&] { return allow_lds(kernel, XS_CAND_LDS + XS_MAX_K * XS_TOK); })) return e;
@@ -1092,7 +1096,8 @@ static int launch_ce_fwd_xs(XsArgs a, hipStream_t st) {
     if (cus < CE_XCDS) return fail(NGPT_EINVAL, "lm_head CE forward: no HIP device (or fewer than %d compute units)", CE_XCDS);
     // workgroups per XCD = token tiles in flight (mg) x vocabulary shares (splits); the split count that needs the
     // fewest unit-steps per workgroup wins, the smaller one on a tie (longer jobs, fewer slab loads)
-    const int per_xcd_slots = cus / CE_XCDS, tiles_m = (a.M + XS_TOK - 1) / XS_TOK, per_xcd = (tiles_m + CE_XCDS - 1) / CE_XCDS;
+    if (a.tiles_m <= 0) a.tiles_m = (a.M + XS_TOK - 1) / XS_TOK;
+    const int per_xcd_slots = cus / CE_XCDS, tiles_m = a.tiles_m, per_xcd = (tiles_m + CE_XCDS - 1) / CE_XCDS;
     const int units = a.V / XS_UNIT;
     int best_splits = 1, best_mg = 1;
     int64_t best_cost = -1;
@@ -1105,10 +1110,10 @@ static int launch_ce_fwd_xs(XsArgs a, hipStream_t st) {
     }
     a.splits = best_splits;
     {
-        ProfileScope prof(PROF_CE_FWD, st);
+        ProfileScope prof(MODE == XS_DL ? PROF_CE_DLOGITS : PROF_CE_FWD, st);
         kernel<<<CE_XCDS * best_splits * best_mg, XS_THREADS, LDS, st>>>(a);
     }
-    return check_launch("lm_head CE forward (token-stationary)");
+    return check_launch(MODE == XS_DL ? "lm_head CE backward (dlogits, token-stationary)" : "lm_head CE forward (token-stationary)");
 }
 
 template <class Cfg, class Iter, class Epi>
@@ -1325,10 +1330,10 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
         a.ncand = prefix_targets ? n_predict + 1 : n_predict;
         int e = NGPT_EINVAL;
         switch (K / 64) {   // the contraction loop is unrolled completely: one instantiation per supported K
-            case 4: e = sigma_codes ? launch_ce_fwd_xs<true, 4>(a, st) : launch_ce_fwd_xs<false, 4>(a, st); break;
-            case 8: e = sigma_codes ? launch_ce_fwd_xs<true, 8>(a, st) : launch_ce_fwd_xs<false, 8>(a, st); break;
-            case 12: e = sigma_codes ? launch_ce_fwd_xs<true, 12>(a, st) : launch_ce_fwd_xs<false, 12>(a, st); break;
-            case 16: e = sigma_codes ? launch_ce_fwd_xs<true, 16>(a, st) : launch_ce_fwd_xs<false, 16>(a, st); break;
+            case 4: e = sigma_codes ? launch_ce_fwd_xs<XS_FWD_CODES, 4>(a, st) : launch_ce_fwd_xs<XS_FWD, 4>(a, st); break;
+            case 8: e = sigma_codes ? launch_ce_fwd_xs<XS_FWD_CODES, 8>(a, st) : launch_ce_fwd_xs<XS_FWD, 8>(a, st); break;
+            case 12: e = sigma_codes ? launch_ce_fwd_xs<XS_FWD_CODES, 12>(a, st) : launch_ce_fwd_xs<XS_FWD, 12>(a, st); break;
+            case 16: e = sigma_codes ? launch_ce_fwd_xs<XS_FWD_CODES, 16>(a, st) : launch_ce_fwd_xs<XS_FWD, 16>(a, st); break;
         }
         if (e) return e;
     } else if (sigma_codes) {
@@ -1410,7 +1415,8 @@ static int64_t flag_bytes(int64_t Mt, int64_t Vp) { return align_up((kProbeBlock
 extern "C" int64_t ngpt_lmhead_ce_bwd_workspace_bytes(int M, int K, int V, int w_layout) {
     (void)w_layout;
     int64_t Mc = bwd_chunk_rows(M), Mt = round256(Mc), Kp = round256(K), Vp = round256(V);
-    return align_up(2 * TAB_BYTES, 256) + 2 * round256(M) * 4 + Kp * Mt + Kp * (int64_t)V + Vp * Mt + bwd_part_bytes(Mc, Mt, K, V) + flag_bytes(Mt, Vp);
+    return align_up(2 * TAB_BYTES, 256) + 2 * round256(M) * 4 + Kp * Mt + Kp * (int64_t)V + Vp * Mt + bwd_part_bytes(Mc, Mt, K, V) + flag_bytes(Mt, Vp) +
+           (xs_eligible(M, K, V) ? align_up(xs_frag_bytes(V, K), 256) : 0);
 }
 
 extern "C" int64_t ngpt_lmhead_ce_codes_bytes(int M, int V) { return round256(M) * round256(V); }
@@ -1457,6 +1463,11 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
     int* count = hits + kProbeBlocks;        // number of listed tiles
     int* flags = count + 1;                  // per 256 x 256 tile of the pass's logits: a sigma of it lies below the code window and matters
     int* list = flags + (Mt_max / 256) * (Vp / 256);
+    ws += flag_bytes(Mt_max, Vp);
+    // the recompute of the logits runs on the token-stationary kernel where that covers the shape; it reads the weights
+    // in fragment order
+    const bool dl_xs = !sigma_codes && xs_eligible(M, K, V);
+    uint8_t* w_frag = ws;
     static_assert(BWD_CHUNK_ROWS / 256 < 65536, "a list entry holds the token tile in its upper 16 bits");
     if (Vp / 256 >= 65536) return fail(NGPT_ERANGE, "%s: V=%d", who, V);
 
@@ -1494,8 +1505,10 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
             a.b_zero = sigma_codes ? (a.nzero + 255) / 256 : 0;
             a.b_wt = first ? ncg * nkv : 0;
             a.b_xt = ncg * nkt;
+            a.w_frag = w_frag;
+            a.b_frag = (first && dl_xs) ? std::min((V / XS_UNIT) * (K / 128), 4 * num_cus()) : 0;
             const int b_probe = sigma_codes ? kProbeBlocks : 0;
-            ce_bwd_prep_kernel<<<a.b_tab + a.b_dcode + a.b_rowf + a.b_zero + a.b_wt + a.b_xt + b_probe, 256, 0, st>>>(a);
+            ce_bwd_prep_kernel<<<a.b_tab + a.b_dcode + a.b_rowf + a.b_zero + a.b_wt + a.b_xt + a.b_frag + b_probe, 256, 0, st>>>(a);
             if (int e = check_launch("ce_bwd_prep_kernel")) return e;
         }
         // 1. recompute the pass's logits and turn them into the e5m2 dlogits panel
@@ -1521,6 +1534,27 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
             g.probe_hits = hits;
             g.probe_limit = limit;
             if (int e = launch_grid_kernel<MainCfg, TileListIter>(g, epi, st, -1, "lm_head CE backward (dlogits of the listed tiles)")) return e;
+        } else if (dl_xs) {
+            XsArgs a{};
+            a.w_frag = w_frag;
+            a.x_f8 = (const uint8_t*)x_f8 + (int64_t)m0 * K;
+            a.M = Mc; a.V = V; a.K = K;
+            a.tiles_m = nkt;                   // every 128-token k-step of the panel, the padding's zeros included
+            a.gtabE = tabD;
+            a.sc = sc;
+            a.scale = x_s * w_s;
+            a.rowf = rowf + m0;
+            a.big = big + (m0 >> 8);
+            a.dl_panel = dw_panel;
+            a.nkt = nkt;
+            int e = NGPT_EINVAL;
+            switch (K / 64) {
+                case 4: e = launch_ce_fwd_xs<XS_DL, 4>(a, st); break;
+                case 8: e = launch_ce_fwd_xs<XS_DL, 8>(a, st); break;
+                case 12: e = launch_ce_fwd_xs<XS_DL, 12>(a, st); break;
+                case 16: e = launch_ce_fwd_xs<XS_DL, 16>(a, st); break;
+            }
+            if (e) return e;
         } else if (int e = launch_grid_kernel<MainCfg, GridIter>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;
         // 2. exact gradient at the target columns
         ce_dl_fix_kernel<<<(Mc + 255) / 256, 256, 0, st>>>(lse, saved_sigma, ca, sc, coef, m0, Mc, nkt, dw_panel);

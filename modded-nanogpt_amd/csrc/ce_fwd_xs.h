@@ -1,6 +1,7 @@
-// Fused lm_head + softcapped CE forward, token-stationary variant (included by ce.hip).
+// Fused lm_head + softcapped CE, token-stationary kernel (included by ce.hip): the forward (XS_FWD, XS_FWD_CODES) and the
+// backward's logits recompute that writes the e5m2 gradient panel (XS_DL).
 //
-// Same arithmetic as EpiCEFwdT on gemm_tn_kernel (rows = vocabulary, columns = tokens, 32x32x64 fp8 MFMAs over the
+// Same arithmetic as EpiCEFwdT / EpiDlStore on gemm_tn_kernel (rows = vocabulary, columns = tokens, 32x32x64 fp8 MFMAs over the
 // contraction in ascending order, softcap through the bf16-indexed table), different data movement:
 //   * a job = 128 tokens x one share of the vocabulary.  The tokens' fp8 activations (128 x K bytes) are loaded into
 //     LDS ONCE per job and stay there; only the weights stream.
@@ -8,9 +9,9 @@
 //     a time (a "unit": 2 x 4 MFMA tiles, 128 accumulator registers) and reads the weights of ITS rows straight from
 //     global memory into MFMA operand registers, a few steps ahead of their use -- no other wave needs them, so they
 //     never pass through LDS and the contraction loop has no workgroup barrier at all.
-//   * the two waves that share a SIMD are started half a unit apart: while one of them runs the table epilogue of its
-//     unit on the vector pipe and the LDS gather path, the other one feeds the matrix pipe, which an eight-wave
-//     lockstep tile leaves idle for the whole epilogue.
+//   * nothing keeps the two waves that share a SIMD in step, and the one in its contraction loop has the higher
+//     priority: while one of them runs the table epilogue of its unit on the vector pipe and the LDS gather path, the
+//     other one feeds the matrix pipe, which an eight-wave lockstep tile leaves idle for the whole epilogue.
 //
 // Weights are read in "fragment-major" order, written by the quantiser next to the row-major fp8 copy:
 //   [V / 64 units][K / 64 steps][2 row blocks][2 parts][64 lanes][16 bytes]
@@ -34,10 +35,13 @@ constexpr int XS_MAX_SPLITS = CE_SPLITS;    // part[] has CE_SPLITS slots per to
 
 __host__ __device__ inline int64_t xs_frag_bytes(int V, int K) { return (int64_t)V * K; }
 
+enum { XS_FWD = 0, XS_FWD_CODES = 1, XS_DL = 2 };
+
 struct XsArgs {
     const uint8_t* w_frag;   // fragment-major weights
     const uint8_t* x_f8;     // [M, K] row-major
     int M, V, K;
+    int tiles_m;             // 128-token tiles to walk: M / 128 rounded up (XS_DL: up to the panel's token padding)
     int splits;              // vocabulary shares per token tile (<= XS_MAX_SPLITS)
     uint8_t* codes;          // CODES: code panel (see EpiCEFwdT)
     int nkp;
@@ -48,10 +52,16 @@ struct XsArgs {
     Softcap sc;
     float scale;
     int ncand;
+    // XS_DL (gtabE then is the table of the gradient factor): see EpiDlStore
+    const float* rowf;       // row factors, zero past the last token up to the panel's padding
+    const int* big;          // per 256 tokens: a product may leave the e5m2 range
+    uint8_t* dl_panel;       // [V / 256 rounded up][nkt] blocks of 256 vocabulary rows x 128 tokens
+    int nkt;
 };
 
-template <bool CODES, int NS /* K / 64 */>
+template <int MODE, int NS /* K / 64 */>
 __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
+    constexpr bool CODES = MODE == XS_FWD_CODES, DL = MODE == XS_DL;
     // weight fragment sets in registers (loads run XS_RING - 1 steps ahead); must divide the number of steps
     constexpr int XS_RING = 4;
     static_assert(NS % XS_RING == 0, "ring slots of a unit's first steps");
@@ -68,7 +78,7 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
 
     // job walk: XCD x owns a contiguous block of token tiles, mg of them in flight, each shared by `splits` workgroups
     const int bid = blockIdx.x, G = gridDim.x;
-    const int tiles_m = (M + XS_TOK - 1) / XS_TOK, units = p.V / XS_UNIT;
+    const int tiles_m = p.tiles_m, units = p.V / XS_UNIT;
     const int xcd = bid % CE_XCDS, slot = bid / CE_XCDS;
     const int mg = max(G / (CE_XCDS * p.splits), 1);
     const int per_xcd = (tiles_m + CE_XCDS - 1) / CE_XCDS;
@@ -93,18 +103,24 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
             for (int li = 0; li < 2; ++li) {
                 const int ld = 2 * wave + li, row = ld * 8 + (lane >> 3);
                 const int q = (lane & 7) ^ ((row >> 1) & 7);
-                const uint8_t* src = p.x_f8 + (int64_t)(c0 + min(row, M - 1 - c0)) * K + q * 16;
+                const uint8_t* src = p.x_f8 + (int64_t)min(c0 + row, M - 1) * K + q * 16;
                 const uint32_t dst = xs_addr + (uint32_t)(ld * 1024 + lane * 16);
 #pragma unroll
                 for (int kc = 0; kc < NS / 2; ++kc) *(lds_w4)(uintptr_t)(dst + kc * 16384) = *(const v4i*)(src + kc * 128);
             }
-            for (int i = tid; i < p.ncand * XS_TOK; i += XS_THREADS) {
-                const int c = i / XS_TOK, jj = i % XS_TOK, m = c0 + jj;
-                const int64_t t = (m < M) ? cand_target(p.ca, m, c) : -1;
-                cand[c * XS_TOK + jj] = (t >= 0 && t < p.ca.V) ? (int)t : -1;
+            if constexpr (DL) {
+                if (tid < XS_TOK) ((float*)cand)[tid] = p.rowf[c0 + tid];
+            } else {
+                for (int i = tid; i < p.ncand * XS_TOK; i += XS_THREADS) {
+                    const int c = i / XS_TOK, jj = i % XS_TOK, m = c0 + jj;
+                    const int64_t t = (m < M) ? cand_target(p.ca, m, c) : -1;
+                    cand[c * XS_TOK + jj] = (t >= 0 && t < p.ca.V) ? (int)t : -1;
+                }
             }
             wg_barrier();
         }
+        int job_big = 0;
+        if constexpr (DL) job_big = ((const __attribute__((address_space(4))) int*)(uintptr_t)p.big)[c0 >> 8];
 
         float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         v16f acc[2][4];
@@ -181,16 +197,73 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
 #pragma unroll
                 for (int tm = 0; tm < 2; ++tm) {
                     const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                    acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                        a[ks % XS_RING][tm], b[pr % (XS_BDEPTH + 1)], ks == 0 ? zero : acc[tm][tn], 0, 0, 0, 0, 0, 0);
+                    // XS_DL: operands swapped, so that a lane owns a vocabulary row and its registers hold tokens
+                    if constexpr (DL)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            b[pr % (XS_BDEPTH + 1)], a[ks % XS_RING][tm], ks == 0 ? zero : acc[tm][tn], 0, 0, 0, 0, 0, 0);
+                    else
+                        acc[tm][tn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            a[ks % XS_RING][tm], b[pr % (XS_BDEPTH + 1)], ks == 0 ? zero : acc[tm][tn], 0, 0, 0, 0, 0, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_s_setprio(0);
 
-            // ---- epilogue of the unit: softcap table, sum of exponentials, sigma codes (as EpiCEFwdT::tile)
             const int el = fresh_lane();
             const int j = el & 31, h = el >> 5;
+            if constexpr (DL) {
+                // ---- epilogue of the unit: dl = e5m2_sat(rowf[token] * D(logit)) into the panel (as EpiDlStore::tile).  A lane
+                // owns vocabulary row 32 tm + j of the unit; registers 4 g ..+3 of acc[tm][tn] are the tokens
+                // 32 tn + 8 g + 4 h ..+3, i.e. the four bytes at position 16 h + 4 g of token group tn of that row.
+                uint8_t* dl_base = p.dl_panel + ((int64_t)(u >> 2) * p.nkt + (c0 >> 7)) * kPanelBytes + (u & 3) * (XS_UNIT * 128);
+                const uint32_t dl_lane = (uint32_t)(j * 128 + 16 * h);
+                const uint32_t rf_addr = (uint32_t)(size_t)((const __attribute__((address_space(3))) uint8_t*)cand) + 16 * h;
+                auto run = [&](auto sat) {
+                    constexpr bool SAT = decltype(sat)::value;
+                    constexpr int NB = 16;      // batch b: token block b / 4, register group b % 4, both vocabulary blocks
+                    uint32_t pk[2][4];
+                    float pv[8], nv[8];
+                    v4f prf, nrf;
+#pragma unroll
+                    for (int b = 0; b <= NB; ++b) {
+                        if (b < NB) {
+                            const int tn = b >> 2, g = b & 3;
+                            uint32_t off[4];
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) {
+                                const v16f& r = acc[k >> 1][tn];
+                                off[k] = tab_offsets2(pack_logits(r[4 * g + 2 * (k & 1)] * p.scale, r[4 * g + 2 * (k & 1) + 1] * p.scale));
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                            nrf = *(const __attribute__((address_space(3))) v4f*)(uintptr_t)(rf_addr + (32 * tn + 8 * g) * 4);
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) {
+                                nv[2 * k] = tab_at(tab, off[k] & 0xffffu);
+                                nv[2 * k + 1] = tab_at(tab, off[k] >> 16);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        if (b > 0) {
+                            const int q = b - 1, tn = q >> 2, g = q & 3;
+                            pk[0][g] = f32x4_to_e5m2_sat<SAT>(prf[0] * pv[0], prf[1] * pv[1], prf[2] * pv[2], prf[3] * pv[3]);
+                            pk[1][g] = f32x4_to_e5m2_sat<SAT>(prf[0] * pv[4], prf[1] * pv[5], prf[2] * pv[6], prf[3] * pv[7]);
+                            if (g == 3) {
+#pragma unroll
+                                for (int tm = 0; tm < 2; ++tm)
+                                    *(v4i*)(dl_base + (dl_lane + tm * 4096 + tn * 32)) =
+                                        (v4i){(int)pk[tm][0], (int)pk[tm][1], (int)pk[tm][2], (int)pk[tm][3]};
+                            }
+                        }
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) pv[k] = nv[k];
+                        prf = nrf;
+                    }
+                };
+                if (job_big) run(std::true_type{});
+                else run(std::false_type{});
+                continue;
+            }
+            // ---- epilogue of the unit: softcap table, sum of exponentials, sigma codes (as EpiCEFwdT::tile)
             // code panel (layout: EpiCEFwdT): row = this lane's token, 16 bytes = the 16 vocabulary rows of one (tm, lane half) group
             uint8_t* cd_base = nullptr;
             uint32_t cd_lane = 0;
@@ -269,6 +342,7 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
             }
         }
 
+        if constexpr (DL) continue;
         // ---- job end: the lanes' sums -> part[split][token]
         wg_barrier();                                  // every wave is done reading the slab: it becomes scratch
         float* red = (float*)xslab;                    // [XS_WAVES][XS_TOK]
@@ -290,9 +364,9 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
 
 // Fragment-major copy of the weights (layout at the top of this file) from the row-major fp8 matrix [V, K]:
 // one workgroup iteration moves 64 rows x 128 contraction bytes = 8 KiB, consecutive in both layouts' units.
-__global__ __launch_bounds__(256) void xs_frag_from_f8_kernel(const uint8_t* __restrict__ w_f8, int V, int K, uint8_t* __restrict__ w_frag) {
+__device__ __forceinline__ void xs_frag_from_f8(const uint8_t* __restrict__ w_f8, int V, int K, uint8_t* __restrict__ w_frag, int block, int nblocks) {
     const int nkc = K / 128, items = (V / XS_UNIT) * nkc;
-    for (int it = blockIdx.x; it < items; it += gridDim.x) {
+    for (int it = block; it < items; it += nblocks) {
         const int u = it / nkc, kc = it % nkc;
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
@@ -302,6 +376,9 @@ __global__ __launch_bounds__(256) void xs_frag_from_f8_kernel(const uint8_t* __r
             *(v4i*)(w_frag + (((int64_t)u * (K / 64) + ks) * 4 + tm * 2 + part) * 1024 + (hh * 32 + i) * 16) = v;
         }
     }
+}
+__global__ __launch_bounds__(256) void xs_frag_from_f8_kernel(const uint8_t* __restrict__ w_f8, int V, int K, uint8_t* __restrict__ w_frag) {
+    xs_frag_from_f8(w_f8, V, K, w_frag, blockIdx.x, gridDim.x);
 }
 
 }  // namespace ngpt
