@@ -4,41 +4,6 @@
 
 namespace ngpt {
 
-// ---------------------------------------------------------------------------------------------
-// Staged byte stores.  An fp8 result tile cannot be written straight from the MFMA register
-// layout (a lane owns one column and scattered rows: 1-byte or 4-byte pieces per row), so the
-// wave parks a strip in its private LDS scratch and writes it back out in 16-byte pieces.
-
-// Strip = 32 rows x WTN columns of bytes in the wave's LDS scratch, rows padded where the scratch allows it
-// (fewer bank conflicts on the 16-byte reads).
-template <class Cfg>
-struct StripU8 {
-    static constexpr int STRIDE = (32 * (Cfg::WTN + 16) <= Cfg::WAVE_SCRATCH) ? Cfg::WTN + 16 : Cfg::WTN;
-    static_assert(32 * STRIDE <= Cfg::WAVE_SCRATCH, "strip does not fit the wave's LDS scratch");
-    // byte of accumulator element (tn, v) of the strip's tm
-    static __device__ __forceinline__ void put(uint8_t* scratch, int lane, int tn, int v, uint32_t code) {
-        const int rl = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        scratch[rl * STRIDE + tn * 32 + (lane & 31)] = (uint8_t)code;
-    }
-};
-// The strip, complete in LDS, to global memory: row-major with leading dimension ld, 16 bytes per lane.
-template <class Cfg>
-__device__ __forceinline__ void strip_flush_rowmajor_u8(uint8_t* scratch, int lane, uint8_t* out, int64_t ld,
-                                                        int grow0 /* global row of strip row 0 */, int gcol0, int R, int C) {
-    constexpr int STRIDE = StripU8<Cfg>::STRIDE;
-    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the wave's own LDS writes have landed
-    constexpr int CH_PER_ROW = Cfg::WTN / 16;
-#pragma unroll
-    for (int p = 0; p < Cfg::WTN / 32; ++p) {
-        int id = p * 64 + lane;
-        int rl = id / CH_PER_ROW, ch = id % CH_PER_ROW;
-        v4i val = *(const v4i*)(scratch + rl * STRIDE + ch * 16);
-        int gr = grow0 + rl, gc = gcol0 + ch * 16;
-        if (gr < R && gc + 16 <= C) *(v4i*)(out + (int64_t)gr * ld + gc) = val;
-    }
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-}
-
 // acc * scale into an fp32 matrix: plain stores, or fire-and-forget L2 atomics (no read-modify-write
 // through registers) when `atomic`.  Shared by the fp32 output and by partial tiles of a split contraction.
 template <class Cfg>
@@ -306,139 +271,44 @@ struct EpiStoreF32 {
 // columns = tokens, post [tokens, hidden] row-major): a lane's four consecutive accumulator registers are
 // four consecutive hidden units of one token.  Every 32-token x 64-hidden block (4 KiB) is collected in the
 // wave's LDS region and written as whole 128-byte lines, 16 bytes per lane (see EpiDpre).  R % 8 == 0.
-struct EpiRelu2Lines {
+// EMIT (R % 16 == 0): also post_f8 = e4m3(min(post / act_scale, 448)), row-major like post, and the largest post of
+// every workgroup in partial_amax[workgroup] (zeros in the slots past the grid).  The e4m3 block of 32 tokens x 64
+// bytes takes the same LDS region after the bf16 lines have been read out of it (80-byte rows: the four-byte
+// writes of 32 lanes then meet at most two per bank) and leaves as 16-byte pieces, 64 bytes per token.  Rows and
+// columns past the matrix edge are copies of the last valid ones (the operand loads clamp), so the maximum needs no mask.
+template <bool EMIT>
+struct EpiRelu2LinesT {
     uint16_t* post;
     int64_t ld;
     const float* dequant;        // 1-element device tensor, or null for a scale of one (bf16 operands)
     int R, C;                    // R = hidden units (tile rows), C = tokens (tile columns)
+    uint8_t* post_f8;            // EMIT
+    int64_t ld_f8;
+    const float* act_scale;      // EMIT: 1-element device tensor
+    float* partial_amax;         // EMIT: n_partials entries, nullable
+    int n_partials;
     static constexpr int EXTRA_LDS = 32768;
     static constexpr bool NEEDS_SCRATCH = false;
     static constexpr bool JOB_END_NEEDS_SCRATCH = false;
-    static constexpr int TILE_STORES = 16;
-    float scale;
+    static constexpr int TILE_STORES = EMIT ? 24 : 16;
+    static constexpr int F8_STRIDE = 80;
+    float scale, inv_act;
+    uint32_t amax2;              // EMIT: running maximum of the bf16 patterns of post (all >= 0), two lanes of 16 bits
     uint8_t* stage;
     bool stored_all;
     __device__ bool all_stores_issued() const { return stored_all; }
     __device__ void partial(bool, int) {}
     __device__ void begin(int, int, uint8_t* extra) {
         scale = dequant ? *dequant : 1.0f;
+        inv_act = EMIT ? 1.0f / *act_scale : 0.0f;
+        amax2 = 0u;
         stage = extra + (threadIdx.x >> 6) * 4096;
         stored_all = false;
     }
-    __device__ void end(uint8_t*, int, int) {}
-    template <class Cfg>
-    __device__ void job_begin(int) {}
-    template <class Cfg>
-    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
-    template <class Cfg>
-    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co, uint8_t*, int lane) {
-        static_assert(Cfg::TM == 2 && Cfg::TN == 4 && Cfg::NWAVES * 4096 <= EXTRA_LDS, "64 x 128 wave tiles, 4 KiB of staging each");
-        const int h = lane >> 5, j = lane & 31;
-        const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
-        stored_all = full;
-        const int rd_row = lane >> 3, rd_chunk = lane & 7;
-        const int n = r0 + co.wave_row0 + rd_chunk * 8;
-        // address = wave-uniform pointer (tile origin + the block's and line group's fixed position) + ONE per-lane offset
-        uint16_t* origin = post + ((int64_t)c0 * ld + r0);
-        const uint32_t lane_off = (uint32_t)(co.wave_col0 + rd_row) * (uint32_t)ld + (uint32_t)(co.wave_row0 + rd_chunk * 8);
-        // relu(bf16(x)) == bf16(relu(x)) (rounding keeps the sign, a NaN becomes 0 either way): the maximum is taken on
-        // the product, which spares the canonicalising pass that a maximum on re-expanded bf16 bits needs
-        auto relu2 = [&](float a0, float a1) {
-            const uint32_t pre = cvt_pk_bf16(fmaxf(a0 * scale, 0.0f), fmaxf(a1 * scale, 0.0f));
-            const float c0f = __uint_as_float(pre << 16), c1f = __uint_as_float(pre & 0xffff0000u);
-            return (int)cvt_pk_bf16(c0f * c0f, c1f * c1f);
-        };
-#pragma unroll
-        for (int tn = 0; tn < Cfg::TN; ++tn) {
-#pragma unroll
-            for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const v16f& a = acc[tm][tn];
-                    *(v2i*)(stage + j * 128 + (((tm * 4 + g) ^ (j & 7)) << 4) + 8 * h) =
-                        (v2i){relu2(a[4 * g], a[4 * g + 1]), relu2(a[4 * g + 2], a[4 * g + 3])};
-                    if (g & 1) __builtin_amdgcn_sched_barrier(0);   // keep the arithmetic next to its LDS write (registers)
-                }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int row = 8 * k + rd_row;
-                const v4i v = *(const v4i*)(stage + row * 128 + ((rd_chunk ^ (row & 7)) << 4));
-                const int m = c0 + co.wave_col0 + tn * 32 + row;
-                if (full || (m < C && n < R)) *(v4i*)(origin + (int64_t)(tn * 32 + 8 * k) * ld + lane_off) = v;
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-};
-
-// post = bf16(max(bf16(acc * *dequant), 0)^2); optionally post_f8 = e4m3(min(post / act_scale, 448))
-// and a per-workgroup running max of post written to partial_amax[bid].
-template <bool EMIT>      // EMIT: also the e4m3 copy of post and the per-workgroup maxima
-struct EpiRelu2T {
-    uint16_t* post;
-    int64_t ld;
-    const float* dequant;        // 1-element device tensor
-    uint8_t* post_f8;            // EMIT only
-    int64_t ld_f8;
-    const float* act_scale;      // 1-element device tensor, EMIT only
-    float* partial_amax;         // EMIT only; n_partials entries
-    int n_partials;
-    int R, C;
-    float scale, inv_act, amax;
-    static constexpr int EXTRA_LDS = 0;
-    static constexpr bool NEEDS_SCRATCH = EMIT;     // the e4m3 strip is staged through the free operand slot
-    static constexpr bool JOB_END_NEEDS_SCRATCH = false;
-    template <class Cfg>
-    __device__ void job_begin(int) {}
-    template <class Cfg>
-    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
-    __device__ void partial(bool, int) {}
-    __device__ void begin(int, int, uint8_t*) {
-        scale = *dequant;
-        inv_act = EMIT ? 1.0f / *act_scale : 0.0f;
-        amax = 0.0f;
-    }
-    template <class Cfg>
-    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co,
-                         uint8_t* scratch, int lane) {
-        // address = wave-uniform pointer + ONE per-lane 32-bit offset, as in EpiStoreBf16
-        uint16_t* origin = post + ((int64_t)r0 * ld + c0);
-        const uint32_t lane_off = (uint32_t)co.row_base * (uint32_t)ld + (uint32_t)co.col_base;
-        const int rlim = R - r0 - co.row_base, clim = C - c0 - co.col_base;
-        const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
-#pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm) {
-#pragma unroll
-            for (int tn = 0; tn < Cfg::TN; ++tn) {
-#pragma unroll
-                for (int v = 0; v < 16; v += 2) {
-                    const int dr = co.dr(tm, v), dc = tn * 32;
-                    // c = bf16(acc * dequant); post = bf16(max(c, 0)^2): both roundings by the packed converter
-                    // (the maximum on the product: relu(bf16(x)) == bf16(relu(x)), see EpiRelu2Lines)
-                    const uint32_t pre = cvt_pk_bf16(fmaxf(acc[tm][tn][v] * scale, 0.0f), fmaxf(acc[tm][tn][v + 1] * scale, 0.0f));
-                    const float c0f = __uint_as_float(pre << 16), c1f = __uint_as_float(pre & 0xffff0000u);
-                    const uint32_t pk = cvt_pk_bf16(c0f * c0f, c1f * c1f);
-                    uint16_t* pu = origin + ((int64_t)dr * ld + dc);
-                    const bool ok0 = full || (dr < rlim && dc < clim), ok1 = full || (dr + 1 < rlim && dc < clim);
-                    if (ok0) pu[lane_off] = (uint16_t)pk;
-                    if (ok1) pu[lane_off + (uint32_t)ld] = (uint16_t)(pk >> 16);
-                    if (EMIT) {
-                        const float p0 = __uint_as_float(pk << 16), p1 = __uint_as_float(pk & 0xffff0000u);
-                        StripU8<Cfg>::put(scratch, lane, tn, v, f32_to_e4m3_sat(fminf(p0 * inv_act, 448.0f)));
-                        StripU8<Cfg>::put(scratch, lane, tn, v + 1, f32_to_e4m3_sat(fminf(p1 * inv_act, 448.0f)));
-                        amax = ok0 ? fmaxf(amax, p0) : amax;
-                        amax = ok1 ? fmaxf(amax, p1) : amax;
-                    }
-                }
-                if (!EMIT) __builtin_amdgcn_sched_barrier(0);
-            }
-            if constexpr (EMIT)
-                strip_flush_rowmajor_u8<Cfg>(scratch, lane, post_f8, ld_f8, r0 + co.wave_row0 + tm * 32, c0 + co.wave_col0, R, C);
-        }
-    }
     __device__ void end(uint8_t* smem, int bid, int G) {
         if (!EMIT || !partial_amax) return;
-        float m = wave_max(amax);
+        const uint32_t top = amax2 > (amax2 << 16) ? (amax2 & 0xffff0000u) : (amax2 << 16);
+        float m = wave_max(__uint_as_float(top));
         float* red = (float*)smem;
         int wave = threadIdx.x >> 6;
         if ((threadIdx.x & 63) == 0) red[wave] = m;
@@ -450,7 +320,78 @@ struct EpiRelu2T {
             for (int i = bid + G; i < n_partials; i += G) partial_amax[i] = 0.0f;
         }
     }
+    template <class Cfg>
+    __device__ void job_begin(int) {}
+    template <class Cfg>
+    __device__ void job_end(int, int, const AccCoords<Cfg>&, uint8_t*) {}
+    template <class Cfg>
+    __device__ void tile(v16f (&acc)[Cfg::TM][Cfg::TN], int r0, int c0, const AccCoords<Cfg>& co, uint8_t*, int lane) {
+        static_assert(Cfg::TM == 2 && Cfg::TN == 4 && Cfg::NWAVES * 4096 <= EXTRA_LDS, "64 x 128 wave tiles, 4 KiB of staging each");
+        typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+        const int h = lane >> 5, j = lane & 31;
+        const bool full = (r0 + Cfg::BM <= R) && (c0 + Cfg::BN <= C);
+        stored_all = full;
+        const int rd_row = lane >> 3, rd_chunk = lane & 7;
+        const int n = r0 + co.wave_row0 + rd_chunk * 8;
+        // address = wave-uniform pointer (tile origin + the block's and line group's fixed position) + ONE per-lane offset
+        uint16_t* origin = post + ((int64_t)c0 * ld + r0);
+        const uint32_t lane_off = (uint32_t)(co.wave_col0 + rd_row) * (uint32_t)ld + (uint32_t)(co.wave_row0 + rd_chunk * 8);
+        // the e4m3 block: lane -> row lane / 4 (+ 16), 16-byte piece lane % 4 of its 64 bytes
+        const int f8_row = lane >> 2, f8_chunk = lane & 3;
+        uint8_t* origin8 = EMIT ? post_f8 + ((int64_t)c0 * ld_f8 + r0) : nullptr;
+        const uint32_t lane_off8 = EMIT ? (uint32_t)(co.wave_col0 + f8_row) * (uint32_t)ld_f8 + (uint32_t)(co.wave_row0 + f8_chunk * 16) : 0u;
+        const int n8 = r0 + co.wave_row0 + f8_chunk * 16;
+        // relu(bf16(x)) == bf16(relu(x)) (rounding keeps the sign, a NaN becomes 0 either way): the maximum is taken on
+        // the product, which spares the canonicalising pass that a maximum on re-expanded bf16 bits needs
+        auto relu2 = [&](float a0, float a1) {
+            const uint32_t pre = cvt_pk_bf16(fmaxf(a0 * scale, 0.0f), fmaxf(a1 * scale, 0.0f));
+            const float c0f = __uint_as_float(pre << 16), c1f = __uint_as_float(pre & 0xffff0000u);
+            return cvt_pk_bf16(c0f * c0f, c1f * c1f);
+        };
+#pragma unroll
+        for (int tn = 0; tn < Cfg::TN; ++tn) {
+            uint32_t f8[EMIT ? 8 : 1];
+#pragma unroll
+            for (int tm = 0; tm < Cfg::TM; ++tm)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const v16f& a = acc[tm][tn];
+                    const uint32_t p01 = relu2(a[4 * g], a[4 * g + 1]), p23 = relu2(a[4 * g + 2], a[4 * g + 3]);
+                    *(v2i*)(stage + j * 128 + (((tm * 4 + g) ^ (j & 7)) << 4) + 8 * h) = (v2i){(int)p01, (int)p23};
+                    if constexpr (EMIT) {
+                        amax2 = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, amax2), __builtin_bit_cast(u16x2, p01)));
+                        amax2 = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, amax2), __builtin_bit_cast(u16x2, p23)));
+                        const float q0 = fminf(__uint_as_float(p01 << 16) * inv_act, 448.0f), q1 = fminf(__uint_as_float(p01 & 0xffff0000u) * inv_act, 448.0f);
+                        const float q2 = fminf(__uint_as_float(p23 << 16) * inv_act, 448.0f), q3 = fminf(__uint_as_float(p23 & 0xffff0000u) * inv_act, 448.0f);
+                        int r = __builtin_amdgcn_cvt_pk_fp8_f32(q0, q1, __builtin_bit_cast(int, q0), false);
+                        f8[tm * 4 + g] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q2, q3, r, true);
+                    }
+                    if (g & 1) __builtin_amdgcn_sched_barrier(0);   // keep the arithmetic next to its LDS write (registers)
+                }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int row = 8 * k + rd_row;
+                const v4i v = *(const v4i*)(stage + row * 128 + ((rd_chunk ^ (row & 7)) << 4));
+                const int m = c0 + co.wave_col0 + tn * 32 + row;
+                if (full || (m < C && n < R)) *(v4i*)(origin + (int64_t)(tn * 32 + 8 * k) * ld + lane_off) = v;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (EMIT) {
+                // hidden units 32 tm + 8 g + 4 h ..+3 of token j: dword 8 tm + 2 g + h of the token's 64 bytes
+#pragma unroll
+                for (int d = 0; d < 8; ++d) *(uint32_t*)(stage + j * F8_STRIDE + (2 * d + h) * 4) = f8[d];
+#pragma unroll
+                for (int k = 0; k < 2; ++k) {
+                    const int row = 16 * k + f8_row;
+                    const v4i v = *(const v4i*)(stage + row * F8_STRIDE + f8_chunk * 16);
+                    const int m = c0 + co.wave_col0 + tn * 32 + row;
+                    if (full || (m < C && n8 < R)) *(v4i*)(origin8 + (int64_t)(tn * 32 + 16 * k) * ld_f8 + lane_off8) = v;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
 };
-
+using EpiRelu2Lines = EpiRelu2LinesT<false>;
 
 }  // namespace ngpt

@@ -436,33 +436,14 @@ extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float
         return fail(NGPT_EINVAL, "ngpt_fc_relu2_fwd: post_f8 needs act_scale and partial_amax");
     if (int e = check_gemm_dims("ngpt_fc_relu2_fwd", M, N, K, K, K)) return e;
     if (N % 16) return fail(NGPT_EALIGN, "ngpt_fc_relu2_fwd: N=%d must be a multiple of 16", N);
-    GemmOperands g{(const uint8_t*)x_f8, (const uint8_t*)w_f8, K, K, M, N, K, 1};
     ProfileScope prof(PROF_FC_RELU2, (hipStream_t)stream);
-    auto fill = [&](auto& epi) {
-        epi.post = (uint16_t*)post_bf16;
-        epi.ld = N;
-        epi.dequant = dequant;
-        epi.post_f8 = (uint8_t*)post_f8;
-        epi.ld_f8 = N;
-        epi.act_scale = act_scale;
-        epi.partial_amax = post_f8 ? partial_amax : nullptr;
-        epi.n_partials = n_partials;
-        epi.R = M;
-        epi.C = N;
-    };
+    // transposed product (tile rows = hidden units, tile columns = tokens): whole-line stores of post
+    GemmOperands gt{(const uint8_t*)w_f8, (const uint8_t*)x_f8, K, K, N, M, K, 1};
     if (post_f8) {
-        EpiRelu2T<true> epi{};
-        fill(epi);
+        EpiRelu2LinesT<true> epi{(uint16_t*)post_bf16, N, dequant, N, M, (uint8_t*)post_f8, N, act_scale, partial_amax, n_partials};
         // one partial-amax slot per persistent workgroup
-        return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(g, epi, (hipStream_t)stream, n_partials);
+        return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(gt, epi, (hipStream_t)stream, n_partials);
     }
-    if (N % 8 == 0) {
-        // without the e4m3 copy: transposed product (tile rows = hidden units, tile columns = tokens), whole-line stores
-        GemmOperands gt{(const uint8_t*)w_f8, (const uint8_t*)x_f8, K, K, N, M, K, 1};
-        EpiRelu2Lines epi{(uint16_t*)post_bf16, N, dequant, N, M};
-        return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(gt, epi, (hipStream_t)stream, 0);
-    }
-    EpiRelu2T<false> epi{};
-    fill(epi);
-    return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(g, epi, (hipStream_t)stream, 0);
+    EpiRelu2Lines epi{(uint16_t*)post_bf16, N, dequant, N, M};
+    return launch_gemm_fmt<MainCfg, FMT_E4M3, FMT_E4M3>(gt, epi, (hipStream_t)stream, 0);
 }
