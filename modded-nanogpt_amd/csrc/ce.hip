@@ -934,7 +934,8 @@ __global__ __launch_bounds__(256) void ce_bwd_prep_kernel(BwdPrepArgs p) {
 }
 
 __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __restrict__ codes, int nkp, int m0, int M,
-                                                             const float* __restrict__ rowf, const float* __restrict__ dcode,
+                                                             const float* __restrict__ rowf, const int* __restrict__ big,
+                                                             const float* __restrict__ dcode,
                                                              int nkt, uint8_t* __restrict__ dl_panel, int nvt, int* __restrict__ flags,
                                                              int* __restrict__ list, int* __restrict__ count,
                                                              const int* __restrict__ probe_hits, int probe_limit) {
@@ -950,19 +951,44 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
     const int tok0 = m0 + a * 128;
     const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes + (tok0 & 128) * 16;
     bool below = false;
+    // the two 128-token halves of a 256-token block ask the same flag: no product of the block leaves the e5m2 range
+    // unless it is set (see ce_rowf_block), and the conversion then needs no clamps
+    const int may_saturate = ((const __attribute__((address_space(4))) int*)(uintptr_t)big)[tok0 >> 8];
+    auto convert = [&](auto sat) {
+        constexpr bool SAT = decltype(sat)::value;
+        // all global loads first, then per 16 codes: sixteen table reads in flight, then products, conversions, LDS writes
+        v4i c[4];
+        float rf[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int i = tid + 256 * j, r = i & 127, ch = i >> 7;   // 16 codes (group ch) of token tok0 + r
-        const v4i c = *(const v4i*)(src + ch * kCodeGroupBytes + r * 16);
-        const float rf = rowf[tok0 + r];                          // zero past the last token
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const uint32_t w = (uint32_t)c[k];
-            below |= (tok0 + r < M) && code_needs_logit(w, rf, d_below);
-            word_at(r, ch * 4 + k) = f32x4_to_e5m2_sat<true>(rf * dtab[w & 0xffu], rf * dtab[(w >> 8) & 0xffu],
-                                                             rf * dtab[(w >> 16) & 0xffu], rf * dtab[w >> 24]);
+        for (int j = 0; j < 4; ++j) {
+            const int i = tid + 256 * j, r = i & 127, ch = i >> 7;   // 16 codes (group ch) of token tok0 + r
+            c[j] = *(const v4i*)(src + ch * kCodeGroupBytes + r * 16);
+            rf[j] = rowf[tok0 + r];                                   // zero past the last token
         }
-    }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = tid + 256 * j, r = i & 127, ch = i >> 7;
+            float d[16];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t w = (uint32_t)c[j][k];
+                d[4 * k] = dtab[w & 0xffu];
+                d[4 * k + 1] = dtab[(w >> 8) & 0xffu];
+                d[4 * k + 2] = dtab[(w >> 16) & 0xffu];
+                d[4 * k + 3] = dtab[w >> 24];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const bool inside = tok0 + r < M;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                below |= inside & code_needs_logit((uint32_t)c[j][k], rf[j], d_below);
+                word_at(r, ch * 4 + k) = f32x4_to_e5m2_sat<SAT>(rf[j] * d[4 * k], rf[j] * d[4 * k + 1], rf[j] * d[4 * k + 2], rf[j] * d[4 * k + 3]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    if (may_saturate) convert(std::true_type{});
+    else convert(std::false_type{});
     if (__syncthreads_or(below) && tid == 0) {
         const int tt = (tok0 - m0) >> 8, vt = kv >> 1;
         if (atomicExch(&flags[tt * nvt + vt], 1) == 0) list[atomicAdd(count, 1)] = (tt << 16) | vt;
@@ -1526,7 +1552,7 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
             // 1'. the pass's dlogits panel from the forward's sigma codes; tiles with a sigma below the code window
             //     that matters (none, normally) are then redone from the logits
             ProfileScope prof(PROF_CE_DLOGITS, st);
-            ce_codes_to_dl_kernel<<<dim3(nbx, nkt), 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, rowf, dcode,
+            ce_codes_to_dl_kernel<<<dim3(nbx, nkt), 256, 0, st>>>((const uint8_t*)sigma_codes, (int)(Vp / 128), m0, M, rowf, big, dcode,
                                                                   nkt, dw_panel, nvt, flags, list, count, hits, limit);
             if (int e = check_launch("ce_codes_to_dl_kernel")) return e;
             g.tile_list = list;
