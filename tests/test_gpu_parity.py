@@ -535,6 +535,40 @@ def test_lmhead_ce_backward_from_sigma_codes(amd, oracle, M, K, V, n_predict, pr
     assert torch.equal(dx0, dx1) and torch.equal(dw0, dw1)
 
 
+@pytest.mark.parametrize("mode", ["codes", "recompute"])
+def test_lmhead_ce_backward_in_several_passes(amd, oracle, mode):
+    """More than 65536 tokens: the backward works through them in passes of 65536 tokens and dW accumulates over
+    the passes.  Checked against the backward of the two parts on their own (one pass each, the case every other
+    test covers): a row's gradient depends on its own statistics only, so dx is the parts' dx and dW their sum."""
+    M0, K, V = 65536, 256, 512
+    M = M0 + 512
+    x, w, t, sc, mtp, ptd, pwd = _codes_case(oracle, M, K, V, 77, 1, False, 0)
+    fwd = (dev(x), dev(w), dev(t), dev(mtp), ptd, pwd, sc["x_s"], sc["w_s"], 23.0, 5.0, 7.5, False)
+    tail = (sc["x_s"], sc["w_s"], sc["grad_s"], 1.0, 23.0, 5.0, 7.5, False)
+    if mode == "codes":
+        _, lse, sig, x_f8, w_f8, codes = torch.ops.nanogpt.lmhead_ce_fwd_codes(*fwd)
+        run = lambda lo, hi, cd: torch.ops.nanogpt.lmhead_ce_bwd_codes(x_f8[lo:hi], w_f8, dev(t)[lo:hi], dev(mtp), ptd[lo:hi], pwd, lse[lo:hi],
+                                                                        sig[:, lo:hi].contiguous(), cd, *tail)
+        # the code panel is made of blocks of 256 tokens, M0 is a multiple of 256: the parts' panels are slices of it
+        per_tile = codes.numel() // (-(-M // 256))
+        dx, dw = run(0, M, codes)
+        dx_a, dw_a = run(0, M0, codes[: per_tile * (M0 // 256)])
+        dx_b, dw_b = run(M0, M, codes[per_tile * (M0 // 256):])
+    else:
+        _, lse, sig, x_f8, w_f8 = torch.ops.nanogpt.lmhead_ce_fwd(*fwd)
+        run = lambda lo, hi: torch.ops.nanogpt.lmhead_ce_bwd(x_f8[lo:hi], w_f8, dev(t)[lo:hi], dev(mtp), ptd[lo:hi], pwd, lse[lo:hi],
+                                                             sig[:, lo:hi].contiguous(), *tail)
+        dx, dw = run(0, M)
+        dx_a, dw_a = run(0, M0)
+        dx_b, dw_b = run(M0, M)
+    assert torch.isfinite(dx.float()).all() and torch.isfinite(dw).all() and dw.abs().max() > 0
+    # the last token of a part has no successor inside the part: with n_predict = 1 the target of row m is targets[m] alone,
+    # so the parts see exactly the rows' own targets
+    assert_close_gemm(dx[:M0], dx_a, tol=2e-3)
+    assert_close_gemm(dx[M0:], dx_b, tol=2e-3)
+    assert_close_gemm(dw, dw_a + dw_b, tol=2e-3)
+
+
 def test_fused_lmhead_ce_backward_modes(amd, oracle, monkeypatch):
     """FusedSoftcappedCrossEntropy in both settings of fused.CE_BACKWARD against the oracle."""
     M, K, V = 512, 256, 3072
