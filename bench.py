@@ -311,6 +311,12 @@ def workload_lmhead_ce(args, amd, lib, dev):
         work["dlogits_from_codes"] = (2.0 * M * V, "hbm")
         mode_desc = "the forward keeps one sigma code byte per logit for the backward (three GEMM passes)"
     extra = {"mean_loss": float(out[0].mean()), "ce_backward": args.ce_backward}
+    # device memory of size ~ M x V that each mode of the backward needs: the code panel lives from the forward to the
+    # backward (the reference keeps an e5m2 gradient of that size there), the dlogits panel is backward workspace
+    bwd_ws = int(lib.ngpt_lmhead_ce_bwd_workspace_bytes(M, K, V, 0))
+    extra["memory_bytes"] = {"codes": {"saved_for_backward": int(lib.ngpt_lmhead_ce_codes_bytes(M, V)), "backward_workspace": bwd_ws},
+                             "recompute": {"saved_for_backward": 0, "backward_workspace": bwd_ws},
+                             "forward_workspace": int(lib.ngpt_lmhead_ce_fwd_workspace_bytes(M, K, V, 0))}
     if args.tail_columns:
         extra["tail_columns"] = args.tail_columns
     if not args.no_other_mode:  # the other mode of the backward, timed the same way on a few steps, for the record

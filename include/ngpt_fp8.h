@@ -106,7 +106,11 @@ int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const void* B, int f
 /* ---- nanogpt::mm / nanogpt::mm_t forward --------------------------------------------------
  * train_gpt_medium.py:40-57 (w_layout OUT_IN, w [N,K]) and train_gpt.py:70-95 (IN_OUT, w [K,N]).
  * x [M,K] bf16.  Writes out [M,N] bf16 = bf16((x_f8 . w_f8^T) * x_s * w_s), x_f8 [M,K] e4m3 and
- * w_f8 (e4m3, same layout as w).  K % 128 == 0, M % 16 == 0, N % 16 == 0. */
+ * w_f8 (e4m3, same layout as w).  K % 128 == 0, M % 16 == 0, N % 16 == 0.
+ * Workspace: IN_OUT needs N x K bytes (the [N, K] copy the GEMM reads).  ngpt_mm_fwd_workspace_bytes adds N x K bytes
+ * for N % 64 == 0, K in {256, 512, 768, 1024} and enough tokens to fill the device: with that much the product runs
+ * on the token-stationary kernel of the fused cross-entropy (weights in MFMA-fragment order), with less on the tile
+ * kernel; same results bit for bit. */
 int64_t ngpt_mm_fwd_workspace_bytes(int M, int N, int K, int w_layout);
 int ngpt_mm_fwd(const void* x_bf16, const void* w_bf16, int M, int N, int K, float x_s, float w_s,
                 void* out_bf16, void* x_f8, void* w_f8, int w_layout,
@@ -132,6 +136,15 @@ int ngpt_mm_bwd(const void* g_bf16, const void* x_f8, const void* w_f8, int M, i
 int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, int M, int N, int K,
                       void* post_bf16, void* post_f8, const float* act_scale,
                       float* partial_amax, int n_partials, void* stream);
+/* The same with a workspace of ngpt_fc_relu2_fwd_workspace_bytes (N x K bytes for N % 64 == 0, K in {256, 512, 768,
+ * 1024} and enough tokens to fill the device, else 0): the token-stationary kernel of the fused cross-entropy then
+ * runs the product (weights re-ordered into the workspace first), with the same results bit for bit.  With post_f8
+ * that kernel needs n_partials >= ngpt_num_cus(); otherwise, or without the workspace, the call is
+ * ngpt_fc_relu2_fwd. */
+int64_t ngpt_fc_relu2_fwd_workspace_bytes(int M, int N, int K);
+int ngpt_fc_relu2_fwd_ws(const void* x_f8, const void* w_f8, const float* dequant, int M, int N, int K,
+                         void* post_bf16, void* post_f8, const float* act_scale,
+                         float* partial_amax, int n_partials, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* The same kernel on bf16 operands (FORWARD without USE_FP8, the reference's DISABLE_FP8 path, launched at
  * triton_kernels.py:716-718): post [M,N] = bf16(max(bf16(x . w^T), 0)^2) for x [M,K], w [N,K] bf16.

@@ -39,6 +39,8 @@ SIGNATURES = {
     "ngpt_mm_bwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
     "ngpt_mm_bwd": (_I, [_P, _P, _P, _I, _I, _I, _F, _F, _F, _P, _P, _I, _P, _L, _P]),
     "ngpt_fc_relu2_fwd": (_I, [_P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _P]),
+    "ngpt_fc_relu2_fwd_workspace_bytes": (_L, [_I, _I, _I]),
+    "ngpt_fc_relu2_fwd_ws": (_I, [_P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _P, _L, _P]),
     "ngpt_linear_relu2_bf16": (_I, [_P, _P, _I, _I, _I, _P, _P]),
     "ngpt_fc_relu2_bwd_dpre": (_I, [_P, _P, _P, _I, _I, _I, _P, _P]),
     "ngpt_gemm_bf16_workspace_bytes": (_L, [_I, _I, _I]),

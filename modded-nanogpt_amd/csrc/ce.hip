@@ -1113,11 +1113,13 @@ static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwdT<CODES>& epi, hip
 static bool xs_eligible(int M, int K, int V) { return M > 0 && V % XS_UNIT == 0 && (K == 256 || K == 512 || K == 768 || K == 1024); }
 
 template <int MODE, int NS>
-static int launch_ce_fwd_xs(XsArgs a, hipStream_t st) {
+static int launch_ce_fwd_xs(XsArgs a, hipStream_t st, int slot = -1) {
     auto kernel = ce_fwd_xs_kernel<MODE, NS>;
-    const int LDS = XS_CAND_LDS + a.K * XS_TOK;      // dynamic part; the table is static LDS
+    // dynamic LDS: candidate targets / row factors + slab (the table is static LDS), or slab + the waves' line staging
+    constexpr int HEAD = MODE >= XS_LINES ? XS_WAVES * XS_LINE_STAGE : XS_CAND_LDS;
+    const int LDS = HEAD + a.K * XS_TOK;
     static PerDeviceOnce configured;
-    if (int e = configured.run([&] { return allow_lds(kernel, XS_CAND_LDS + XS_MAX_K * XS_TOK); })) return e;
+    if (int e = configured.run([&] { return allow_lds(kernel, HEAD + NS * 64 * XS_TOK); })) return e;
     const int cus = num_cus();
     if (cus < CE_XCDS) return fail(NGPT_EINVAL, "lm_head CE forward: no HIP device (or fewer than %d compute units)", CE_XCDS);
     // workgroups per XCD = token tiles in flight (mg) x vocabulary shares (splits); the split count that needs the
@@ -1136,10 +1138,12 @@ static int launch_ce_fwd_xs(XsArgs a, hipStream_t st) {
     }
     a.splits = best_splits;
     {
-        ProfileScope prof(MODE == XS_DL ? PROF_CE_DLOGITS : PROF_CE_FWD, st);
+        ProfileScope prof(slot >= 0 ? slot : MODE == XS_DL ? PROF_CE_DLOGITS : PROF_CE_FWD, st, slot != -2);     // -2: the caller's scope covers it
+        if (MODE == XS_RELU2_EMIT && a.partial_amax && a.n_partials < CE_XCDS * best_splits * best_mg)
+            return fail(NGPT_EINVAL, "fc + relu^2: %d partial maxima for %d workgroups", a.n_partials, CE_XCDS * best_splits * best_mg);
         kernel<<<CE_XCDS * best_splits * best_mg, XS_THREADS, LDS, st>>>(a);
     }
-    return check_launch(MODE == XS_DL ? "lm_head CE backward (dlogits, token-stationary)" : "lm_head CE forward (token-stationary)");
+    return check_launch(MODE >= XS_LINES ? "fp8 GEMM (token-stationary)" : MODE == XS_DL ? "lm_head CE backward (dlogits, token-stationary)" : "lm_head CE forward (token-stationary)");
 }
 
 template <class Cfg, class Iter, class Epi>
@@ -1231,12 +1235,12 @@ namespace ngpt {
 // Everything the forward's GEMM kernel starts from, in one launch.  Block ranges: [0, bx) the e4m3 copy of the
 // activations; then bw blocks for the e4m3 copy of (out, in) weights, which also goes to the token-stationary kernel's
 // fragment order if w_frag is given (each 8-byte piece of a row is 8 bytes of one 16-byte fragment entry, see
-// xs_frag_from_f8_kernel); then the lookup tables; then the zeros of the partial sums (an empty vocabulary split must
+// xs_frag_from_f8_kernel); then b_tab blocks for the lookup tables; then the zeros of the partial sums (an empty vocabulary split must
 // read as zero) and of the saved sigmas (entries of candidates without a target are never written by the kernel).
 struct FwdPrepArgs {
     const v4i* x; v2i* x_f8; int64_t nx8; float x_s;
     const v4i* w; v2i* w_f8; int64_t nw8; float w_s; uint8_t* w_frag; int K8;
-    int bx, bw;
+    int bx, bw, b_tab;
     float *tabE, *tabD; Softcap sc; bool embed_codes;
     float* zero0; int64_t n0; float* zero1; int64_t n1;
 };
@@ -1263,13 +1267,70 @@ __global__ __launch_bounds__(256) void ce_fwd_prep_kernel(FwdPrepArgs p) {
         return;
     }
     b -= p.bw;
-    if (b < TAB_BLOCKS) {
+    if (b < p.b_tab) {
         ce_table_entry(b * 256 + tid, p.tabE, p.tabD, p.sc, p.embed_codes);
         return;
     }
-    const int64_t i = (int64_t)(b - TAB_BLOCKS) * 256 + tid;
+    const int64_t i = (int64_t)(b - p.b_tab) * 256 + tid;
     if (i < p.n0) p.zero0[i] = 0.0f;
     else if (i - p.n0 < p.n1) p.zero1[i - p.n0] = 0.0f;
+}
+
+bool xs_gemm_eligible(int M, int N, int K) { return xs_eligible(M, K, N); }
+int64_t xs_gemm_frag_bytes(int N, int K) { return align_up(xs_frag_bytes(N, K), 256); }
+int xs_gemm_make_frag(const void* w_f8, int N, int K, void* w_frag, hipStream_t st) {
+    xs_frag_from_f8_kernel<<<std::min((N / XS_UNIT) * (K / 128), 8 * num_cus()), 256, 0, st>>>((const uint8_t*)w_f8, N, K, (uint8_t*)w_frag);
+    return check_launch("xs_frag_from_f8_kernel");
+}
+static void prep_quant_blocks(FwdPrepArgs& a) {   // quantiser blocks in proportion to the sizes
+    const int64_t cap = (int64_t)num_cus() * 16;
+    int64_t bx = (a.nx8 + 255) / 256, bw = (a.nw8 + 255) / 256;
+    if (bx + bw > cap) {
+        bx = std::max<int64_t>(1, bx * cap / (bx + bw));
+        bw = a.nw8 ? std::max<int64_t>(1, cap - bx) : 0;
+    }
+    a.bx = (int)bx;
+    a.bw = (int)bw;
+}
+int xs_gemm_quant_pair_frag(const void* x_bf16, void* x_f8, int64_t nx, float x_s, const void* w_bf16, void* w_f8, int N, int K, float w_s,
+                            void* w_frag, hipStream_t st) {
+    FwdPrepArgs a{};
+    a.x = (const v4i*)x_bf16; a.x_f8 = (v2i*)x_f8; a.nx8 = nx / 8; a.x_s = x_s;
+    a.w = (const v4i*)w_bf16; a.w_f8 = (v2i*)w_f8; a.nw8 = (int64_t)N * K / 8; a.w_s = w_s;
+    a.w_frag = (uint8_t*)w_frag;
+    a.K8 = K / 8;
+    prep_quant_blocks(a);
+    ce_fwd_prep_kernel<<<a.bx + a.bw, 256, 0, st>>>(a);
+    return check_launch("ce_fwd_prep_kernel");
+}
+int xs_gemm_lines(int mode, const void* x_f8, const void* w_frag, int M, int N, int K, float scale, const float* dscale,
+                  void* out_bf16, int64_t ld_out, void* out_f8, int64_t ld_f8, const float* act_scale, float* partial_amax, int n_partials,
+                  int slot, hipStream_t st) {
+    XsArgs a{};
+    a.w_frag = (const uint8_t*)w_frag;
+    a.x_f8 = (const uint8_t*)x_f8;
+    a.M = M; a.V = N; a.K = K;
+    a.scale = scale;
+    a.dscale = dscale;
+    a.out = (uint16_t*)out_bf16; a.ld_out = ld_out;
+    a.out_f8 = (uint8_t*)out_f8; a.ld_f8 = ld_f8;
+    a.act_scale = act_scale; a.partial_amax = partial_amax; a.n_partials = n_partials;
+    auto go = [&](auto ns) -> int {
+        constexpr int NS = decltype(ns)::value;
+        switch (mode) {
+            case XS_LINES: return launch_ce_fwd_xs<XS_LINES, NS>(a, st, slot);
+            case XS_RELU2: return launch_ce_fwd_xs<XS_RELU2, NS>(a, st, slot);
+            case XS_RELU2_EMIT: return launch_ce_fwd_xs<XS_RELU2_EMIT, NS>(a, st, slot);
+        }
+        return fail(NGPT_EINVAL, "xs_gemm_lines: mode %d", mode);
+    };
+    switch (K / 64) {
+        case 4: return go(std::integral_constant<int, 4>{});
+        case 8: return go(std::integral_constant<int, 8>{});
+        case 12: return go(std::integral_constant<int, 12>{});
+        case 16: return go(std::integral_constant<int, 16>{});
+    }
+    return fail(NGPT_EINVAL, "xs_gemm_lines: K=%d", K);
 }
 
 // Forward of the fused lm_head + CE on a workspace that the caller (ngpt_lmhead_ce_fwd) or the library itself
@@ -1307,19 +1368,13 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
         a.w = (const v4i*)w_bf16; a.w_f8 = (v2i*)w_f8_vk; a.nw8 = w_here ? (int64_t)V * K / 8 : 0; a.w_s = w_s;
         a.w_frag = (w_here && use_xs) ? w_frag : nullptr;
         a.K8 = K / 8;
-        // quantiser blocks in proportion to the sizes
-        const int64_t cap = (int64_t)num_cus() * 16;
-        int64_t bx = (a.nx8 + 255) / 256, bw = (a.nw8 + 255) / 256;
-        if (bx + bw > cap) {
-            bx = std::max<int64_t>(1, bx * cap / (bx + bw));
-            bw = a.nw8 ? std::max<int64_t>(1, cap - bx) : 0;
-        }
-        a.bx = (int)bx; a.bw = (int)bw;
+        prep_quant_blocks(a);
+        a.b_tab = TAB_BLOCKS;
         a.tabE = tabE; a.tabD = tabD; a.sc = sc; a.embed_codes = sigma_codes != nullptr;
         a.zero0 = part; a.n0 = (int64_t)CE_SPLITS * M;
         a.zero1 = saved_sigma; a.n1 = (int64_t)MAX_CAND * M;
         const int64_t fill_blocks = (a.n0 + a.n1 + 255) / 256;
-        ce_fwd_prep_kernel<<<(int)(bx + bw + TAB_BLOCKS + fill_blocks), 256, 0, st>>>(a);
+        ce_fwd_prep_kernel<<<(int)(a.bx + a.bw + TAB_BLOCKS + fill_blocks), 256, 0, st>>>(a);
         if (int e = check_launch("ce_fwd_prep_kernel")) return e;
         if (!w_here)
             if (int e = ngpt_quant_fp8_2d(w_bf16, K, V, w_s, NGPT_FMT_E4M3, nullptr, w_f8_vk, stream)) return e;

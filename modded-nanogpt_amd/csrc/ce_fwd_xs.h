@@ -1,5 +1,8 @@
 // Fused lm_head + softcapped CE, token-stationary kernel (included by ce.hip): the forward (XS_FWD, XS_FWD_CODES) and the
-// backward's logits recompute that writes the e5m2 gradient panel (XS_DL).
+// backward's logits recompute that writes the e5m2 gradient panel (XS_DL).  The same contraction loop also serves plain
+// fp8 GEMMs with a row-major bf16 output [tokens, N] whose rows are written as whole 128-byte lines: XS_LINES
+// (bf16(acc * scale): nanogpt::mm forward), XS_RELU2 and XS_RELU2_EMIT (the FP8 c_fc with its ReLU^2 epilogue, see
+// EpiRelu2LinesT); there "vocabulary" reads "output features".
 //
 // Same arithmetic as EpiCEFwdT / EpiDlStore on gemm_tn_kernel (rows = vocabulary, columns = tokens, 32x32x64 fp8 MFMAs over the
 // contraction in ascending order, softcap through the bf16-indexed table), different data movement:
@@ -35,7 +38,8 @@ constexpr int XS_MAX_SPLITS = CE_SPLITS;    // part[] has CE_SPLITS slots per to
 
 __host__ __device__ inline int64_t xs_frag_bytes(int V, int K) { return (int64_t)V * K; }
 
-enum { XS_FWD = 0, XS_FWD_CODES = 1, XS_DL = 2 };
+enum { XS_FWD = 0, XS_FWD_CODES = 1, XS_DL = 2, XS_LINES = 3, XS_RELU2 = 4, XS_RELU2_EMIT = 5 };
+constexpr int XS_LINE_STAGE = 4096;         // XS_LINES..: LDS bytes per wave for turning accumulator registers into whole lines
 
 struct XsArgs {
     const uint8_t* w_frag;   // fragment-major weights
@@ -57,23 +61,43 @@ struct XsArgs {
     const int* big;          // per 256 tokens: a product may leave the e5m2 range
     uint8_t* dl_panel;       // [V / 256 rounded up][nkt] blocks of 256 vocabulary rows x 128 tokens
     int nkt;
+    // XS_LINES, XS_RELU2, XS_RELU2_EMIT
+    uint16_t* out;           // bf16 [M, ld_out]
+    int64_t ld_out;
+    const float* dscale;     // nullable: one more factor of the scale, read from device memory
+    uint8_t* out_f8;         // XS_RELU2_EMIT: e4m3(min(out / *act_scale, 448)), [M, ld_f8]
+    int64_t ld_f8;
+    const float* act_scale;
+    float* partial_amax;     // XS_RELU2_EMIT: largest output of every workgroup, zeros up to n_partials; nullable
+    int n_partials;
 };
 
 template <int MODE, int NS /* K / 64 */>
 __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
-    constexpr bool CODES = MODE == XS_FWD_CODES, DL = MODE == XS_DL;
+    constexpr bool CODES = MODE == XS_FWD_CODES, DL = MODE == XS_DL, LINES = MODE >= XS_LINES, EMIT = MODE == XS_RELU2_EMIT;
     // weight fragment sets in registers (loads run XS_RING - 1 steps ahead); must divide the number of steps
     constexpr int XS_RING = 4;
     static_assert(NS % XS_RING == 0, "ring slots of a unit's first steps");
     extern __shared__ __attribute__((aligned(1024))) uint8_t xs_smem[];
     int* const cand = (int*)xs_smem;                  // [MAX_CAND][XS_TOK] valid target column of the job's tokens, else -1
-    uint8_t* const xslab = xs_smem + XS_CAND_LDS;     // [K / 128][128 tokens][128 bytes], chunks swizzled as in gemm_tn.h
-    const float* const tab = lds_table();
-    load_table(lds_table(), p.gtabE);
+    uint8_t* const xslab = xs_smem + (LINES ? 0 : XS_CAND_LDS);     // [K / 128][128 tokens][128 bytes], chunks swizzled as in gemm_tn.h
+    const float* tab = nullptr;
+    if constexpr (!LINES) {
+        tab = lds_table();
+        load_table(lds_table(), p.gtabE);
+    }
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int M = p.M, K = p.K;
+    // XS_LINES..: the wave's staging block behind the slab; scale and running maximum of the ReLU^2 modes
+    uint8_t* const line_stage = xslab + K * XS_TOK + wave * XS_LINE_STAGE;
+    float line_scale = p.scale, inv_act = 0.0f;
+    uint32_t amax2 = 0u;
+    if constexpr (LINES) {
+        if (p.dscale) line_scale *= ((const __attribute__((address_space(4))) float*)(uintptr_t)p.dscale)[0];
+        if constexpr (EMIT) inv_act = 1.0f / ((const __attribute__((address_space(4))) float*)(uintptr_t)p.act_scale)[0];
+    }
     const int64_t unit_bytes = (int64_t)K * XS_UNIT;
 
     // job walk: XCD x owns a contiguous block of token tiles, mg of them in flight, each shared by `splits` workgroups
@@ -110,7 +134,7 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
             }
             if constexpr (DL) {
                 if (tid < XS_TOK) ((float*)cand)[tid] = p.rowf[c0 + tid];
-            } else {
+            } else if constexpr (!LINES) {
                 for (int i = tid; i < p.ncand * XS_TOK; i += XS_THREADS) {
                     const int c = i / XS_TOK, jj = i % XS_TOK, m = c0 + jj;
                     const int64_t t = (m < M) ? cand_target(p.ca, m, c) : -1;
@@ -263,6 +287,67 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
                 else run(std::false_type{});
                 continue;
             }
+            if constexpr (LINES) {
+                // ---- epilogue of the unit: bf16 results as whole lines (as EpiRelu2LinesT::tile).  Registers 4 g ..+3 of
+                // acc[tm][tn] are the output features 32 tm + 8 g + 4 h ..+3 of token 32 tn + j: every 32-token x 64-feature
+                // block (4 KiB) is collected in the wave's LDS block and leaves as 128-byte lines, 16 bytes per lane.
+                typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+                uint8_t* const stage = line_stage;
+                const int rd_row = el >> 3, rd_chunk = el & 7;
+                uint16_t* const obase = p.out + ((int64_t)c0 * p.ld_out + u * XS_UNIT);
+                const uint32_t lane_off = (uint32_t)rd_row * (uint32_t)p.ld_out + (uint32_t)(rd_chunk * 8);
+                const int f8_row = el >> 2, f8_chunk = el & 3;
+                uint8_t* const obase8 = EMIT ? p.out_f8 + ((int64_t)c0 * p.ld_f8 + u * XS_UNIT) : nullptr;
+                const uint32_t lane_off8 = EMIT ? (uint32_t)f8_row * (uint32_t)p.ld_f8 + (uint32_t)(f8_chunk * 16) : 0u;
+                auto pair_of = [&](float a0, float a1) -> uint32_t {
+                    if constexpr (MODE == XS_LINES) return cvt_pk_bf16(a0 * line_scale, a1 * line_scale);
+                    // c = bf16(acc * scale); bf16(max(c, 0)^2): the maximum on the product (relu(bf16(x)) == bf16(relu(x)))
+                    const uint32_t pre = cvt_pk_bf16(fmaxf(a0 * line_scale, 0.0f), fmaxf(a1 * line_scale, 0.0f));
+                    const float c0f = __uint_as_float(pre << 16), c1f = __uint_as_float(pre & 0xffff0000u);
+                    return cvt_pk_bf16(c0f * c0f, c1f * c1f);
+                };
+#pragma unroll
+                for (int tn = 0; tn < 4; ++tn) {
+                    uint32_t f8[EMIT ? 8 : 1];
+#pragma unroll
+                    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const v16f& r = acc[tm][tn];
+                            const uint32_t p01 = pair_of(r[4 * g], r[4 * g + 1]), p23 = pair_of(r[4 * g + 2], r[4 * g + 3]);
+                            *(v2i*)(stage + j * 128 + (((tm * 4 + g) ^ (j & 7)) << 4) + 8 * h) = (v2i){(int)p01, (int)p23};
+                            if constexpr (EMIT) {
+                                amax2 = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, amax2), __builtin_bit_cast(u16x2, p01)));
+                                amax2 = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, amax2), __builtin_bit_cast(u16x2, p23)));
+                                const float q0 = fminf(__uint_as_float(p01 << 16) * inv_act, 448.0f), q1 = fminf(__uint_as_float(p01 & 0xffff0000u) * inv_act, 448.0f);
+                                const float q2 = fminf(__uint_as_float(p23 << 16) * inv_act, 448.0f), q3 = fminf(__uint_as_float(p23 & 0xffff0000u) * inv_act, 448.0f);
+                                int rr = __builtin_amdgcn_cvt_pk_fp8_f32(q0, q1, __builtin_bit_cast(int, q0), false);
+                                f8[tm * 4 + g] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q2, q3, rr, true);
+                            }
+                            if (g & 1) __builtin_amdgcn_sched_barrier(0);
+                        }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int row = 8 * k + rd_row;
+                        const v4i v = *(const v4i*)(stage + row * 128 + ((rd_chunk ^ (row & 7)) << 4));
+                        if (c0 + tn * 32 + row < M) *(v4i*)(obase + (int64_t)(tn * 32 + 8 * k) * p.ld_out + lane_off) = v;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (EMIT) {
+                        constexpr int F8_STRIDE = 80;
+#pragma unroll
+                        for (int d = 0; d < 8; ++d) *(uint32_t*)(stage + j * F8_STRIDE + (2 * d + h) * 4) = f8[d];
+#pragma unroll
+                        for (int k = 0; k < 2; ++k) {
+                            const int row = 16 * k + f8_row;
+                            const v4i v = *(const v4i*)(stage + row * F8_STRIDE + f8_chunk * 16);
+                            if (c0 + tn * 32 + row < M) *(v4i*)(obase8 + (int64_t)(tn * 32 + 16 * k) * p.ld_f8 + lane_off8) = v;
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                continue;
+            }
             // ---- epilogue of the unit: softcap table, sum of exponentials, sigma codes (as EpiCEFwdT::tile)
             // code panel (layout: EpiCEFwdT): row = this lane's token, 16 bytes = the 16 vocabulary rows of one (tm, lane half) group
             uint8_t* cd_base = nullptr;
@@ -342,7 +427,7 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
             }
         }
 
-        if constexpr (DL) continue;
+        if constexpr (DL || LINES) continue;
         // ---- job end: the lanes' sums -> part[split][token]
         wg_barrier();                                  // every wave is done reading the slab: it becomes scratch
         float* red = (float*)xslab;                    // [XS_WAVES][XS_TOK]
@@ -358,6 +443,22 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
             for (int w = 0; w < XS_WAVES; ++w) s += red[w * XS_TOK + tid];
             const int m = c0 + tid;
             if (m < M) p.part[(int64_t)split * M + m] = s;
+        }
+    }
+    if constexpr (EMIT) {
+        if (p.partial_amax) {      // the outputs are >= 0: the larger bf16 pattern is the larger value
+            const uint32_t top = amax2 > (amax2 << 16) ? (amax2 & 0xffff0000u) : (amax2 << 16);
+            const float m = wave_max(__uint_as_float(top));
+            wg_barrier();          // the last job's slab is done with
+            float* red = (float*)xslab;
+            if (lane == 0) red[wave] = m;
+            wg_barrier();
+            if (tid == 0) {
+                float t = 0.0f;
+                for (int w = 0; w < XS_WAVES; ++w) t = fmaxf(t, red[w]);
+                p.partial_amax[bid] = t;
+                for (int i = bid + G; i < p.n_partials; i += G) p.partial_amax[i] = 0.0f;
+            }
         }
     }
 }

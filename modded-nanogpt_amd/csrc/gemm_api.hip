@@ -275,9 +275,11 @@ extern "C" int ngpt_gemm_fp8_tn(const void* A, int fmt_a, int64_t lda, const voi
 }
 
 // ------------------------------------------------------------------------------------------ mm forward
+// The token-stationary kernel (128-token jobs x up to 4 output shares) needs about one job per compute unit to pay.
+static bool mm_fwd_xs(int M, int N, int K) { return xs_gemm_eligible(M, N, K) && (int64_t)(M / 128) * 4 >= num_cus(); }
+// [N, K] e4m3 copy of (in, out) weights | fragment-ordered weights (token-stationary kernel)
 extern "C" int64_t ngpt_mm_fwd_workspace_bytes(int M, int N, int K, int w_layout) {
-    (void)M;
-    return w_layout == NGPT_W_IN_OUT ? align_up((int64_t)N * K, 256) : 0;
+    return (w_layout == NGPT_W_IN_OUT ? align_up((int64_t)N * K, 256) : 0) + (mm_fwd_xs(M, N, K) ? xs_gemm_frag_bytes(N, K) : 0);
 }
 
 extern "C" int ngpt_mm_fwd(const void* x_bf16, const void* w_bf16, int M, int N, int K, float x_s, float w_s,
@@ -288,19 +290,28 @@ extern "C" int ngpt_mm_fwd(const void* x_bf16, const void* w_bf16, int M, int N,
     if (K % 128 || M % 16 || N % 16)
         return fail(NGPT_EALIGN, "ngpt_mm_fwd: need K %% 128 == 0, M %% 16 == 0, N %% 16 == 0 (M=%d N=%d K=%d)", M, N, K);
     if (w_layout != NGPT_W_OUT_IN && w_layout != NGPT_W_IN_OUT) return fail(NGPT_EINVAL, "ngpt_mm_fwd: w_layout=%d", w_layout);
-    int64_t need = ngpt_mm_fwd_workspace_bytes(M, N, K, w_layout);
+    // needed: the [N, K] copy of (in, out) weights; with room for the fragment-ordered weights as well the product runs
+    // on the token-stationary kernel
+    const int64_t need = w_layout == NGPT_W_IN_OUT ? align_up((int64_t)N * K, 256) : 0;
     if (need > 0 && (!workspace || workspace_bytes < need))
         return fail(NGPT_EWORKSPACE, "ngpt_mm_fwd: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
     hipStream_t st = (hipStream_t)stream;
     const void* w_nk = w_f8;
+    const bool xs = mm_fwd_xs(M, N, K) && workspace && workspace_bytes >= ngpt_mm_fwd_workspace_bytes(M, N, K, w_layout);
+    uint8_t* w_frag = (uint8_t*)workspace + (w_layout == NGPT_W_IN_OUT ? align_up((int64_t)N * K, 256) : 0);
     if (w_layout == NGPT_W_OUT_IN) {
-        if (int e = quant_e4m3_pair(x_bf16, x_f8, (int64_t)M * K, x_s, w_bf16, w_f8, (int64_t)N * K, w_s, st)) return e;
+        if (xs) {
+            if (int e = xs_gemm_quant_pair_frag(x_bf16, x_f8, (int64_t)M * K, x_s, w_bf16, w_f8, N, K, w_s, w_frag, st)) return e;
+        } else if (int e = quant_e4m3_pair(x_bf16, x_f8, (int64_t)M * K, x_s, w_bf16, w_f8, (int64_t)N * K, w_s, st)) return e;
     } else {
         if (int e = ngpt_quant_fp8(x_bf16, x_f8, (int64_t)M * K, x_s, NGPT_FMT_E4M3, stream)) return e;
         // w is [K, N]: one pass writes w_f8 [K, N] and the [N, K] copy the GEMM reads
         if (int e = ngpt_quant_fp8_2d(w_bf16, K, N, w_s, NGPT_FMT_E4M3, w_f8, workspace, stream)) return e;
         w_nk = workspace;
+        if (xs)
+            if (int e = xs_gemm_make_frag(w_nk, N, K, w_frag, st)) return e;
     }
+    if (xs) return xs_gemm_lines(3, x_f8, w_frag, M, N, K, x_s * w_s, nullptr, out_bf16, N, nullptr, 0, nullptr, nullptr, 0, PROF_GEMM, st);
     return gemm_store(x_f8, FMT_E4M3, K, w_nk, FMT_E4M3, K, M, N, K, x_s * w_s, out_bf16, N, 0, st, 1);
 }
 
@@ -428,14 +439,30 @@ extern "C" int ngpt_linear_relu2_bf16(const void* x_bf16, const void* w_bf16, in
 }
 
 // ------------------------------------------------------------------------------------------ fc + relu^2
+extern "C" int64_t ngpt_fc_relu2_fwd_workspace_bytes(int M, int N, int K) { return mm_fwd_xs(M, N, K) ? xs_gemm_frag_bytes(N, K) : 0; }
+
 extern "C" int ngpt_fc_relu2_fwd(const void* x_f8, const void* w_f8, const float* dequant, int M, int N, int K,
                                  void* post_bf16, void* post_f8, const float* act_scale,
                                  float* partial_amax, int n_partials, void* stream) {
+    return ngpt_fc_relu2_fwd_ws(x_f8, w_f8, dequant, M, N, K, post_bf16, post_f8, act_scale, partial_amax, n_partials, nullptr, 0, stream);
+}
+
+extern "C" int ngpt_fc_relu2_fwd_ws(const void* x_f8, const void* w_f8, const float* dequant, int M, int N, int K,
+                                    void* post_bf16, void* post_f8, const float* act_scale,
+                                    float* partial_amax, int n_partials, void* workspace, int64_t workspace_bytes, void* stream) {
     if (!x_f8 || !w_f8 || !dequant || !post_bf16) return fail(NGPT_EINVAL, "ngpt_fc_relu2_fwd: null pointer");
     if (post_f8 && (!act_scale || !partial_amax || n_partials <= 0))
         return fail(NGPT_EINVAL, "ngpt_fc_relu2_fwd: post_f8 needs act_scale and partial_amax");
     if (int e = check_gemm_dims("ngpt_fc_relu2_fwd", M, N, K, K, K)) return e;
     if (N % 16) return fail(NGPT_EALIGN, "ngpt_fc_relu2_fwd: N=%d must be a multiple of 16", N);
+    // with room for the weights in fragment order: the token-stationary kernel (the partial maxima then are one per
+    // workgroup of its grid, at most one per compute unit)
+    if (mm_fwd_xs(M, N, K) && workspace && workspace_bytes >= xs_gemm_frag_bytes(N, K) && (!post_f8 || n_partials >= num_cus())) {
+        ProfileScope prof(PROF_FC_RELU2, (hipStream_t)stream);
+        if (int e = xs_gemm_make_frag(w_f8, N, K, workspace, (hipStream_t)stream)) return e;
+        return xs_gemm_lines(post_f8 ? 5 : 4, x_f8, workspace, M, N, K, 1.0f, dequant, post_bf16, N, post_f8, N, act_scale, partial_amax, n_partials,
+                             -2, (hipStream_t)stream);
+    }
     ProfileScope prof(PROF_FC_RELU2, (hipStream_t)stream);
     // transposed product (tile rows = hidden units, tile columns = tokens): whole-line stores of post
     GemmOperands gt{(const uint8_t*)w_f8, (const uint8_t*)x_f8, K, K, N, M, K, 1};

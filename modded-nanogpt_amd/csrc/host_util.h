@@ -27,6 +27,20 @@ inline int check_launch(const char* what) {
 int quant_e4m3_pair(const void* in0, void* out0, int64_t n0, float s0, const void* in1, void* out1, int64_t n1, float s1,
                     hipStream_t st);
 
+// fp8 GEMM with a row-major bf16 output on the token-stationary kernel (ce.hip, ce_fwd_xs.h): out [M, N] = x [M, K] . w [N, K]^T,
+// w given in fragment order (xs_gemm_frag_bytes bytes, written by xs_gemm_make_frag from the row-major e4m3 matrix or by
+// xs_gemm_quant_pair_frag together with the e4m3 copies of both bf16 operands).  mode: 3 = bf16(acc * scale), 4 = the
+// ReLU^2 epilogue of c_fc, 5 = the same with the e4m3 copy and per-workgroup maxima; the scale is `scale` times
+// *dscale (device, nullable).  `slot`: profile slot of the launch.
+bool xs_gemm_eligible(int M, int N, int K);
+int64_t xs_gemm_frag_bytes(int N, int K);
+int xs_gemm_make_frag(const void* w_f8, int N, int K, void* w_frag, hipStream_t st);
+int xs_gemm_quant_pair_frag(const void* x_bf16, void* x_f8, int64_t nx, float x_s, const void* w_bf16, void* w_f8, int N, int K, float w_s,
+                            void* w_frag, hipStream_t st);
+int xs_gemm_lines(int mode, const void* x_f8, const void* w_frag, int M, int N, int K, float scale, const float* dscale,
+                  void* out_bf16, int64_t ld_out, void* out_f8, int64_t ld_f8, const float* act_scale, float* partial_amax, int n_partials,
+                  int slot, hipStream_t st);
+
 // Index of the current HIP device (-1 if there is none) and its number of compute units (cached per device).
 constexpr int kMaxDevices = 64;
 int current_device();

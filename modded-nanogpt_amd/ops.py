@@ -60,8 +60,9 @@ def mm_op(x: Tensor, w: Tensor, x_s: float, w_s: float, grad_s: float) -> tuple[
     out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     x_f8 = torch.empty((M, K), dtype=E4M3, device=x.device)
     w_f8 = torch.empty((N, K), dtype=E4M3, device=x.device)
+    ws = _workspace(lib.ngpt_mm_fwd_workspace_bytes(M, N, K, _lib.W_OUT_IN), x.device)
     _lib.check(lib.ngpt_mm_fwd(_p(x), _p(w), M, N, K, x_s, w_s, _p(out), _p(x_f8), _p(w_f8),
-                               _lib.W_OUT_IN, None, 0, _stream(x)), "ngpt_mm_fwd")
+                               _lib.W_OUT_IN, _p(ws), ws.numel(), _stream(x)), "ngpt_mm_fwd")
     return out, x_f8, w_f8
 
 
@@ -378,8 +379,9 @@ def fc_relu2_fwd(x_f8: Tensor, w_f8: Tensor, dequant_scale: Tensor) -> Tensor:
     M, K = x_f8.shape
     N = w_f8.shape[0]
     post = torch.empty((M, N), dtype=torch.bfloat16, device=x_f8.device)
-    _lib.check(lib.ngpt_fc_relu2_fwd(_p(x_f8), _p(w_f8), _p(dequant_scale), M, N, K, _p(post), None, None,
-                                     None, 0, _stream(x_f8)), "ngpt_fc_relu2_fwd")
+    ws = _workspace(lib.ngpt_fc_relu2_fwd_workspace_bytes(M, N, K), x_f8.device)
+    _lib.check(lib.ngpt_fc_relu2_fwd_ws(_p(x_f8), _p(w_f8), _p(dequant_scale), M, N, K, _p(post), None, None,
+                                        None, 0, _p(ws), ws.numel(), _stream(x_f8)), "ngpt_fc_relu2_fwd")
     return post
 
 
@@ -401,9 +403,10 @@ def fc_relu2_fwd_emit(x_f8: Tensor, w_f8: Tensor, dequant_scale: Tensor, activat
     N = w_f8.shape[0]
     post = torch.empty((M, N), dtype=torch.bfloat16, device=x_f8.device)
     post_f8 = torch.empty((M, N), dtype=E4M3, device=x_f8.device)
-    _lib.check(lib.ngpt_fc_relu2_fwd(_p(x_f8), _p(w_f8), _p(dequant_scale), M, N, K, _p(post), _p(post_f8),
-                                     _p(activation_scale), _p(partial_amax), partial_amax.numel(),
-                                     _stream(x_f8)), "ngpt_fc_relu2_fwd")
+    ws = _workspace(lib.ngpt_fc_relu2_fwd_workspace_bytes(M, N, K), x_f8.device)
+    _lib.check(lib.ngpt_fc_relu2_fwd_ws(_p(x_f8), _p(w_f8), _p(dequant_scale), M, N, K, _p(post), _p(post_f8),
+                                        _p(activation_scale), _p(partial_amax), partial_amax.numel(),
+                                        _p(ws), ws.numel(), _stream(x_f8)), "ngpt_fc_relu2_fwd")
     return post, post_f8
 
 

@@ -262,6 +262,56 @@ def test_fc_relu2_emit_fp8_and_amax(amd, oracle):
     assert_close_gemm(post_f8.float().cpu() * act, pf8_ref.float() * act)
 
 
+@pytest.mark.parametrize("M,K,N", [(8192, 256, 512), (8320, 768, 3072), (8192 + 48, 1024, 1024)])
+def test_fc_relu2_and_mm_forward_kernels_agree(amd, M, K, N):
+    """c_fc (with and without the e4m3 copy) and the mm forward on the tile kernel (no workspace) and on the
+    token-stationary kernel (workspace with room for the re-ordered weights): every output byte equal.  Both kernels
+    contract in ascending order with the same MFMA, so the accumulators agree bit for bit; M, K, N include a ragged
+    last token tile and every supported contraction length."""
+    lib = amd._lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).bfloat16().cuda()
+    w = (torch.randn(N, K, generator=g) / K ** 0.5).bfloat16().cuda()
+    x_f8, w_f8 = (x / 0.05).to(E4M3), (w / 0.002).to(E4M3)
+    dequant = torch.tensor([0.05 * 0.002], device="cuda")
+    act = torch.tensor([0.01], device="cuda")
+    nws = lib.ngpt_fc_relu2_fwd_workspace_bytes(M, N, K)
+    assert nws >= N * K           # these shapes are covered by the token-stationary kernel
+    ws = torch.empty(nws, dtype=torch.uint8, device="cuda")
+    ptr = lambda t: t.data_ptr()
+    res = {}
+    for which in ("tile", "stationary"):
+        post = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        post_e = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        post_f8 = torch.zeros((M, N), dtype=torch.uint8, device="cuda")
+        partial = torch.full((512,), -1.0, device="cuda")
+        wsp, wsn = (None, 0) if which == "tile" else (ptr(ws), nws)
+        print(f"c_fc {which} M={M} K={K} N={N}", flush=True)
+        rc = lib.ngpt_fc_relu2_fwd_ws(ptr(x_f8), ptr(w_f8), ptr(dequant), M, N, K, ptr(post), None, None, None, 0, wsp, wsn, stream)
+        assert rc == 0, lib.ngpt_last_error()
+        rc = lib.ngpt_fc_relu2_fwd_ws(ptr(x_f8), ptr(w_f8), ptr(dequant), M, N, K, ptr(post_e), ptr(post_f8), ptr(act), ptr(partial), 512,
+                                      wsp, wsn, stream)
+        assert rc == 0, lib.ngpt_last_error()
+        # mm forward from the bf16 operands
+        out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        xq, wq = torch.zeros((M, K), dtype=torch.uint8, device="cuda"), torch.zeros((N, K), dtype=torch.uint8, device="cuda")
+        nmm = lib.ngpt_mm_fwd_workspace_bytes(M, N, K, 0)
+        wmm = torch.empty(max(nmm, 1), dtype=torch.uint8, device="cuda")
+        print(f"mm forward {which}", flush=True)
+        rc = lib.ngpt_mm_fwd(ptr(x), ptr(w), M, N, K, 0.05, 0.002, ptr(out), ptr(xq), ptr(wq), 0,
+                             *((None, 0) if which == "tile" else (ptr(wmm), nmm)), stream)
+        assert rc == 0, lib.ngpt_last_error()
+        torch.cuda.synchronize()
+        res[which] = dict(post=post, post_e=post_e, post_f8=post_f8, amax=partial.max().item(), out=out, xq=xq, wq=wq)
+        assert (partial >= 0).all()
+    a, b = res["tile"], res["stationary"]
+    for name in ("post", "post_e", "post_f8", "out", "xq", "wq"):
+        assert torch.isfinite(b[name].float()).all() and torch.equal(a[name], b[name]), name
+    assert torch.equal(a["post"], a["post_e"]) and a["amax"] == b["amax"] == a["post"].float().max().item()
+    assert int((a["post"] > 0).sum()) > 0.3 * M * N and int((a["post_f8"] != 0).sum()) > 0.2 * M * N
+
+
 def test_mlp_backward(amd, oracle):
     M, D, H = 512, 256, 768
     x, w_fc, w_proj_t = oracle.make_cfg2(seed=9, M=M, D=D, H=H)
