@@ -1096,7 +1096,9 @@ static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwdT<CODES>& epi, hip
     static PerDeviceOnce configured;
     if (int e = configured.run([&] { return allow_lds(kernel, LDS); })) return e;
     int cus = num_cus();
-    if (cus < CE_XCDS * CE_SPLITS) return fail(NGPT_EINVAL, "no HIP device (or fewer than %d compute units)", CE_XCDS * CE_SPLITS);
+    if (cus <= 0) return fail(NGPT_EINVAL, "lm_head CE forward: no HIP device");
+    if (cus < CE_XCDS * CE_SPLITS)
+        return fail(NGPT_EINVAL, "lm_head CE forward: the job walk needs at least %d compute units, the device has %d", CE_XCDS * CE_SPLITS, cus);
     int tiles_m = (g.C + Cfg::BN - 1) / Cfg::BN;
     int per_xcd = (tiles_m + CE_XCDS - 1) / CE_XCDS;
     int mg = cus * Cfg::WGS_PER_CU / (CE_XCDS * CE_SPLITS);      // token tiles in flight per XCD
@@ -1121,7 +1123,8 @@ static int launch_ce_fwd_xs(XsArgs a, hipStream_t st, int slot = -1) {
     static PerDeviceOnce configured;
     if (int e = configured.run([&] { return allow_lds(kernel, HEAD + NS * 64 * XS_TOK); })) return e;
     const int cus = num_cus();
-    if (cus < CE_XCDS) return fail(NGPT_EINVAL, "lm_head CE forward: no HIP device (or fewer than %d compute units)", CE_XCDS);
+    if (cus <= 0) return fail(NGPT_EINVAL, "token-stationary kernel: no HIP device");
+    if (cus < CE_XCDS) return fail(NGPT_EINVAL, "token-stationary kernel: the job walk needs at least %d compute units, the device has %d", CE_XCDS, cus);
     // workgroups per XCD = token tiles in flight (mg) x vocabulary shares (splits); the split count that needs the
     // fewest unit-steps per workgroup wins, the smaller one on a tie (longer jobs, fewer slab loads)
     if (a.tiles_m <= 0) a.tiles_m = (a.M + XS_TOK - 1) / XS_TOK;
