@@ -60,9 +60,10 @@ def mm_op(x: Tensor, w: Tensor, x_s: float, w_s: float, grad_s: float) -> tuple[
     out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     x_f8 = torch.empty((M, K), dtype=E4M3, device=x.device)
     w_f8 = torch.empty((N, K), dtype=E4M3, device=x.device)
-    ws = _workspace(lib.ngpt_mm_fwd_workspace_bytes(M, N, K, _lib.W_OUT_IN), x.device)
+    nws = lib.ngpt_mm_fwd_workspace_bytes(M, N, K, _lib.W_OUT_IN)      # 0 for shapes that stay on the tile kernel
+    ws = _workspace(nws, x.device) if nws else None
     _lib.check(lib.ngpt_mm_fwd(_p(x), _p(w), M, N, K, x_s, w_s, _p(out), _p(x_f8), _p(w_f8),
-                               _lib.W_OUT_IN, _p(ws), ws.numel(), _stream(x)), "ngpt_mm_fwd")
+                               _lib.W_OUT_IN, _p(ws) if nws else None, nws, _stream(x)), "ngpt_mm_fwd")
     return out, x_f8, w_f8
 
 
