@@ -1118,7 +1118,7 @@ template <int MODE, int NS>
 static int launch_ce_fwd_xs(XsArgs a, hipStream_t st, int slot = -1) {
     auto kernel = ce_fwd_xs_kernel<MODE, NS>;
     // dynamic LDS: candidate targets / row factors + slab (the table is static LDS), or slab + the waves' line staging
-    constexpr int HEAD = MODE >= XS_LINES ? XS_WAVES * XS_LINE_STAGE : XS_CAND_LDS;
+    constexpr int HEAD = MODE >= XS_LINES ? XS_WAVES * XS_LINE_STAGE : XS_CAND_LDS + (MODE == XS_DL && NS <= 12 ? XS_WAVES * XS_LINE_STAGE : 0);
     const int LDS = HEAD + a.K * XS_TOK;
     static PerDeviceOnce configured;
     if (int e = configured.run([&] { return allow_lds(kernel, HEAD + NS * 64 * XS_TOK); })) return e;

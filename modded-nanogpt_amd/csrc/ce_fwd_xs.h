@@ -75,6 +75,8 @@ struct XsArgs {
 template <int MODE, int NS /* K / 64 */>
 __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
     constexpr bool CODES = MODE == XS_FWD_CODES, DL = MODE == XS_DL, LINES = MODE >= XS_LINES, EMIT = MODE == XS_RELU2_EMIT;
+    // XS_DL: the gradient bytes pass through the waves' line staging where LDS has room for it beside slab and table
+    constexpr bool DL_STAGED = DL && NS <= 12;
     // weight fragment sets in registers (loads run XS_RING - 1 steps ahead); must divide the number of steps
     constexpr int XS_RING = 4;
     static_assert(NS % XS_RING == 0, "ring slots of a unit's first steps");
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int M = p.M, K = p.K;
-    // XS_LINES..: the wave's staging block behind the slab; scale and running maximum of the ReLU^2 modes
+    // XS_LINES.., XS_DL (staged): the wave's staging block behind the slab; scale and running maximum of the ReLU^2 modes
     uint8_t* const line_stage = xslab + K * XS_TOK + wave * XS_LINE_STAGE;
     float line_scale = p.scale, inv_act = 0.0f;
     uint32_t amax2 = 0u;
@@ -244,7 +246,57 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
                 const uint32_t rf_addr = (uint32_t)(size_t)((const __attribute__((address_space(3))) uint8_t*)cand) + 16 * h;
                 auto run = [&](auto sat) {
                     constexpr bool SAT = decltype(sat)::value;
-                    constexpr int NB = 16;      // batch b: token block b / 4, register group b % 4, both vocabulary blocks
+                    constexpr int NB = 16;
+                    if constexpr (DL_STAGED) {
+                        // batch b: vocabulary block b / 8, token block b / 2 % 4, registers 8 (b % 2) ..+7 (two groups of four
+                        // tokens).  The block's 32 rows x 128 bytes are collected in the wave's LDS block (16-byte pieces
+                        // swizzled by the row) and leave as whole 128-byte rows: a 64-lane store then touches 8 lines
+                        // instead of 64, which is what the address unit charges for.
+                        uint8_t* const stage = line_stage;
+                        const int rd_row = el >> 3, rd_chunk = el & 7;
+                        float pv[8], nv[8];
+                        v4f prf[2], nrf[2];
+#pragma unroll
+                        for (int b = 0; b <= NB; ++b) {
+                            if (b < NB) {
+                                const int tm = b >> 3, tn = (b >> 1) & 3, gp = b & 1;
+                                const v16f& r = acc[tm][tn];
+                                uint32_t off[4];
+#pragma unroll
+                                for (int k = 0; k < 4; ++k) off[k] = tab_offsets2(pack_logits(r[8 * gp + 2 * k] * p.scale, r[8 * gp + 2 * k + 1] * p.scale));
+                                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                                for (int q = 0; q < 2; ++q)
+                                    nrf[q] = *(const __attribute__((address_space(3))) v4f*)(uintptr_t)(rf_addr + (32 * tn + 8 * (2 * gp + q)) * 4);
+#pragma unroll
+                                for (int k = 0; k < 4; ++k) {
+                                    nv[2 * k] = tab_at(tab, off[k] & 0xffffu);
+                                    nv[2 * k + 1] = tab_at(tab, off[k] >> 16);
+                                }
+                                __builtin_amdgcn_sched_barrier(0);
+                            }
+                            if (b > 0) {
+                                const int q = b - 1, tm = q >> 3, tn = (q >> 1) & 3, gp = q & 1;
+                                const uint32_t w0 = f32x4_to_e5m2_sat<SAT>(prf[0][0] * pv[0], prf[0][1] * pv[1], prf[0][2] * pv[2], prf[0][3] * pv[3]);
+                                const uint32_t w1 = f32x4_to_e5m2_sat<SAT>(prf[1][0] * pv[4], prf[1][1] * pv[5], prf[1][2] * pv[6], prf[1][3] * pv[7]);
+                                *(v2i*)(stage + j * 128 + (((2 * tn + h) ^ (j & 7)) << 4) + 8 * gp) = (v2i){(int)w0, (int)w1};
+                                if ((q & 7) == 7) {     // the vocabulary block is complete
+#pragma unroll
+                                    for (int k = 0; k < 4; ++k) {
+                                        const int row = 8 * k + rd_row;
+                                        const v4i v = *(const v4i*)(stage + row * 128 + ((rd_chunk ^ (row & 7)) << 4));
+                                        *(v4i*)(dl_base + ((tm * 32 + row) * 128 + rd_chunk * 16)) = v;
+                                    }
+                                }
+                            }
+#pragma unroll
+                            for (int k = 0; k < 8; ++k) pv[k] = nv[k];
+                            prf[0] = nrf[0];
+                            prf[1] = nrf[1];
+                        }
+                        return;
+                    }
+                    // batch b: token block b / 4, register group b % 4, both vocabulary blocks; 16-byte stores from the registers
                     uint32_t pk[2][4];
                     float pv[8], nv[8];
                     v4f prf, nrf;
