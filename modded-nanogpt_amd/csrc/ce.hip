@@ -942,29 +942,31 @@ __global__ __launch_bounds__(256) void ce_codes_to_dl_kernel(const uint8_t* __re
     constexpr int kStride = 33;
     __shared__ uint32_t tile[128 * kStride];
     __shared__ float dtab[256];
-    if (probe_total(probe_hits) > probe_limit) return;      // the whole panel is recomputed instead (see ce_bwd_prep_kernel)
     const int kv = blockIdx.x, a = blockIdx.y, tid = threadIdx.x;
-    dtab[tid] = dcode[tid];
-    const float d_below = dcode[256];
-    __syncthreads();
-    auto word_at = [&](int r, int w) -> uint32_t& { return tile[r * kStride + (w ^ (((r >> 4) & 7) << 2))]; };
     const int tok0 = m0 + a * 128;
     const uint8_t* src = codes + ((int64_t)(tok0 >> 8) * nkp + kv) * kPanelBytes + (tok0 & 128) * 16;
+    // The workgroup's codes and row factors are requested before anything else: the probe counts, the code table and
+    // its barrier would otherwise put a round trip to memory in front of them (a workgroup lives only a few of those).
+    v4i c[4];
+    float rf[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int i = tid + 256 * j, r = i & 127, ch = i >> 7;   // 16 codes (group ch) of token tok0 + r
+        c[j] = *(const v4i*)(src + ch * kCodeGroupBytes + r * 16);
+        rf[j] = rowf[tok0 + r];                                   // zero past the last token
+    }
+    const float dcode_mine = dcode[tid], d_below = dcode[256];
+    if (probe_total(probe_hits) > probe_limit) return;      // the whole panel is recomputed instead (see ce_bwd_prep_kernel)
+    dtab[tid] = dcode_mine;
+    __syncthreads();
+    auto word_at = [&](int r, int w) -> uint32_t& { return tile[r * kStride + (w ^ (((r >> 4) & 7) << 2))]; };
     bool below = false;
     // the two 128-token halves of a 256-token block ask the same flag: no product of the block leaves the e5m2 range
     // unless it is set (see ce_rowf_block), and the conversion then needs no clamps
     const int may_saturate = ((const __attribute__((address_space(4))) int*)(uintptr_t)big)[tok0 >> 8];
     auto convert = [&](auto sat) {
         constexpr bool SAT = decltype(sat)::value;
-        // all global loads first, then per 16 codes: sixteen table reads in flight, then products, conversions, LDS writes
-        v4i c[4];
-        float rf[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int i = tid + 256 * j, r = i & 127, ch = i >> 7;   // 16 codes (group ch) of token tok0 + r
-            c[j] = *(const v4i*)(src + ch * kCodeGroupBytes + r * 16);
-            rf[j] = rowf[tok0 + r];                                   // zero past the last token
-        }
+        // per 16 codes: sixteen table reads in flight, then products, conversions, LDS writes
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int i = tid + 256 * j, r = i & 127, ch = i >> 7;
