@@ -440,8 +440,10 @@ __global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
                         cw[2 * (b & 1)] = pack_codes4(cur[0], cur[1], cur[2], cur[3]);
                         cw[2 * (b & 1) + 1] = pack_codes4(cur[4], cur[5], cur[6], cur[7]);
                         if (b & 1)      // (tn, tm) = (b / 4, b / 2 % 2)
-                            *(v4i*)(cd_base + (cd_lane + (b >> 2) * 512 + ((b >> 1) & 1) * 2 * kCodeGroupBytes)) =
-                                (v4i){(int)cw[0], (int)cw[1], (int)cw[2], (int)cw[3]};
+                            // non-temporal: the codes are next read by the conversion pass, long after they have left every
+                            // cache, and should not push the weights out of L2 on their way (measured: 0.05 ms of the step)
+                            __builtin_nontemporal_store((v4i){(int)cw[0], (int)cw[1], (int)cw[2], (int)cw[3]},
+                                                        (v4i*)(cd_base + (cd_lane + (b >> 2) * 512 + ((b >> 1) & 1) * 2 * kCodeGroupBytes)));
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     if (b + 1 < NB) gather(off, cur);
