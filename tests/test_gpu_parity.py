@@ -543,6 +543,8 @@ def _codes_case(oracle, M, K, V, seed, n_predict, prefix, below_window):
     (256, 128, 512, 1, False, False, 0, 1.0),        # one tile
     (640, 256, 2432, 1, False, False, 0, 1.0),       # ragged token and vocabulary tiles (rows / columns of clamped duplicates)
     (384, 768, 5120, 3, True, True, 0, 1.0),         # multi-token prediction + prefix targets, (in, out) weight
+    (512, 512, 1024, 2, False, False, 0, 1.0),       # the other two contraction lengths of the token-stationary kernels
+    (640, 1024, 1536, 1, True, False, 0, 1.0),       # (K = 1024: gradient bytes stored from the registers, no LDS staging)
     (1024, 256, 2048, 1, False, False, 300, 1.0),    # sigmas below the code window in two of four token tiles, first vocabulary tile: those two tiles are recomputed
     (1024, 256, 2048, 2, True, True, 1024, 1.0),     # ... in every token tile
     (1024, 256, 2048, 1, False, False, 300, 0.01),   # ... with row factors so small that those gradients are exact zeros: nothing is recomputed
