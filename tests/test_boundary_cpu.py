@@ -90,6 +90,11 @@ def test_argument_errors_do_not_need_a_gpu(amd):
     assert lib.ngpt_gemm_bf16(1, 0, 64, 1, 0, 64, 12, 768, 64, 1, 768, 1, 1 << 30, None) == -2
     assert lib.ngpt_linear_relu2_bf16(1, 1, 64, 100, 64, 1, None) == -2
     assert lib.ngpt_gemm_fp8_scaled(1, 0, 128, 1, 0, 128, 64, 64, 128, None, None, 1, 64, 1, 1 << 20, None) == -1      # scales are required
+    # c_fc with a workspace: same argument checks as without one, whichever kernel the workspace would select
+    assert lib.ngpt_fc_relu2_fwd_ws(1, 1, None, 8192, 3072, 768, 1, None, None, None, 0, None, 0, None) == -1
+    assert lib.ngpt_fc_relu2_fwd_ws(1, 1, 1, 8192, 3072, 768, 1, 1, None, None, 0, None, 0, None) == -1               # e4m3 copy without its scale
+    assert lib.ngpt_fc_relu2_fwd_ws(1, 1, 1, 8192, 3000, 768, 1, None, None, None, 0, None, 0, None) == -2 and b"N=3000" in lib.ngpt_last_error()
+    assert lib.ngpt_fc_relu2_fwd_workspace_bytes(8192, 3000, 768) == 0 and lib.ngpt_fc_relu2_fwd_workspace_bytes(8192, 3072, 100) == 0
     with pytest.raises(amd._lib.NgptError):
         amd._lib.check(-2, "probe")
 
