@@ -668,7 +668,7 @@ __global__ void ce_finalize_kernel(const float* __restrict__ part, const float* 
 }
 
 }  // namespace ngpt
-#include "ce_fwd_xs.h"
+#include "token_stationary.h"
 namespace ngpt {
 
 // =====================================================================================================
@@ -1113,12 +1113,12 @@ static int launch_ce_fwd(const GemmOperands& g, const EpiCEFwdT<CODES>& epi, hip
     return check_launch("lm_head CE forward");
 }
 
-// The token-stationary forward (ce_fwd_xs.h) covers V % 64 == 0, K % 256 == 0, K <= XS_MAX_K; other shapes take the tile kernel.
+// The token-stationary forward (token_stationary.h) covers V % 64 == 0, K % 256 == 0, K <= XS_MAX_K; other shapes take the tile kernel.
 static bool xs_eligible(int M, int K, int V) { return M > 0 && V % XS_UNIT == 0 && (K == 256 || K == 512 || K == 768 || K == 1024); }
 
 template <int MODE, int NS>
-static int launch_ce_fwd_xs(XsArgs a, hipStream_t st, int slot = -1) {
-    auto kernel = ce_fwd_xs_kernel<MODE, NS>;
+static int launch_token_stationary(XsArgs a, hipStream_t st, int slot = -1) {
+    auto kernel = token_stationary_kernel<MODE, NS>;
     // dynamic LDS: candidate targets / row factors + slab (the table is static LDS), or slab + the waves' line staging
     constexpr int HEAD = MODE >= XS_LINES ? XS_WAVES * XS_LINE_STAGE : XS_CAND_LDS + (MODE == XS_DL && NS <= 12 ? XS_WAVES * XS_LINE_STAGE : 0);
     const int LDS = HEAD + a.K * XS_TOK;
@@ -1323,9 +1323,9 @@ int xs_gemm_lines(int mode, const void* x_f8, const void* w_frag, int M, int N, 
     auto go = [&](auto ns) -> int {
         constexpr int NS = decltype(ns)::value;
         switch (mode) {
-            case XS_LINES: return launch_ce_fwd_xs<XS_LINES, NS>(a, st, slot);
-            case XS_RELU2: return launch_ce_fwd_xs<XS_RELU2, NS>(a, st, slot);
-            case XS_RELU2_EMIT: return launch_ce_fwd_xs<XS_RELU2_EMIT, NS>(a, st, slot);
+            case XS_LINES: return launch_token_stationary<XS_LINES, NS>(a, st, slot);
+            case XS_RELU2: return launch_token_stationary<XS_RELU2, NS>(a, st, slot);
+            case XS_RELU2_EMIT: return launch_token_stationary<XS_RELU2_EMIT, NS>(a, st, slot);
         }
         return fail(NGPT_EINVAL, "xs_gemm_lines: mode %d", mode);
     };
@@ -1416,10 +1416,10 @@ static int lmhead_ce_fwd_impl(const char* who, const void* x_bf16, const void* w
         a.ncand = prefix_targets ? n_predict + 1 : n_predict;
         int e = NGPT_EINVAL;
         switch (K / 64) {   // the contraction loop is unrolled completely: one instantiation per supported K
-            case 4: e = sigma_codes ? launch_ce_fwd_xs<XS_FWD_CODES, 4>(a, st) : launch_ce_fwd_xs<XS_FWD, 4>(a, st); break;
-            case 8: e = sigma_codes ? launch_ce_fwd_xs<XS_FWD_CODES, 8>(a, st) : launch_ce_fwd_xs<XS_FWD, 8>(a, st); break;
-            case 12: e = sigma_codes ? launch_ce_fwd_xs<XS_FWD_CODES, 12>(a, st) : launch_ce_fwd_xs<XS_FWD, 12>(a, st); break;
-            case 16: e = sigma_codes ? launch_ce_fwd_xs<XS_FWD_CODES, 16>(a, st) : launch_ce_fwd_xs<XS_FWD, 16>(a, st); break;
+            case 4: e = sigma_codes ? launch_token_stationary<XS_FWD_CODES, 4>(a, st) : launch_token_stationary<XS_FWD, 4>(a, st); break;
+            case 8: e = sigma_codes ? launch_token_stationary<XS_FWD_CODES, 8>(a, st) : launch_token_stationary<XS_FWD, 8>(a, st); break;
+            case 12: e = sigma_codes ? launch_token_stationary<XS_FWD_CODES, 12>(a, st) : launch_token_stationary<XS_FWD, 12>(a, st); break;
+            case 16: e = sigma_codes ? launch_token_stationary<XS_FWD_CODES, 16>(a, st) : launch_token_stationary<XS_FWD, 16>(a, st); break;
         }
         if (e) return e;
     } else if (sigma_codes) {
@@ -1635,10 +1635,10 @@ static int lmhead_ce_bwd_impl(const char* who, const void* x_f8, const void* w_f
             a.nkt = nkt;
             int e = NGPT_EINVAL;
             switch (K / 64) {
-                case 4: e = launch_ce_fwd_xs<XS_DL, 4>(a, st); break;
-                case 8: e = launch_ce_fwd_xs<XS_DL, 8>(a, st); break;
-                case 12: e = launch_ce_fwd_xs<XS_DL, 12>(a, st); break;
-                case 16: e = launch_ce_fwd_xs<XS_DL, 16>(a, st); break;
+                case 4: e = launch_token_stationary<XS_DL, 4>(a, st); break;
+                case 8: e = launch_token_stationary<XS_DL, 8>(a, st); break;
+                case 12: e = launch_token_stationary<XS_DL, 12>(a, st); break;
+                case 16: e = launch_token_stationary<XS_DL, 16>(a, st); break;
             }
             if (e) return e;
         } else if (int e = launch_grid_kernel<MainCfg, GridIter>(g, epi, st, PROF_CE_DLOGITS, "lm_head CE backward (dlogits)")) return e;

@@ -27,7 +27,7 @@ inline int check_launch(const char* what) {
 int quant_e4m3_pair(const void* in0, void* out0, int64_t n0, float s0, const void* in1, void* out1, int64_t n1, float s1,
                     hipStream_t st);
 
-// fp8 GEMM with a row-major bf16 output on the token-stationary kernel (ce.hip, ce_fwd_xs.h): out [M, N] = x [M, K] . w [N, K]^T,
+// fp8 GEMM with a row-major bf16 output on the token-stationary kernel (ce.hip, token_stationary.h): out [M, N] = x [M, K] . w [N, K]^T,
 // w given in fragment order (xs_gemm_frag_bytes bytes, written by xs_gemm_make_frag from the row-major e4m3 matrix or by
 // xs_gemm_quant_pair_frag together with the e4m3 copies of both bf16 operands).  mode: 3 = bf16(acc * scale), 4 = the
 // ReLU^2 epilogue of c_fc, 5 = the same with the e4m3 copy and per-workgroup maxima; the scale is `scale` times

@@ -73,7 +73,7 @@ struct XsArgs {
 };
 
 template <int MODE, int NS /* K / 64 */>
-__global__ __launch_bounds__(XS_THREADS, 1) void ce_fwd_xs_kernel(XsArgs p) {
+__global__ __launch_bounds__(XS_THREADS, 1) void token_stationary_kernel(XsArgs p) {
     constexpr bool CODES = MODE == XS_FWD_CODES, DL = MODE == XS_DL, LINES = MODE >= XS_LINES, EMIT = MODE == XS_RELU2_EMIT;
     // XS_DL: the gradient bytes pass through the waves' line staging where LDS has room for it beside slab and table
     constexpr bool DL_STAGED = DL && NS <= 12;
